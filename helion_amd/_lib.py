@@ -1,0 +1,77 @@
+"""ctypes binding of libhx_kernels.so (the C ABI declared in include/hx_kernels.h).
+
+There is no fallback: if the shared object is missing, every entry point raises.  Build it with
+``python -m helion_amd.build`` (hipcc, gfx950)."""
+from __future__ import annotations
+
+import ctypes
+import pathlib
+
+HX_F16, HX_BF16, HX_F32, HX_E4M3 = 0, 1, 2, 3
+
+_LIB_PATH = pathlib.Path(__file__).resolve().parent / "libhx_kernels.so"
+_lib = None
+
+_c = ctypes
+_SIGNATURES = {
+    "hx_version": (_c.c_int, []),
+    "hx_last_error": (_c.c_char_p, []),
+    "hx_fp8_gemm": (
+        _c.c_int,
+        [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64,
+         _c.c_int64, _c.c_int64, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_size_t, _c.c_void_p],
+    ),
+    "hx_fp8_gemm_workspace_bytes": (_c.c_size_t, [_c.c_int64, _c.c_int64, _c.c_int64]),
+    "hx_fp8_gemm_path": (
+        _c.c_int,
+        [_c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_void_p,
+         _c.c_void_p, _c.c_void_p],
+    ),
+    "hx_fp8_attention": (
+        _c.c_int,
+        [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int,
+         _c.c_int, _c.c_void_p],
+    ),
+    "hx_moe_grouped_gemm": (
+        _c.c_int,
+        [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int64,
+         _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int, _c.c_void_p, _c.c_size_t, _c.c_void_p],
+    ),
+    "hx_moe_workspace_bytes": (_c.c_size_t, [_c.c_int64, _c.c_int64]),
+}
+
+
+def lib_path() -> pathlib.Path:
+    return _LIB_PATH
+
+
+def exported_symbols() -> list[str]:
+    return list(_SIGNATURES)
+
+
+def load():
+    """Load (once) and return the ctypes handle; raises if the library has not been built."""
+    global _lib
+    if _lib is None:
+        if not _LIB_PATH.exists():
+            raise RuntimeError(
+                f"{_LIB_PATH} is missing: the HIP kernels are not built. Run `python -m helion_amd.build` "
+                "(needs hipcc; cross-compiles for gfx950 without a GPU). There is no CPU or PyTorch fallback."
+            )
+        lib = ctypes.CDLL(str(_LIB_PATH))
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def check(rc: int, what: str) -> None:
+    """Turn a non-zero C-ABI return into a Python exception (ValueError for argument errors)."""
+    if rc == 0:
+        return
+    msg = load().hx_last_error().decode("utf-8", "replace")
+    if rc < 0:
+        raise ValueError(f"{what}: {msg} (code {rc})")
+    raise RuntimeError(f"{what}: {msg} (hipError {rc})")

@@ -1,0 +1,395 @@
+// FP8 (OCP e4m3fn) GEMM for gfx950: C[M,N] = cast((A[M,K] @ B[K,N]) * scale_a*scale_b), fp32 accumulate.
+// Drop-in device side of examples/fp8_gemm.py:29-57 of the reference.
+//
+// Three kernels:
+//   hx_fp8_gemm_tile256 : 256x256x128 workgroup tile, 4 waves (2x2) of 128x128, 32x32x64 fp8 MFMA,
+//                         A/B k-tiles DMA'd global->LDS (double buffered, XOR-swizzled 16B chunks).
+//   hx_fp8_gemm_skinny  : M <= 16; HBM-bound streaming of B through 16x16x128 MFMA, K split across
+//                         the 8 waves of a workgroup, wave partials reduced through LDS.
+//   hx_fp8_gemm_general : bounds-checked, arbitrary strides (fallback for ragged/unaligned inputs).
+#include "hx_common.h"
+
+// ------------------------------------------------------------------------------------------
+// tile256
+// ------------------------------------------------------------------------------------------
+// LDS tile layout (A and B alike; B is addressed as B^T[N][K], K contiguous):
+//   tile[row 0..255][pos 0..7] of 16-byte chunks, row stride 128 B (one 128-byte k-tile per row);
+//   the chunk stored at (row, pos) is global chunk  pos ^ swz(row),  swz(row) = (row >> 1) & 7.
+// One DMA instruction of a wave moves 8 rows x 128 B (lane = row_in_8 * 8 + pos), so global reads
+// are whole 128-byte lines and LDS writes are 1024 contiguous bytes.
+// MFMA operand fetch: lane (r = lane%32, g = lane/32) of k-step t reads chunks 4t+2g and 4t+2g+1 of
+// row r: two ds_read_b128.  A and B use the same lane->k mapping, which is all the contraction needs.
+
+#define T256_BM 256
+#define T256_BN 256
+#define T256_BK 128
+#define T256_TILE_BYTES (256 * 128)
+
+template <int OUT>
+__global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __restrict__ A, const uint8_t* __restrict__ Bt,
+                                                          typename OutT<OUT>::T* __restrict__ C, int K, long lda, long ldb,
+                                                          long ldc, const float* __restrict__ scale_a,
+                                                          const float* __restrict__ scale_b, int tiles_m, int tiles_n) {
+  typedef typename OutT<OUT>::T out_t;
+  __shared__ __attribute__((aligned(1024))) uint8_t sA0[T256_TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) uint8_t sA1[T256_TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) uint8_t sB0[T256_TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) uint8_t sB1[T256_TILE_BYTES];
+
+  // ---- workgroup -> tile. Workgroup i runs on XCD i%8 (each XCD has its own 4 MB L2): give every
+  // XCD a contiguous range of a grouped (8 tile-rows tall) raster so concurrently resident tiles of
+  // one XCD share A row-panels and B column-panels in that L2.
+  int tile;
+  {
+    const int nwg = gridDim.x, wg = blockIdx.x;
+    const int per = nwg >> 3, rem = nwg & 7, xcd = wg & 7, loc = wg >> 3;
+    tile = (xcd < rem) ? xcd * (per + 1) + loc : rem * (per + 1) + (xcd - rem) * per + loc;
+  }
+  const int GM = 8;
+  const int group_size = GM * tiles_n;
+  const int gid = tile / group_size;
+  const int first_m = gid * GM;
+  const int gm = min(tiles_m - first_m, GM);
+  const int tm = first_m + (tile % group_size) % gm;
+  const int tn = (tile % group_size) / gm;
+  const long m0 = (long)tm * T256_BM, n0 = (long)tn * T256_BN;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = w >> 1, wn = w & 1;
+
+  // ---- DMA addressing: wave w owns tile rows [64w, 64w+64); instruction j covers rows 64w+8j .. +7
+  const int lrow = lane >> 3, lpos = lane & 7;
+  const int coff0 = (lpos ^ ((lrow >> 1) & 7)) * 16;        // j even: swz = (lrow>>1)
+  const int coff1 = (lpos ^ ((4 + (lrow >> 1)) & 7)) * 16;  // j odd : swz = 4 + (lrow>>1)
+  const uint8_t* gA = A + (m0 + w * 64 + lrow) * lda;
+  const uint8_t* gB = Bt + (n0 + w * 64 + lrow) * ldb;
+
+  auto issue = [&](int kt, uint8_t* sa, uint8_t* sb) {
+    const long kb = (long)kt * T256_BK;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int co = (j & 1) ? coff1 : coff0;
+      hx_g2l16(gA + (long)j * 8 * lda + kb + co, sa + (w * 64 + j * 8) * 128);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int co = (j & 1) ? coff1 : coff0;
+      hx_g2l16(gB + (long)j * 8 * ldb + kb + co, sb + (w * 64 + j * 8) * 128);
+    }
+  };
+
+  // ---- MFMA operand addressing
+  const int r31 = lane & 31, g = lane >> 5;
+  const int x = ((g * 2) ^ ((r31 >> 1) & 7)) * 16;
+  const int a_base = (wm * 128 + r31) * 128;
+  const int b_base = (wn * 128 + r31) * 128;
+
+  v16f acc[4][4];  // [bj][bi]: rows = n (B side), cols = m (A side)
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  auto compute = [&](const uint8_t* sa, const uint8_t* sb) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      v8i af[4], bf[4];
+      const int o0 = x ^ (t * 64), o1 = x ^ (t * 64 + 16);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v4i lo = *(const v4i*)(sa + a_base + i * 4096 + o0);
+        v4i hi = *(const v4i*)(sa + a_base + i * 4096 + o1);
+        af[i] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v4i lo = *(const v4i*)(sb + b_base + i * 4096 + o0);
+        v4i hi = *(const v4i*)(sb + b_base + i * 4096 + o1);
+        bf[i] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      }
+#pragma unroll
+      for (int bj = 0; bj < 4; ++bj)
+#pragma unroll
+        for (int bi = 0; bi < 4; ++bi) acc[bj][bi] = hx_mfma_32x32x64_e4m3(bf[bj], af[bi], acc[bj][bi]);
+    }
+  };
+
+  const int nk = K / T256_BK;
+  issue(0, sA0, sB0);
+  for (int kt = 0; kt < nk; kt += 2) {
+    HX_WAIT_VM0();
+    __syncthreads();
+    if (kt + 1 < nk) issue(kt + 1, sA1, sB1);
+    compute(sA0, sB0);
+    if (kt + 1 < nk) {
+      HX_WAIT_VM0();
+      __syncthreads();
+      if (kt + 2 < nk) issue(kt + 2, sA0, sB0);
+      compute(sA1, sB1);
+    }
+  }
+
+  // ---- epilogue: acc[bj][bi][4a+b] is C[m0 + wm*128 + bi*32 + lane%32][n0 + wn*128 + bj*32 + 8a + 4g + b]
+  float alpha = 1.f;
+  if (scale_a) alpha = *scale_a;
+  if (scale_b) alpha = alpha * *scale_b;
+#pragma unroll
+  for (int bi = 0; bi < 4; ++bi) {
+    out_t* crow = C + (m0 + wm * 128 + bi * 32 + r31) * ldc + n0 + wn * 128 + 4 * g;
+#pragma unroll
+    for (int bj = 0; bj < 4; ++bj)
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        typedef out_t ov4 __attribute__((ext_vector_type(4)));
+        ov4 o;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) o[b] = (out_t)(acc[bj][bi][4 * a + b] * alpha);
+        *(ov4*)(crow + bj * 32 + 8 * a) = o;
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// skinny (M <= 16): one workgroup = 8 waves; the workgroup owns column groups of 16 columns and
+// streams the 16 x K bytes of B^T for each exactly once from HBM.  K is split across the waves in
+// 128-byte steps (wave w takes steps w, w+8, ...); each wave accumulates a 16x16 fp32 partial with
+// 16x16x128 MFMA and the 8 partials are summed through LDS.  The A panel (16 x K bytes) sits in LDS
+// in MFMA-fragment order for the whole kernel when K <= SK_KC, else it is re-staged per K chunk.
+// ------------------------------------------------------------------------------------------
+#define SK_WAVES 8
+#define SK_KC 8192        // bytes of K per LDS-resident A chunk (16 rows -> 128 KB)
+#define SK_U 4            // k-steps (of 128 B) a wave loads per batch: 4 x 2 KB in flight per wave
+
+template <int OUT>
+__global__ __launch_bounds__(512) void hx_fp8_gemm_skinny(const uint8_t* __restrict__ A, const uint8_t* __restrict__ Bt,
+                                                         typename OutT<OUT>::T* __restrict__ C, int M, int N, int K, long lda,
+                                                         long ldb, long ldc, const float* __restrict__ scale_a,
+                                                         const float* __restrict__ scale_b) {
+  typedef typename OutT<OUT>::T out_t;
+  __shared__ __attribute__((aligned(1024))) uint8_t sA[16 * SK_KC];  // [k-step][half][lane][16 B]
+  __shared__ __attribute__((aligned(16))) float red[2][SK_WAVES][64][4];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int li = lane & 15, g = lane >> 4;
+
+  float alpha = 1.f;
+  if (scale_a) alpha = *scale_a;
+  if (scale_b) alpha = alpha * *scale_b;
+
+  const int ncg = (N + 15) >> 4;
+  const int nchunk = (K + SK_KC - 1) / SK_KC;
+  const int arow = min(li, M - 1);
+  const uint8_t* gArow = A + (long)arow * lda + g * 16;
+
+  auto stage_A = [&](int chunk) {  // all 8 waves: k-steps of this chunk, two 1 KB DMA each
+    const int k0 = chunk * SK_KC;
+    const int steps = (min(K - k0, SK_KC)) >> 7;
+    for (int s = w; s < steps; s += SK_WAVES) {
+      hx_g2l16(gArow + k0 + s * 128, sA + s * 2048);
+      hx_g2l16(gArow + k0 + s * 128 + 64, sA + s * 2048 + 1024);
+    }
+  };
+
+  if (nchunk == 1) {
+    stage_A(0);
+    HX_WAIT_VM0();
+    __syncthreads();
+  }
+
+  int parity = 0;
+  for (int cg = blockIdx.x; cg < ncg; cg += gridDim.x) {
+    const int brow = min(cg * 16 + li, N - 1);
+    const uint8_t* gBrow = Bt + (long)brow * ldb + g * 16;
+    v4f acc = {0.f, 0.f, 0.f, 0.f};
+    for (int chunk = 0; chunk < nchunk; ++chunk) {
+      const int k0 = chunk * SK_KC;
+      const int steps = (min(K - k0, SK_KC)) >> 7;
+      if (nchunk > 1) {
+        __syncthreads();  // everyone done reading the previous chunk
+        stage_A(chunk);
+        HX_WAIT_VM0();
+        __syncthreads();
+      }
+      // wave w: steps w, w+8, ... in batches of SK_U, register double-buffered
+      const int nmine = (steps - w + SK_WAVES - 1) / SK_WAVES;  // may be <= 0
+      v4i b0[SK_U][2], b1[SK_U][2];
+      auto load_batch = [&](v4i(&dst)[SK_U][2], int first) {
+#pragma unroll
+        for (int u = 0; u < SK_U; ++u) {
+          const int idx = first + u;
+          if (idx < nmine) {
+            const uint8_t* p = gBrow + k0 + (long)(w + idx * SK_WAVES) * 128;
+            dst[u][0] = __builtin_nontemporal_load((const v4i*)p);
+            dst[u][1] = __builtin_nontemporal_load((const v4i*)(p + 64));
+          }
+        }
+      };
+      auto mma_batch = [&](v4i(&src)[SK_U][2], int first) {
+#pragma unroll
+        for (int u = 0; u < SK_U; ++u) {
+          const int idx = first + u;
+          if (idx < nmine) {
+            const uint8_t* pa = sA + (w + idx * SK_WAVES) * 2048 + lane * 16;
+            v4i alo = *(const v4i*)pa;
+            v4i ahi = *(const v4i*)(pa + 1024);
+            v8i af = (v8i){alo.x, alo.y, alo.z, alo.w, ahi.x, ahi.y, ahi.z, ahi.w};
+            v8i bf = (v8i){src[u][0].x, src[u][0].y, src[u][0].z, src[u][0].w,
+                           src[u][1].x, src[u][1].y, src[u][1].z, src[u][1].w};
+            acc = hx_mfma_16x16x128_e4m3(af, bf, acc);
+          }
+        }
+      };
+      load_batch(b0, 0);
+      for (int first = 0; first < nmine; first += 2 * SK_U) {
+        load_batch(b1, first + SK_U);
+        mma_batch(b0, first);
+        load_batch(b0, first + 2 * SK_U);
+        mma_batch(b1, first + SK_U);
+      }
+    }
+    // ---- reduce the 8 wave partials: acc[r] is C[4g + r][cg*16 + li]
+    *(v4f*)&red[parity][w][lane][0] = acc;
+    __syncthreads();
+    if (tid < 256) {
+      const int l2 = tid & 63, r = tid >> 6;
+      float s = 0.f;
+#pragma unroll
+      for (int ww = 0; ww < SK_WAVES; ++ww) s += red[parity][ww][l2][r];
+      const int m = 4 * (l2 >> 4) + r, n = cg * 16 + (l2 & 15);
+      if (m < M && n < N) C[(long)m * ldc + n] = (out_t)(s * alpha);
+    }
+    parity ^= 1;
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// general: 64x64 tile, 256 threads, 4x4 outputs per thread, fp32 FMAs on decoded e4m3.
+// ------------------------------------------------------------------------------------------
+template <int OUT>
+__global__ __launch_bounds__(256) void hx_fp8_gemm_general(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
+                                                          typename OutT<OUT>::T* __restrict__ C, int M, int N, int K, long lda,
+                                                          long ldb_k, long ldb_n, long ldc, const float* __restrict__ scale_a,
+                                                          const float* __restrict__ scale_b) {
+  typedef typename OutT<OUT>::T out_t;
+  __shared__ float sa[16][64 + 1];
+  __shared__ float sb[16][64 + 1];
+  const int tid = threadIdx.x;
+  const int tx = tid & 15, ty = tid >> 4;
+  const long m0 = (long)blockIdx.y * 64, n0 = (long)blockIdx.x * 64;
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < K; k0 += 16) {
+    for (int e = tid; e < 64 * 16; e += 256) {
+      const int kk = e & 15, r = e >> 4;
+      const long m = m0 + r, k = k0 + kk;
+      sa[kk][r] = (m < M && k < K) ? hx_e4m3_to_f32(A[m * lda + k]) : 0.f;
+      const long n = n0 + r;
+      sb[kk][r] = (n < N && k < K) ? hx_e4m3_to_f32(B[k * ldb_k + n * ldb_n]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 16; ++kk) {
+      float av[4], bv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) av[i] = sa[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) bv[j] = sb[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_fmaf(av[i], bv[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+  float alpha = 1.f;
+  if (scale_a) alpha = *scale_a;
+  if (scale_b) alpha = alpha * *scale_b;
+  for (int i = 0; i < 4; ++i)
+    for (int j = 0; j < 4; ++j) {
+      const long m = m0 + ty * 4 + i, n = n0 + tx * 4 + j;
+      if (m < M && n < N) C[m * ldc + n] = (out_t)(acc[i][j] * alpha);
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// host dispatch
+// ------------------------------------------------------------------------------------------
+static inline bool aligned(const void* p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
+
+extern "C" int hx_fp8_gemm_path(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
+                                const void* a, const void* b, const void* c) {
+  const bool kmajor = (ldb_k == 1) && (lda % 16 == 0) && (ldb_n % 16 == 0) && (K % 128 == 0) && aligned(a, 16) &&
+                      aligned(b, 16) && K >= 128;
+  if (kmajor && M <= 16 && lda >= K && ldb_n >= K) return 2;
+  if (kmajor && (M % 256 == 0) && (N % 256 == 0) && (ldc % 4 == 0) && aligned(c, 16) &&
+      M * lda < (1LL << 31) && N * ldb_n < (1LL << 31))
+    return 1;
+  return 0;
+}
+
+template <int OUT>
+static int launch_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k,
+                           int64_t ldb_n, int64_t ldc, const float* sa, const float* sb, hipStream_t stream) {
+  typedef typename OutT<OUT>::T out_t;
+  const int path = hx_fp8_gemm_path(M, N, K, lda, ldb_k, ldb_n, ldc, a, b, c);
+  if (path == 1) {
+    const int tiles_m = (int)(M / 256), tiles_n = (int)(N / 256);
+    hipLaunchKernelGGL(hx_fp8_gemm_tile256<OUT>, dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
+                       (const uint8_t*)b, (out_t*)c, (int)K, (long)lda, (long)ldb_n, (long)ldc, sa, sb, tiles_m, tiles_n);
+  } else if (path == 2) {
+    int dev = 0, cus = 256;
+    (void)hipGetDevice(&dev);
+    (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    const int ncg = (int)((N + 15) / 16);
+    const int grid = ncg < cus ? ncg : cus;
+    hipLaunchKernelGGL(hx_fp8_gemm_skinny<OUT>, dim3(grid), dim3(512), 0, stream, (const uint8_t*)a, (const uint8_t*)b,
+                       (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb_n, (long)ldc, sa, sb);
+  } else {
+    dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
+    hipLaunchKernelGGL(hx_fp8_gemm_general<OUT>, grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)b, (out_t*)c,
+                       (int)M, (int)N, (int)K, (long)lda, (long)ldb_k, (long)ldb_n, (long)ldc, sa, sb);
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    hx_set_error("hx_fp8_gemm: launch failed: %s", hipGetErrorString(e));
+    return (int)e;
+  }
+  return 0;
+}
+
+extern "C" size_t hx_fp8_gemm_workspace_bytes(int64_t, int64_t, int64_t) { return 0; }
+
+extern "C" int hx_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k,
+                           int64_t ldb_n, int64_t ldc, const float* scale_a, const float* scale_b, int out_dtype,
+                           void* /*workspace*/, size_t /*workspace_bytes*/, void* stream) {
+  if (M < 0 || N < 0 || K < 0) {
+    hx_set_error("hx_fp8_gemm: negative size M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+    return HX_ERR_BAD_ARG;
+  }
+  if (M == 0 || N == 0) return 0;
+  if (!a || !b || !c) {
+    hx_set_error("hx_fp8_gemm: null operand pointer");
+    return HX_ERR_BAD_ARG;
+  }
+  if (M >= (1LL << 31) || N >= (1LL << 31) || K >= (1LL << 31)) {
+    hx_set_error("hx_fp8_gemm: dimension exceeds int32");
+    return HX_ERR_UNSUPPORTED;
+  }
+  if (lda < K || ldc < N) {
+    hx_set_error("hx_fp8_gemm: leading dimension smaller than row length (lda=%lld K=%lld ldc=%lld N=%lld)",
+                 (long long)lda, (long long)K, (long long)ldc, (long long)N);
+    return HX_ERR_BAD_ARG;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  switch (out_dtype) {
+    case HX_F16: return launch_fp8_gemm<HX_F16>(a, b, c, M, N, K, lda, ldb_k, ldb_n, ldc, scale_a, scale_b, s);
+    case HX_BF16: return launch_fp8_gemm<HX_BF16>(a, b, c, M, N, K, lda, ldb_k, ldb_n, ldc, scale_a, scale_b, s);
+    case HX_F32: return launch_fp8_gemm<HX_F32>(a, b, c, M, N, K, lda, ldb_k, ldb_n, ldc, scale_a, scale_b, s);
+    default:
+      hx_set_error("hx_fp8_gemm: unknown out_dtype tag %d", out_dtype);
+      return HX_ERR_BAD_ARG;
+  }
+}

@@ -1,0 +1,70 @@
+// Shared device helpers for the gfx950 kernels: vector types, MFMA wrappers, global->LDS DMA,
+// e4m3 conversion, output casts, error plumbing.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/hx_kernels.h"
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef short v4s __attribute__((ext_vector_type(4)));
+typedef short v8s __attribute__((ext_vector_type(8)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+
+#define HX_LDS(p) ((__attribute__((address_space(3))) void*)(p))
+#define HX_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
+
+// 16-byte global->LDS DMA: every lane supplies its own global address; the wave writes 1024
+// contiguous bytes at lds_wave_base + lane*16 (lds_wave_base must be wave-uniform).
+__device__ __forceinline__ void hx_g2l16(const void* gptr, void* lds_wave_base) {
+  __builtin_amdgcn_global_load_lds(HX_GLB(gptr), HX_LDS(lds_wave_base), 16, 0, 0);
+}
+
+// s_waitcnt encodings (gfx9): vmcnt [3:0]+[15:14], expcnt [6:4], lgkmcnt [11:8]
+#define HX_WAIT_VM0() __builtin_amdgcn_s_waitcnt(0x0F70)
+#define HX_WAIT_LGKM0() __builtin_amdgcn_s_waitcnt(0xC07F)
+__device__ __forceinline__ constexpr int hx_vmcnt_imm(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
+
+// D(32x32 f32) += A(32 rows x 64 k, e4m3) * B(64 k x 32 cols, e4m3).
+// lane l supplies 32 bytes of row/col (l%32), k = (l/32)*32 .. +31; the result lane l holds
+// column (l%32), rows 8*(r/4) + 4*(l/32) + (r%4) for r = 0..15.
+__device__ __forceinline__ v16f hx_mfma_32x32x64_e4m3(v8i a, v8i b, v16f c) {
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+// D(16x16 f32) += A(16 x 128 e4m3) * B(128 x 16 e4m3); lane l: row/col l%16, k = (l/16)*32 .. +31;
+// result lane l: column l%16, rows 4*(l/16) + r, r = 0..3.
+__device__ __forceinline__ v4f hx_mfma_16x16x128_e4m3(v8i a, v8i b, v4f c) {
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+
+template <int OUT>
+struct OutT;
+template <>
+struct OutT<HX_F16> {
+  typedef _Float16 T;
+};
+template <>
+struct OutT<HX_BF16> {
+  typedef __bf16 T;
+};
+template <>
+struct OutT<HX_F32> {
+  typedef float T;
+};
+
+// pack two fp32 -> two e4m3 bytes in the low (hi=false) or high (hi=true) half of `old`
+#define HX_CVT_PK_E4M3(a, b, old, hi) __builtin_amdgcn_cvt_pk_fp8_f32((a), (b), (old), (hi))
+
+__device__ __forceinline__ float hx_e4m3_to_f32(uint8_t code) {
+  return __builtin_amdgcn_cvt_f32_fp8((int)code, 0);
+}
+
+void hx_set_error(const char* fmt, ...);

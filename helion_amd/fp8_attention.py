@@ -1,0 +1,36 @@
+"""Drop-in for the reference's examples/fp8_attention.py."""
+from __future__ import annotations
+
+from typing import Callable
+
+import torch
+
+from .ops import fp8_attention_op
+
+
+def fp8_attention_kernel(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batch: int, heads: int, *,
+                         out_dtype: torch.dtype = torch.float8_e4m3fn, exact_max: bool = True) -> torch.Tensor:
+    """Scaled dot-product attention on e4m3 tensors (reference: examples/fp8_attention.py:22-106).
+    q, k: [batch*heads, seq, dim]; v: [batch*heads, dim, seq] (pre-transposed); returns
+    [batch, heads, seq, dim] float8_e4m3fn.  ``exact_max=True`` (default) quantises the un-normalised
+    probabilities against the exact row max, which is what the reference computes when its kernel body
+    is executed with one tile per loop; ``exact_max=False`` is the single-pass online softmax."""
+    return fp8_attention_op(q, k, v, batch, heads, out_dtype, exact_max)
+
+
+def preprocess_fp8_attention_inputs(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
+    """examples/fp8_attention.py:110-133: cast to e4m3 (v permuted to [B,H,D,S] first), flatten batch*heads."""
+    q_fp8 = q.to(torch.float8_e4m3fn)
+    k_fp8 = k.to(torch.float8_e4m3fn)
+    v = v.permute(0, 1, 3, 2)
+    v_fp8 = v.to(torch.float8_e4m3fn)
+    batch, heads, seq_len, head_dim = q.shape
+    return (q_fp8.reshape(batch * heads, seq_len, head_dim), k_fp8.reshape(batch * heads, seq_len, head_dim),
+            v_fp8.reshape(batch * heads, head_dim, seq_len))
+
+
+def fp8_attention_tritonbench(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> Callable[[], torch.Tensor]:
+    """examples/fp8_attention.py:137-154: preprocessing hoisted out of the returned thunk."""
+    batch, heads, seq_len, head_dim = q.shape
+    q_fp8, k_fp8, v_fp8 = preprocess_fp8_attention_inputs(q, k, v)
+    return lambda: fp8_attention_kernel(q_fp8, k_fp8, v_fp8, batch, heads)

@@ -1,0 +1,35 @@
+"""Drop-in for the reference's examples/fp8_gemm.py: same callables, same signatures, same layouts and
+output dtype, backed by the gfx950 HIP kernels."""
+from __future__ import annotations
+
+import torch
+
+from .ops import fp8_gemm_op
+
+
+def fp8_gemm(x: torch.Tensor, y: torch.Tensor, *, scale_a: torch.Tensor | None = None,
+             scale_b: torch.Tensor | None = None, out_dtype: torch.dtype = torch.float16) -> torch.Tensor:
+    """``out[m,n] = fp16(sum_k x[m,k] * y[k,n])`` with fp32 accumulation (reference:
+    examples/fp8_gemm.py:29-57).  x: [m,k] float8_e4m3fn, y: [k,n] float8_e4m3fn with any strides
+    (column-major y, strides (1,k), is the fast layout).  Keyword-only extensions, all defaulting to
+    the reference behaviour: per-tensor fp32 scales (one-element device tensors) and ``out_dtype``."""
+    return fp8_gemm_op(x, y, scale_a, scale_b, out_dtype)
+
+
+def fp8_gemm_scaled(x: torch.Tensor, y: torch.Tensor, scale_a: torch.Tensor, scale_b: torch.Tensor,
+                    out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """``cast((x @ y) * scale_a * scale_b)`` — the per-tensor-scaled form torch._scaled_mm computes."""
+    return fp8_gemm_op(x, y, scale_a, scale_b, out_dtype)
+
+
+def reference_fp8_gemm_pytorch(x_fp8: torch.Tensor, y_fp8: torch.Tensor) -> torch.Tensor:
+    """The reference's baseline (examples/fp8_gemm.py:61-78): torch._scaled_mm with unit scales, fp16 out."""
+    y_fp8_t = y_fp8.T.contiguous().T
+    scale_a = torch.tensor(1.0, device=x_fp8.device)
+    scale_b = torch.tensor(1.0, device=x_fp8.device)
+    return torch._scaled_mm(x_fp8, y_fp8_t, scale_a, scale_b, use_fast_accum=False, out_dtype=torch.float16)
+
+
+def fp8_gemm_tritonbench(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """examples/fp8_gemm.py:82-91."""
+    return fp8_gemm(a, b)

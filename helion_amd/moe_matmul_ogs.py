@@ -1,0 +1,44 @@
+"""Drop-in for the reference's examples/moe_matmul_ogs.py."""
+from __future__ import annotations
+
+import torch
+
+from .ops import moe_matmul_ogs_op
+
+
+def moe_matmul_ogs(A: torch.Tensor, W: torch.Tensor, expert_token_counts: torch.Tensor,
+                   expert_token_offsets: torch.Tensor, sorted_to_orig_token_idx: torch.Tensor,
+                   max_T_per_expert_tensor: torch.Tensor) -> torch.Tensor:
+    """``C[r] = A[r] @ W[e]`` for every row r routed to expert e (reference: examples/moe_matmul_ogs.py:25-80).
+    A: [T,K], W: [E,K,N]; returns [T,N] in promote_types(A.dtype, W.dtype).  As in the reference only the
+    *numel* of ``max_T_per_expert_tensor`` is used."""
+    return moe_matmul_ogs_op(A, W, expert_token_counts, expert_token_offsets, sorted_to_orig_token_idx,
+                             int(max_T_per_expert_tensor.numel()))
+
+
+def moe_matmul_ogs_helion_kernel_args_gen(A: torch.Tensor, W: torch.Tensor, top1_expert_per_token: torch.Tensor):
+    """examples/moe_matmul_ogs.py:84-121: stable sort of rows by expert, per-expert counts and offsets."""
+    E = W.size(0)
+    device = A.device
+    sorted_to_orig_token_idx = torch.argsort(top1_expert_per_token, stable=True).to(torch.int32)
+    expert_token_counts = torch.bincount(top1_expert_per_token, minlength=E).to(torch.int32)
+    expert_token_offsets = torch.empty(E + 1, dtype=torch.int32, device=device)
+    expert_token_offsets[0] = 0
+    expert_token_offsets[1:] = torch.cumsum(expert_token_counts, 0, dtype=torch.int32)
+    max_T_per_expert = int(expert_token_counts.max().item())
+    return (A, W, expert_token_counts, expert_token_offsets, sorted_to_orig_token_idx,
+            torch.empty(max_T_per_expert, device=device))
+
+
+def moe_matmul_ogs_reference(A: torch.Tensor, W: torch.Tensor, top1_expert_per_token: torch.Tensor) -> torch.Tensor:
+    """examples/moe_matmul_ogs.py:125-148 (pure torch; rows of unused experts are left as allocated)."""
+    T, K = A.shape
+    N = W.size(2)
+    device, dtype = A.device, torch.promote_types(A.dtype, W.dtype)
+    C = torch.empty(T, N, device=device, dtype=dtype)
+    for e in range(W.size(0)):
+        token_idx = (top1_expert_per_token == e).nonzero(as_tuple=True)[0]
+        if token_idx.numel() == 0:
+            continue
+        C[token_idx] = A[token_idx] @ W[e]
+    return C

@@ -1,0 +1,137 @@
+"""torch.library registrations: each op validates, allocates the output (and workspace) with torch
+and calls the C ABI on the current HIP stream.  Tensors are plumbing; the arithmetic is in
+libhx_kernels.so."""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+_DT = {torch.float16: _lib.HX_F16, torch.bfloat16: _lib.HX_BF16, torch.float32: _lib.HX_F32,
+       torch.float8_e4m3fn: _lib.HX_E4M3}
+
+
+def _stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _require_cuda(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("helion_amd ops run on the GPU only (HIP kernels); got a tensor on " + str(t.device))
+
+
+# ------------------------------------------------------------------------------ fp8 gemm
+@torch.library.custom_op("helion_amd::fp8_gemm", mutates_args=())
+def fp8_gemm_op(x: torch.Tensor, y: torch.Tensor, scale_a: torch.Tensor | None, scale_b: torch.Tensor | None,
+                out_dtype: torch.dtype) -> torch.Tensor:
+    _require_cuda(x, y, scale_a, scale_b)
+    if x.dtype != torch.float8_e4m3fn or y.dtype != torch.float8_e4m3fn:
+        raise TypeError(f"fp8_gemm expects float8_e4m3fn operands, got {x.dtype} and {y.dtype}")
+    if x.dim() != 2 or y.dim() != 2:
+        raise ValueError("fp8_gemm expects 2-D operands")
+    m, k = x.shape
+    k2, n = y.shape
+    assert k == k2, f"size mismatch {k} != {k2}"
+    if out_dtype not in (torch.float16, torch.bfloat16, torch.float32):
+        raise TypeError(f"unsupported out_dtype {out_dtype}")
+    for s in (scale_a, scale_b):
+        if s is not None and (s.dtype != torch.float32 or s.numel() != 1):
+            raise TypeError("scales must be one-element float32 tensors")
+    if x.stride(1) != 1 and k > 1:
+        x = x.contiguous()
+    lda = x.stride(0) if m > 1 else max(k, 1)
+    if lda < k:
+        x = x.contiguous()
+        lda = k
+    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    if m == 0 or n == 0:
+        return out
+    # B strides: (k stride, n stride); size-1 dims get the canonical stride
+    ldb_k = y.stride(0) if k > 1 else 1
+    ldb_n = y.stride(1) if n > 1 else max(k, 1)
+    lib = _lib.load()
+    rc = lib.hx_fp8_gemm(x.data_ptr(), y.data_ptr(), out.data_ptr(), m, n, k, lda, ldb_k, ldb_n, n,
+                         scale_a.data_ptr() if scale_a is not None else None,
+                         scale_b.data_ptr() if scale_b is not None else None,
+                         _DT[out_dtype], None, 0, _stream_ptr(x.device))
+    _lib.check(rc, "hx_fp8_gemm")
+    return out
+
+
+@fp8_gemm_op.register_fake
+def _(x, y, scale_a, scale_b, out_dtype):
+    return x.new_empty((x.shape[0], y.shape[1]), dtype=out_dtype)
+
+
+# ------------------------------------------------------------------------------ fp8 attention
+@torch.library.custom_op("helion_amd::fp8_attention", mutates_args=())
+def fp8_attention_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batch: int, heads: int,
+                     out_dtype: torch.dtype, exact_max: bool) -> torch.Tensor:
+    _require_cuda(q, k, v)
+    for t in (q, k, v):
+        if t.dtype != torch.float8_e4m3fn:
+            raise TypeError(f"fp8_attention expects float8_e4m3fn tensors, got {t.dtype}")
+        if t.dim() != 3:
+            raise ValueError("fp8_attention expects [batch*heads, seq, dim] / [batch*heads, dim, seq] tensors")
+    bh, s, d = q.shape
+    if bh != batch * heads:
+        raise ValueError(f"q.size(0)={bh} != batch*heads={batch * heads}")
+    if tuple(k.shape) != (bh, s, d) or tuple(v.shape) != (bh, d, s):
+        raise ValueError(f"shape mismatch: q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)} (v must be [BH, D, S])")
+    if out_dtype not in (torch.float8_e4m3fn, torch.float32):
+        raise TypeError(f"unsupported out_dtype {out_dtype}")
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    out = torch.empty((batch, heads, s, d), dtype=out_dtype, device=q.device)
+    if bh == 0 or s == 0:
+        return out
+    lib = _lib.load()
+    rc = lib.hx_fp8_attention(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), bh, s, d, _DT[out_dtype],
+                              1 if exact_max else 0, _stream_ptr(q.device))
+    _lib.check(rc, "hx_fp8_attention")
+    return out
+
+
+@fp8_attention_op.register_fake
+def _(q, k, v, batch, heads, out_dtype, exact_max):
+    return q.new_empty((batch, heads, q.shape[1], q.shape[2]), dtype=out_dtype)
+
+
+# ------------------------------------------------------------------------------ moe grouped gemm
+@torch.library.custom_op("helion_amd::moe_matmul_ogs", mutates_args=())
+def moe_matmul_ogs_op(A: torch.Tensor, W: torch.Tensor, expert_token_counts: torch.Tensor,
+                      expert_token_offsets: torch.Tensor, sorted_to_orig_token_idx: torch.Tensor,
+                      max_T_per_expert: int) -> torch.Tensor:
+    _require_cuda(A, W, expert_token_counts, expert_token_offsets, sorted_to_orig_token_idx)
+    if A.dim() != 2 or W.dim() != 3:
+        raise ValueError("moe_matmul_ogs expects A [T,K] and W [E,K,N]")
+    T, K = A.shape
+    E, K2, N = W.shape
+    if K != K2:
+        raise ValueError(f"size mismatch K={K} vs W.size(1)={K2}")
+    dtype = torch.promote_types(A.dtype, W.dtype)
+    if dtype not in (torch.bfloat16, torch.float16):
+        raise TypeError(f"moe_matmul_ogs supports float16/bfloat16, got {A.dtype} x {W.dtype}")
+    A = A.to(dtype).contiguous()
+    W = W.to(dtype).contiguous()
+    counts = expert_token_counts.to(torch.int32).contiguous()
+    offsets = expert_token_offsets.to(torch.int32).contiguous()
+    idx = sorted_to_orig_token_idx.to(torch.int32).contiguous()
+    if counts.numel() != E or offsets.numel() != E + 1 or idx.numel() != T:
+        raise ValueError("routing tables must have shapes [E], [E+1], [T]")
+    C = torch.empty((T, N), dtype=dtype, device=A.device)
+    if T == 0 or N == 0:
+        return C
+    lib = _lib.load()
+    ws_bytes = lib.hx_moe_workspace_bytes(T, E)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=A.device)
+    rc = lib.hx_moe_grouped_gemm(A.data_ptr(), W.data_ptr(), C.data_ptr(), counts.data_ptr(), offsets.data_ptr(),
+                                 idx.data_ptr(), T, K, N, E, max_T_per_expert, _DT[dtype], ws.data_ptr(), ws_bytes,
+                                 _stream_ptr(A.device))
+    _lib.check(rc, "hx_moe_grouped_gemm")
+    return C
+
+
+@moe_matmul_ogs_op.register_fake
+def _(A, W, expert_token_counts, expert_token_offsets, sorted_to_orig_token_idx, max_T_per_expert):
+    return A.new_empty((A.shape[0], W.shape[2]), dtype=torch.promote_types(A.dtype, W.dtype))

@@ -1,0 +1,94 @@
+/* C ABI of libhx_kernels.so — hand-written gfx950 (MI355X) kernels behind the three Helion example
+ * entry points fp8_gemm, fp8_attention_kernel and moe_matmul_ogs.
+ *
+ * Conventions (all functions):
+ *   - plain pointers and sizes only; every pointer is DEVICE memory owned by the caller;
+ *   - the library never allocates, frees or retains device memory; scratch comes in through the
+ *     `workspace` arguments (sizes from the hx_*_workspace_bytes queries);
+ *   - kernels are enqueued on `stream` (a hipStream_t passed as void*; NULL = default stream),
+ *     nothing synchronises the host;
+ *   - return 0 on success; a negative value is an argument/shape error detected before any
+ *     launch; a positive value is the hipError_t of a failed launch.  hx_last_error() returns a
+ *     thread-local message for the last non-zero return.
+ */
+#ifndef HX_KERNELS_H
+#define HX_KERNELS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element type tags used by out_dtype / dtype arguments */
+enum {
+  HX_F16 = 0,
+  HX_BF16 = 1,
+  HX_F32 = 2,
+  HX_E4M3 = 3 /* OCP float8_e4m3fn */
+};
+
+/* error codes (negative returns) */
+enum {
+  HX_ERR_BAD_ARG = -1,     /* null pointer, negative size, unknown dtype tag */
+  HX_ERR_UNSUPPORTED = -2, /* shape/stride/alignment outside what the kernels handle */
+  HX_ERR_WORKSPACE = -3    /* workspace missing or too small */
+};
+
+int hx_version(void);
+const char* hx_last_error(void);
+
+/* Replaces the device side of `fp8_gemm(x, y)` (reference: examples/fp8_gemm.py:29-57, whose
+ * generated launcher is test/test_examples.expected:821-841) and of its baseline
+ * `torch._scaled_mm` call (examples/fp8_gemm.py:61-78).
+ *   c[m,n] = cast( (sum_k f32(a[m,k]) * f32(b[k,n])) * (scale_a*scale_b) )
+ * a: [M,K] e4m3fn, element (m,k) at a[m*lda + k].
+ * b: [K,N] e4m3fn, element (k,n) at b[k*ldb_k + n*ldb_n]  (ldb_k==1: "column-major" B, the layout
+ *    torch._scaled_mm wants; ldb_n==1: row-major B as the example's check() feeds).
+ * c: [M,N] of out_dtype (HX_F16 = reference default, HX_BF16, HX_F32), element (m,n) at c[m*ldc+n].
+ * scale_a/scale_b: device pointers to one fp32 each, or NULL for 1.0 (the reference hard-codes
+ *    1.0, helion/language/matmul_ops.py:232-233).
+ * Chooses between the 256x256 MFMA tile kernel, the skinny (M<=16) wave-split-K kernel and a
+ * bounds-checked general kernel from the shape, strides and alignment. */
+int hx_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int64_t lda,
+                int64_t ldb_k, int64_t ldb_n, int64_t ldc, const float* scale_a, const float* scale_b,
+                int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
+size_t hx_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/* Which kernel hx_fp8_gemm would launch for these arguments: 0 general, 1 tile256, 2 skinny.
+ * (Diagnostic; lets tests assert that the fast paths are the ones exercised.) */
+int hx_fp8_gemm_path(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n,
+                     int64_t ldc, const void* a, const void* b, const void* c);
+
+/* Replaces the device side of `fp8_attention_kernel(q, k, v, batch, heads)` (reference:
+ * examples/fp8_attention.py:22-106; generated kernel test/test_examples.expected:718-766).
+ * q,k: [BH,S,D] e4m3fn contiguous; v: [BH,D,S] e4m3fn contiguous (pre-transposed);
+ * out: [BH,S,D] contiguous (== [batch,heads,S,D]) of out_dtype HX_E4M3 (reference) or HX_F32.
+ * exact_max != 0: two passes, P is quantised to e4m3 against the exact row max (bit-faithful to
+ *   the reference's ref-eager execution); exact_max == 0: one pass, online softmax, P quantised
+ *   against the running max (what the reference's compiled kernel does).
+ * Supported: D == 128 or 64, S % 64 == 0. */
+int hx_fp8_attention(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t S,
+                     int64_t D, int out_dtype, int exact_max, void* stream);
+
+/* Replaces the device side of `moe_matmul_ogs(A, W, expert_token_counts, expert_token_offsets,
+ * sorted_to_orig_token_idx, max_T_per_expert_tensor)` (reference: examples/moe_matmul_ogs.py:25-80;
+ * semantics = moe_matmul_ogs_reference, :125-148).
+ *   for each expert e, for i in [0, counts[e]):  r = idx[offsets[e]+i];  C[r,:] = cast(A[r,:] @ W[e])
+ *   rows of C that no expert covers are set to zero.
+ * A: [T,K] row-major; W: [E,K,N] row-major (N contiguous); C: [T,N] row-major; dtype HX_BF16 or
+ * HX_F16 for all three; counts [E], offsets [E+1], idx [T] are int32 device arrays.
+ * max_T (the numel of the reference's dummy tensor) is accepted for signature parity and is only
+ * validated (>= 0); the tile table is built on the device from counts/offsets.
+ * workspace: hx_moe_workspace_bytes(T, E) bytes, 16-byte aligned. */
+int hx_moe_grouped_gemm(const void* A, const void* W, void* C, const int32_t* counts,
+                        const int32_t* offsets, const int32_t* idx, int64_t T, int64_t K, int64_t N,
+                        int64_t E, int64_t max_T, int dtype, void* workspace, size_t workspace_bytes,
+                        void* stream);
+size_t hx_moe_workspace_bytes(int64_t T, int64_t E);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HX_KERNELS_H */
