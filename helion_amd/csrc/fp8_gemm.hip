@@ -370,7 +370,7 @@ extern "C" int hx_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int
     return HX_ERR_BAD_ARG;
   }
   if (M == 0 || N == 0) return 0;
-  if (!a || !b || !c) {
+  if (!c || (K > 0 && (!a || !b))) {
     hx_set_error("hx_fp8_gemm: null operand pointer");
     return HX_ERR_BAD_ARG;
   }

@@ -1,0 +1,65 @@
+"""The C-ABI library loads, exports every symbol include/hx_kernels.h declares, and rejects bad
+arguments before touching the GPU (so these run without one)."""
+import ctypes
+import pathlib
+import re
+
+import pytest
+
+from helion_amd import _lib
+
+ROOT = pathlib.Path(__file__).resolve().parent.parent
+
+
+def _declared_symbols():
+    text = (ROOT / "include" / "hx_kernels.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(hx_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    assert _declared_symbols() == sorted(_lib.exported_symbols())
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(str(_lib.lib_path()))
+    for name in _declared_symbols():
+        assert hasattr(lib, name), f"{name} declared in include/hx_kernels.h but not exported"
+    assert _lib.load().hx_version() >= 1
+
+
+def test_gemm_argument_errors_are_reported_without_a_launch():
+    lib = _lib.load()
+    assert lib.hx_fp8_gemm(None, None, None, -1, 4, 4, 4, 1, 4, 4, None, None, 0, None, 0, None) == -1
+    assert b"negative" in lib.hx_last_error()
+    assert lib.hx_fp8_gemm(None, None, None, 4, 4, 4, 4, 1, 4, 4, None, None, 0, None, 0, None) == -1
+    assert b"null" in lib.hx_last_error()
+    assert lib.hx_fp8_gemm(1, 1, 1, 4, 4, 4, 4, 1, 4, 4, None, None, 9, None, 0, None) == -1  # bad dtype tag
+    assert lib.hx_fp8_gemm(1, 1, 1, 4, 4, 8, 4, 1, 8, 4, None, None, 0, None, 0, None) == -1  # lda < K
+    assert lib.hx_fp8_gemm(None, None, None, 0, 4, 4, 4, 1, 4, 4, None, None, 0, None, 0, None) == 0  # empty
+    with pytest.raises(ValueError):
+        _lib.check(-1, "x")
+
+
+def test_gemm_path_selection():
+    lib = _lib.load()
+    A = 1 << 20  # any 16-byte aligned fake address; the query never dereferences
+    assert lib.hx_fp8_gemm_path(8192, 8192, 8192, 8192, 1, 8192, 8192, A, A, A) == 1
+    assert lib.hx_fp8_gemm_path(16, 28672, 8192, 8192, 1, 8192, 28672, A, A, A) == 2
+    assert lib.hx_fp8_gemm_path(1, 512, 256, 256, 1, 256, 512, A, A, A) == 2
+    assert lib.hx_fp8_gemm_path(256, 256, 256, 256, 256, 1, 256, A, A, A) == 0  # row-major B
+    assert lib.hx_fp8_gemm_path(100, 70, 50, 50, 1, 50, 70, A, A, A) == 0  # ragged
+    assert lib.hx_fp8_gemm_path(256, 256, 256, 256, 1, 256, 256, A + 1, A, A) == 0  # misaligned
+
+
+def test_attention_and_moe_argument_errors():
+    lib = _lib.load()
+    assert lib.hx_fp8_attention(1, 1, 1, 1, -1, 64, 64, 3, 1, None) == -1
+    assert lib.hx_fp8_attention(16, 16, 16, 16, 2, 100, 64, 3, 1, None) == -2  # S % 64
+    assert lib.hx_fp8_attention(16, 16, 16, 16, 2, 128, 96, 3, 1, None) == -2  # D
+    assert lib.hx_fp8_attention(16, 16, 16, 16, 2, 128, 64, 1, 1, None) == -1  # bf16 output not offered
+    assert lib.hx_fp8_attention(None, None, None, None, 0, 128, 64, 3, 1, None) == 0
+    assert lib.hx_moe_workspace_bytes(1000, 30) >= 1000
+    assert lib.hx_moe_grouped_gemm(16, 16, 16, 16, 16, 16, 8, 8, 8, 2, 8, 2, None, 0, None) == -1  # f32 tag
+    assert lib.hx_moe_grouped_gemm(16, 16, 16, 16, 16, 16, 8, 8, 8, 2, 8, 1, None, 0, None) == -3  # no workspace
+    assert b"workspace" in lib.hx_last_error()

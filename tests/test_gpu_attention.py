@@ -1,0 +1,104 @@
+"""GPU parity of hx_fp8_attention against the CPU oracle (ref-eager semantics), the golden fixture,
+closed-form cases, and at the benchmark size sampled heads plus key-permutation invariance."""
+import pathlib
+
+import numpy as np
+import pytest
+import torch
+
+import helion_amd as hx
+from helion_amd import inputs
+from oracle import oracle as orc
+from tests._util import TOL, rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+E4M3 = torch.float8_e4m3fn
+G = pathlib.Path(__file__).resolve().parent / "golden"
+
+
+def _run(q, k, v, b, h, **kw):
+    return hx.fp8_attention_kernel(q.to(DEV), k.to(DEV), v.to(DEV), b, h, **kw)
+
+
+@pytest.mark.parametrize("b,h,s,d", [(1, 2, 128, 64), (2, 4, 256, 64), (4, 8, 512, 128),  # examples/fp8_attention.py:291-293
+                                     (1, 1, 64, 64), (1, 3, 192, 128), (1, 9, 320, 128), (2, 5, 64, 128), (1, 1, 1024, 128)])
+def test_exact_max_vs_oracle(b, h, s, d):
+    q, k, v = inputs.attention_inputs(b, h, s, d, seed=s + d + h)
+    ref32 = orc.fp8_attention(q, k, v, b, h, torch.float32)
+    out32 = _run(q, k, v, b, h, out_dtype=torch.float32)
+    assert out32.shape == (b, h, s, d)
+    assert rel_err(out32, ref32) <= TOL
+    out8 = _run(q, k, v, b, h)
+    assert out8.dtype == E4M3
+    ref8 = orc.fp8_attention(q, k, v, b, h)
+    # after e4m3 output rounding a single differing code is 1/8..1/16 of that element; compare as values
+    assert rel_err(out8, ref8) <= 0.08
+    assert (out8.cpu().view(torch.uint8) == ref8.view(torch.uint8)).float().mean().item() > 0.98
+
+
+@pytest.mark.parametrize("b,h,s,d", [(2, 4, 256, 64), (1, 2, 512, 128)])
+def test_online_mode_tracks_the_oracle_loosely(b, h, s, d):
+    # running-max quantisation of P deviates by a few percent from the exact-max reference by construction
+    q, k, v = inputs.attention_inputs(b, h, s, d, seed=5)
+    ref = orc.fp8_attention(q, k, v, b, h, torch.float32)
+    out = _run(q, k, v, b, h, out_dtype=torch.float32, exact_max=False)
+    assert rel_err(out, ref) <= 0.08
+
+
+def test_golden_fixture():
+    z = np.load(G / "fp8_attention_small.npz")
+    for name in ("d64", "d128"):
+        b, h, s, d = (int(x) for x in z[f"{name}_shape"])
+        q, k, v = (torch.from_numpy(z[f"{name}_{t}"].copy()).view(E4M3) for t in "qkv")
+        out = _run(q, k, v, b, h, out_dtype=torch.float32)
+        assert rel_err(out, torch.from_numpy(z[f"{name}_out_f32"].copy())) <= TOL
+
+
+def test_uniform_scores_give_mean_of_v_and_single_hot_key():
+    s, d = 128, 128
+    g = torch.Generator().manual_seed(6)
+    q = torch.zeros(1, s, d).to(E4M3)
+    k = torch.randn(1, s, d, generator=g).to(E4M3)
+    v = torch.randn(1, d, s, generator=g).to(E4M3)
+    out = _run(q, k, v, 1, 1, out_dtype=torch.float32)[0, 0].cpu()
+    mean = orc.dq(v)[0].double().mean(1).float()
+    assert torch.allclose(out, mean.expand(s, d), rtol=0, atol=2e-6)
+    # one key dominates by a huge margin: output is that key's value row
+    q2 = torch.zeros(1, s, d); k2 = torch.zeros(1, s, d)
+    q2[0, :, 0] = 16.0; k2[0, 37, 0] = 448.0
+    out2 = _run(q2.to(E4M3), k2.to(E4M3), v, 1, 1, out_dtype=torch.float32)[0, 0].cpu()
+    assert torch.allclose(out2, orc.dq(v)[0][:, 37].expand(s, d), rtol=0, atol=1e-6)
+
+
+def test_tritonbench_thunk_and_layout():
+    torch.manual_seed(42)
+    q, k, v = (torch.randn(2, 3, 128, 64, dtype=torch.float16) for _ in range(3))
+    fn = hx.fp8_attention_tritonbench(q.to(DEV), k.to(DEV), v.to(DEV))
+    out = fn()
+    assert out.shape == (2, 3, 128, 64) and out.dtype == E4M3
+    q8, k8, v8 = orc.preprocess_fp8_attention_inputs(q, k, v)
+    assert rel_err(out, orc.fp8_attention(q8, k8, v8, 2, 3)) <= 0.08
+
+
+def test_unsupported_shapes_raise():
+    x = torch.zeros(1, 100, 64).to(E4M3).to(DEV)
+    with pytest.raises(ValueError, match="unsupported shape"):
+        hx.fp8_attention_kernel(x, x, torch.zeros(1, 64, 100).to(E4M3).to(DEV), 1, 1)
+    y = torch.zeros(2, 64, 64).to(E4M3).to(DEV)
+    with pytest.raises(ValueError):
+        hx.fp8_attention_kernel(y, y, y, 1, 1)  # batch*heads mismatch
+
+
+def test_c4_sampled_heads_and_key_permutation():
+    b, h, s, d = 4, 32, 4096, 128
+    q, k, v = inputs.attention_c4()
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    out = hx.fp8_attention_kernel(qd, kd, vd, b, h, out_dtype=torch.float32)
+    for bh in (0, 77, 127):
+        ref = orc.fp8_attention(q[bh : bh + 1], k[bh : bh + 1], v[bh : bh + 1], 1, 1, torch.float32)
+        assert rel_err(out[bh // h, bh % h], ref[0, 0]) <= TOL
+    perm = torch.randperm(s, generator=torch.Generator().manual_seed(1)).to(DEV)
+    out_p = hx.fp8_attention_kernel(qd, kd[:, perm].contiguous(), vd[:, :, perm].contiguous(), b, h, out_dtype=torch.float32)
+    # same exact row max, same quantisation grid; only MFMA summation order differs
+    assert rel_err(out_p, out) <= 5e-3

@@ -1,0 +1,132 @@
+"""GPU parity of hx_fp8_gemm (all three kernels) against the CPU oracle, the golden fixture and, at the
+benchmark sizes, sampled rows plus a checksum identity.  Everything goes through the C ABI."""
+import ctypes
+import pathlib
+
+import numpy as np
+import pytest
+import torch
+
+import helion_amd as hx
+from helion_amd import _lib, inputs
+from oracle import oracle as orc
+from tests._util import TOL, rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+E4M3 = torch.float8_e4m3fn
+G = pathlib.Path(__file__).resolve().parent / "golden"
+
+
+def _path(m, n, k):
+    return _lib.load().hx_fp8_gemm_path(m, n, k, k, 1, k, n, 1 << 20, 1 << 20, 1 << 20)
+
+
+@pytest.mark.parametrize("m,n,k,path", [
+    (256, 256, 256, 1), (512, 512, 512, 1), (1024, 1024, 1024, 1), (256, 768, 128, 1), (768, 256, 1152, 1),
+    (16, 512, 1024, 2), (1, 16, 128, 2), (5, 48, 256, 2), (16, 1000, 384, 2), (9, 33, 8192 + 128, 2), (16, 64, 16384, 2),
+    (100, 70, 50, 0), (17, 256, 256, 0), (256, 256, 200, 0), (3, 5, 7, 0), (64, 64, 0, 0),
+])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_shapes_vs_oracle(m, n, k, path, out_dtype):
+    assert _path(m, n, k) == path
+    a, b, sa, sb = inputs.gemm_scaled(m, n, k, seed=m + 31 * n + 7 * k)
+    out = hx.fp8_gemm(a.to(DEV), b.to(DEV), scale_a=sa.to(DEV), scale_b=sb.to(DEV), out_dtype=out_dtype)
+    assert out.dtype == out_dtype and out.shape == (m, n)
+    ref = orc.fp8_gemm(a, b, sa, sb, out_dtype)
+    assert rel_err(out, ref) <= (1e-2 if out_dtype != torch.float32 else 1e-4)
+
+
+def test_reference_call_form_and_defaults():
+    # examples/fp8_gemm.py:95-109: randn -> e4m3, row-major y, fp16 result, unit scales
+    g = torch.Generator().manual_seed(0)
+    for m, k, n in [(256, 256, 256), (512, 512, 512)]:
+        x = torch.randn(m, k, generator=g).to(E4M3); y = torch.randn(k, n, generator=g).to(E4M3)
+        out = hx.fp8_gemm(x.to(DEV), y.to(DEV))
+        assert out.dtype == torch.float16
+        assert rel_err(out, orc.fp8_gemm(x, y)) <= 1e-2
+        base = hx.reference_fp8_gemm_pytorch(x.to(DEV), y.to(DEV))
+        torch.testing.assert_close(out.float(), base.float(), rtol=1e-2, atol=1e-1)  # helion/_testing.py:376-381
+        assert torch.equal(hx.fp8_gemm_tritonbench(x.to(DEV), y.to(DEV)), out)
+
+
+def test_golden_fixture():
+    z = np.load(G / "fp8_gemm_small.npz")
+    for name in ("ragged", "skinny"):
+        x = torch.from_numpy(z[f"{name}_x"].copy()).view(E4M3).to(DEV)
+        yt = torch.from_numpy(z[f"{name}_yt"].copy()).view(E4M3).to(DEV)
+        sa, sb = (torch.tensor(float(s), device=DEV) for s in z[f"{name}_scales"])
+        out = hx.fp8_gemm(x, yt.T, scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16)
+        ref = torch.from_numpy(z[f"{name}_out_bf16"].copy()).view(torch.bfloat16)
+        assert rel_err(out, ref) <= 1e-2
+        ref16 = torch.from_numpy(z[f"{name}_out_f16_unit"].copy()).view(torch.float16)
+        assert rel_err(hx.fp8_gemm(x, yt.T), ref16) <= 1e-2
+
+
+def test_direct_c_abi_call_with_padded_leading_dimensions():
+    lib = _lib.load()
+    m, n, k, lda, ldb, ldc = 256, 512, 384, 512, 400, 520
+    g = torch.Generator().manual_seed(3)
+    abuf = torch.randn(m, lda, generator=g).to(E4M3); bbuf = torch.randn(n, ldb, generator=g).to(E4M3)
+    ad, bd = abuf.to(DEV), bbuf.to(DEV)
+    cd = torch.full((m, ldc), 7.0, dtype=torch.bfloat16, device=DEV)
+    rc = lib.hx_fp8_gemm(ad.data_ptr(), bd.data_ptr(), cd.data_ptr(), m, n, k, lda, 1, ldb, ldc, None, None, _lib.HX_BF16,
+                         None, 0, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, lib.hx_last_error()
+    torch.cuda.synchronize()
+    ref = orc.fp8_gemm(abuf[:, :k], bbuf[:, :k].T, out_dtype=torch.bfloat16)
+    assert rel_err(cd[:, :n], ref) <= 1e-2
+    assert bool((cd[:, n:] == 7.0).all())  # padding columns untouched
+
+
+def test_noncontiguous_x_and_nan_propagation():
+    g = torch.Generator().manual_seed(4)
+    big = torch.randn(64, 512, generator=g).to(E4M3)
+    x = big[:, ::2]  # stride 2 along k -> the op makes it contiguous
+    y = torch.randn(256, 128, generator=g).to(E4M3)
+    out = hx.fp8_gemm(x.to(DEV), y.to(DEV), out_dtype=torch.float32)
+    assert rel_err(out, orc.fp8_gemm(x.contiguous(), y, out_dtype=torch.float32)) <= 1e-4
+    xn = torch.randn(256, 256, generator=g).to(E4M3); yn = torch.randn(256, 256, generator=g).to(E4M3)
+    xb = xn.view(torch.uint8).clone(); xb[5, 17] = 0x7F
+    xn = xb.view(E4M3)
+    out = hx.fp8_gemm(xn.to(DEV), yn.T.contiguous().T.to(DEV), out_dtype=torch.float32).cpu()
+    assert bool(torch.isnan(out[5]).all()) and not bool(torch.isnan(out[[0, 4, 6, 255]]).any())
+
+
+def test_linearity_in_power_of_two_scales():
+    a, b, sa, sb = inputs.gemm_scaled(256, 256, 512, 9, DEV)
+    o1 = hx.fp8_gemm(a, b, scale_a=sa, scale_b=sb, out_dtype=torch.float32)
+    o2 = hx.fp8_gemm(a, b, scale_a=sa * 2, scale_b=sb * 4, out_dtype=torch.float32)
+    assert torch.equal(o2, o1 * 8)
+    assert torch.equal(hx.fp8_gemm(a, b, out_dtype=torch.float32), hx.fp8_gemm(a, b, out_dtype=torch.float32))  # deterministic
+
+
+def test_c1_1024_cube_matches_ref_eager_form():
+    a, b = inputs.gemm_c1()
+    out = hx.fp8_gemm(a.to(DEV), b.to(DEV), out_dtype=torch.bfloat16)
+    ref = orc.fp8_gemm(a, b, out_dtype=torch.bfloat16)
+    assert rel_err(out, ref) <= 1e-2
+
+
+def test_c3_decode_shape_full_oracle():
+    a, b, sa, sb = inputs.gemm_c3()
+    assert _path(16, 28672, 8192) == 2
+    out = hx.fp8_gemm(a.to(DEV), b.to(DEV), scale_a=sa.to(DEV), scale_b=sb.to(DEV), out_dtype=torch.bfloat16)
+    ref = orc.fp8_gemm(a, b, sa, sb, torch.bfloat16)
+    assert rel_err(out, ref) <= 1e-2
+
+
+def test_c2_8192_cube_sampled_rows_and_checksum():
+    a, b, sa, sb = inputs.gemm_c2()
+    ad, bd = a.to(DEV), b.to(DEV)
+    out = hx.fp8_gemm(ad, bd, scale_a=sa.to(DEV), scale_b=sb.to(DEV), out_dtype=torch.bfloat16)
+    rows = torch.arange(0, 8192, 67)  # 123 rows spread over every row tile
+    ref = orc.fp8_gemm(a[rows], b, sa, sb, torch.bfloat16)
+    assert rel_err(out[rows.to(DEV)], ref) <= 1e-2
+    # checksum of checksums: sum_n C[m,n] == alpha * A[m,:] . (sum_n B[:,n]); bf16 rounding noise averages out
+    alpha = float(sa) * float(sb)
+    bsum = orc.dq(b.T.contiguous()).double().sum(0)  # [K]
+    expect = (orc.dq(a).double() @ bsum) * alpha
+    got = out.double().sum(1).cpu()
+    scale = (orc.dq(a).double().abs() @ orc.dq(b.T.contiguous()).double().abs().sum(0)) * alpha
+    assert float(((got - expect).abs() / scale).max()) < 1e-4

@@ -1,0 +1,80 @@
+"""GPU parity of hx_moe_grouped_gemm against the CPU oracle (= moe_matmul_ogs_reference semantics), the
+golden fixture, ragged/empty-expert edge cases and sampled rows at the benchmark size."""
+import pathlib
+
+import numpy as np
+import pytest
+import torch
+
+import helion_amd as hx
+from helion_amd import inputs
+from oracle import oracle as orc
+from tests._util import TOL, rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+G = pathlib.Path(__file__).resolve().parent / "golden"
+
+
+def _run(A, W, ex):
+    args = hx.moe_matmul_ogs_helion_kernel_args_gen(A.to(DEV), W.to(DEV), ex.to(DEV))
+    return hx.moe_matmul_ogs(*args)
+
+
+@pytest.mark.parametrize("T,K,N,E,topk,dtype", [
+    (1000, 500, 200, 30, 1, torch.float16),    # examples/moe_matmul_ogs.py:186 (general kernel)
+    (512, 256, 512, 4, 1, torch.bfloat16),     # tile256 kernel
+    (700, 128, 256, 5, 1, torch.float16),
+    (2048, 512, 768, 8, 2, torch.bfloat16),    # top-2 expanded rows
+    (300, 64, 256, 16, 1, torch.bfloat16),     # most tiles nearly empty
+    (37, 100, 19, 3, 1, torch.bfloat16),
+])
+def test_shapes_vs_oracle(T, K, N, E, topk, dtype):
+    A, W, ex = inputs.moe_inputs(T // topk, K, N, E, topk, seed=T + K, dtype=dtype)
+    out = _run(A, W, ex)
+    assert out.dtype == dtype and out.shape == (A.shape[0], N)
+    assert rel_err(out, orc.moe_matmul_ogs_reference(A, W, ex)) <= 1e-2
+
+
+def test_golden_fixture():
+    z = np.load(G / "moe_small.npz")
+    for name, dt in (("bf16", torch.bfloat16), ("f16", torch.float16)):
+        A = torch.from_numpy(z[f"{name}_A"].copy()).view(dt); W = torch.from_numpy(z[f"{name}_W"].copy()).view(dt)
+        ex = torch.from_numpy(z[f"{name}_expert"].copy())
+        ref = torch.from_numpy(z[f"{name}_out"].copy()).view(dt)
+        assert rel_err(_run(A, W, ex), ref) <= 1e-2
+
+
+@pytest.mark.parametrize("K,N", [(128, 256), (96, 40)])
+def test_empty_experts_and_uncovered_rows_are_zero(K, N):
+    A, W, ex = inputs.moe_inputs(400, K, N, 6, 1, seed=1, dtype=torch.bfloat16)
+    ex[ex == 2] = 4  # expert 2 empty
+    A_, W_, counts, offsets, idx, mt = hx.moe_matmul_ogs_helion_kernel_args_gen(A.to(DEV), W.to(DEV), ex.to(DEV))
+    counts2 = counts.clone(); counts2[1] = 0  # expert 1 switched off: its rows must come out zero
+    out = hx.moe_matmul_ogs(A_, W_, counts2, offsets, idx, mt).cpu()
+    ref = orc.moe_matmul_ogs(A, W, counts2.cpu(), offsets.cpu(), idx.cpu())
+    assert rel_err(out, ref) <= 1e-2
+    assert bool((out[ex == 1] == 0).all())
+
+
+def test_all_rows_one_expert_equals_dense_matmul():
+    g = torch.Generator().manual_seed(2)
+    A = torch.randn(512, 256, generator=g).bfloat16(); W = (torch.randn(3, 256, 256, generator=g) * 0.1).bfloat16()
+    ex = torch.full((512,), 2)
+    out = _run(A, W, ex)
+    assert rel_err(out, (A.float() @ W[2].float()).bfloat16()) <= 1e-2
+
+
+def test_c5_sampled_rows():
+    A, W, ex = inputs.moe_c5()
+    assert A.shape == (32768, 4096) and W.shape == (8, 4096, 14336)
+    Ad, Wd, exd = A.to(DEV), W.to(DEV), ex.to(DEV)
+    out = hx.moe_matmul_ogs(*hx.moe_matmul_ogs_helion_kernel_args_gen(Ad, Wd, exd))
+    g = torch.Generator().manual_seed(0)
+    for e in range(8):
+        rows = (ex == e).nonzero(as_tuple=True)[0]
+        pick = rows[torch.randperm(rows.numel(), generator=g)[:48]]
+        ref = (A[pick].float() @ W[e].float()).bfloat16()
+        assert rel_err(out[pick.to(DEV)], ref) <= 1e-2
+    # top-2: the two rows of a token hold the same activations but different experts
+    assert not torch.equal(out[0], out[1])

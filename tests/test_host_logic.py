@@ -1,0 +1,75 @@
+"""Host-side mirror of the reference's Python entry points: signatures, routing prep, preprocessing,
+shape inference of the registered ops, and loud failure off-GPU."""
+import inspect
+
+import pytest
+import torch
+
+import helion_amd as hx
+from oracle import oracle as orc
+
+
+def test_signatures_match_the_reference_entry_points():
+    # examples/fp8_gemm.py:30, examples/fp8_attention.py:23-29, examples/moe_matmul_ogs.py:26-33
+    assert list(inspect.signature(hx.fp8_gemm).parameters)[:2] == ["x", "y"]
+    assert list(inspect.signature(hx.fp8_attention_kernel).parameters)[:5] == ["q", "k", "v", "batch", "heads"]
+    assert list(inspect.signature(hx.moe_matmul_ogs).parameters) == [
+        "A", "W", "expert_token_counts", "expert_token_offsets", "sorted_to_orig_token_idx", "max_T_per_expert_tensor"]
+    for name, p in inspect.signature(hx.fp8_gemm).parameters.items():
+        if name not in ("x", "y"):
+            assert p.kind is inspect.Parameter.KEYWORD_ONLY
+    assert inspect.signature(hx.fp8_gemm).parameters["out_dtype"].default is torch.float16
+    assert inspect.signature(hx.fp8_attention_kernel).parameters["out_dtype"].default is torch.float8_e4m3fn
+
+
+def test_args_gen_matches_oracle_on_cpu():
+    g = torch.Generator().manual_seed(0)
+    A = torch.randn(64, 8, generator=g).half(); W = torch.randn(5, 8, 8, generator=g).half()
+    ex = torch.randint(5, (64,), generator=g)
+    ours = hx.moe_matmul_ogs_helion_kernel_args_gen(A, W, ex)
+    ref = orc.moe_args_gen(A, W, ex)
+    for a, b in zip(ours[2:5], ref[2:5]):
+        assert torch.equal(a, b)
+    assert ours[5].numel() == ref[5].numel()
+
+
+def test_preprocess_matches_oracle_on_cpu():
+    g = torch.Generator().manual_seed(1)
+    q, k, v = (torch.randn(2, 3, 16, 8, generator=g) for _ in range(3))
+    for a, b in zip(hx.preprocess_fp8_attention_inputs(q, k, v), orc.preprocess_fp8_attention_inputs(q, k, v)):
+        assert torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+    assert hx.preprocess_fp8_attention_inputs(q, k, v)[2].shape == (6, 8, 16)
+
+
+def test_ops_refuse_cpu_tensors():
+    x = torch.zeros(4, 4).to(torch.float8_e4m3fn)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        hx.fp8_gemm(x, x)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        hx.fp8_attention_kernel(x.reshape(1, 4, 4), x.reshape(1, 4, 4), x.reshape(1, 4, 4), 1, 1)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        hx.moe_matmul_ogs(torch.zeros(4, 4).half(), torch.zeros(1, 4, 4).half(), torch.zeros(1, dtype=torch.int32),
+                          torch.zeros(2, dtype=torch.int32), torch.zeros(4, dtype=torch.int32), torch.empty(4))
+
+
+def test_registered_ops_infer_shapes_on_meta_tensors():
+    x = torch.empty(32, 64, dtype=torch.float8_e4m3fn, device="meta")
+    y = torch.empty(64, 48, dtype=torch.float8_e4m3fn, device="meta")
+    out = torch.ops.helion_amd.fp8_gemm(x, y, None, None, torch.float16)
+    assert out.shape == (32, 48) and out.dtype == torch.float16
+    q = torch.empty(6, 128, 64, dtype=torch.float8_e4m3fn, device="meta")
+    v = torch.empty(6, 64, 128, dtype=torch.float8_e4m3fn, device="meta")
+    o = torch.ops.helion_amd.fp8_attention(q, q, v, 2, 3, torch.float8_e4m3fn, True)
+    assert o.shape == (2, 3, 128, 64) and o.dtype == torch.float8_e4m3fn
+    A = torch.empty(10, 8, dtype=torch.bfloat16, device="meta"); W = torch.empty(3, 8, 12, dtype=torch.bfloat16, device="meta")
+    i32 = lambda n: torch.empty(n, dtype=torch.int32, device="meta")
+    c = torch.ops.helion_amd.moe_matmul_ogs(A, W, i32(3), i32(4), i32(10), 5)
+    assert c.shape == (10, 12) and c.dtype == torch.bfloat16
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from helion_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "_LIB_PATH", tmp_path / "nope.so")
+    with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
+        _lib.load()

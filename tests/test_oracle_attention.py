@@ -1,0 +1,102 @@
+"""Pins oracle.fp8_attention against: the literal single-tile walk of the reference kernel body, a float64
+brute force written independently in C, and closed-form special cases."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+
+E4M3 = torch.float8_e4m3fn
+
+
+def _inputs(b, h, s, d, seed, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    q, k, v = (torch.randn(b, h, s, d, generator=g).to(dtype) for _ in range(3))
+    return orc.preprocess_fp8_attention_inputs(q, k, v)
+
+
+def test_scale_constant_matches_the_golden_literal():
+    # test/test_examples.expected:742-743 shows 0.18033688 for D=64
+    assert float(orc.attention_scale(64)) == np.float32(0.18033688)
+    assert float(orc.attention_scale(128)) == np.float32((1.0 / math.sqrt(128.0)) * 1.44269504)
+
+
+@pytest.mark.parametrize("b,h,s,d", [(1, 2, 128, 64), (2, 2, 256, 64), (1, 1, 64, 128)])
+def test_closed_form_equals_literal_walk(b, h, s, d):
+    q, k, v = _inputs(b, h, s, d, 42, torch.float16)  # examples/fp8_attention.py:267-272 uses seed 42, fp16
+    lit = orc.fp8_attention_literal(q, k, v, b, h)
+    closed = orc.fp8_attention(q, k, v, b, h)
+    assert torch.equal(lit.view(torch.uint8), closed.view(torch.uint8))
+    assert not torch.isnan(closed.float()).any()
+
+
+@pytest.mark.parametrize("s,d", [(8, 16), (32, 32), (16, 64)])
+def test_against_float64_bruteforce(oracle_c, s, d):
+    q, k, v = _inputs(1, 1, s, d, 3)
+    out = np.empty((s, d), dtype=np.float32)
+    qb, kb, vb = (t[0].contiguous().view(torch.uint8).numpy().copy() for t in (q, k, v))
+    oracle_c.orc_fp8_attention_f64(qb.ctypes.data, kb.ctypes.data, vb.ctypes.data, out.ctypes.data, s, d)
+    got = orc.fp8_attention(q, k, v, 1, 1, torch.float32)[0, 0].numpy()
+    # identical quantisation points, only summation precision differs (an exp2 ulp can flip an e4m3 tie
+    # in principle; none does for these seeds)
+    assert np.abs(got - out).max() <= 2e-6 * max(1.0, np.abs(out).max())
+
+
+def test_single_key_returns_v():
+    d = 32
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(2, 1, d, generator=g).to(E4M3)
+    k = torch.randn(2, 1, d, generator=g).to(E4M3)
+    v = torch.randn(2, d, 1, generator=g).to(E4M3)
+    out = orc.fp8_attention(q, k, v, 1, 2, torch.float32)
+    assert torch.equal(out[0, :, 0, :], orc.dq(v)[:, :, 0])  # p == 1, l == 1
+
+
+def test_uniform_scores_give_mean_of_v():
+    s, d = 16, 32
+    q = torch.zeros(1, s, d).to(E4M3)  # all scores 0 -> p = 1 everywhere, exactly representable
+    g = torch.Generator().manual_seed(6)
+    k = torch.randn(1, s, d, generator=g).to(E4M3)
+    v = torch.randn(1, d, s, generator=g).to(E4M3)
+    out = orc.fp8_attention(q, k, v, 1, 1, torch.float32)[0, 0]
+    mean = orc.dq(v)[0].double().mean(dim=1).float()
+    assert torch.allclose(out, mean.expand(s, d), rtol=0, atol=1e-6)
+
+
+def test_p_is_quantised_but_l_is_not():
+    # two keys, scores chosen so p = [1, 2^-0.5]: e4m3(0.70710678) = 0.6875, l = 1.70710678
+    d = 16
+    q = torch.zeros(1, 1, d); k = torch.zeros(1, 2, d)
+    q[0, 0, 0] = 2.0
+    c = float(orc.attention_scale(d))
+    # want (q.k1 - q.k0)*c = -0.5  ->  k1[0]-k0[0] = -0.25/c ; pick representable values by search
+    cands = orc.E4M3_DECODE_TABLE[:0x7F]
+    best = min(((abs((2.0 * float(a)) * c - 0.5), float(a)) for a in cands), key=lambda t: t[0])[1]
+    k[0, 0, 0] = best
+    v = torch.zeros(1, d, 2); v[0, :, 0] = 0.0; v[0, :, 1] = 1.0
+    q8, k8, v8 = q.to(E4M3), k.to(E4M3), v.to(E4M3)
+    s0 = np.float32(np.float32(2.0 * best) * np.float32(c))
+    p1 = np.exp2(np.float32(0.0) - s0, dtype=np.float32)
+    p1_q = float(orc.e4m3_decode(orc.e4m3_encode(np.array([p1], dtype=np.float32)))[0])
+    expect = np.float32(p1_q) / (np.float32(1.0) + p1)
+    out = orc.fp8_attention(q8, k8, v8, 1, 1, torch.float32)[0, 0, 0, 0].item()
+    assert abs(out - float(expect)) <= 1e-7
+    assert p1_q != float(p1)  # the case really exercises the quantisation
+
+
+def test_key_permutation_invariance():
+    q, k, v = _inputs(1, 1, 64, 32, 7)
+    perm = torch.randperm(64, generator=torch.Generator().manual_seed(8))
+    a = orc.fp8_attention(q, k, v, 1, 1, torch.float32)
+    b = orc.fp8_attention(q, k[:, perm], v[:, :, perm], 1, 1, torch.float32)
+    assert torch.allclose(a, b, rtol=0, atol=2e-6)
+
+
+def test_output_layout_batch_heads():
+    q, k, v = _inputs(2, 3, 64, 16, 9)
+    out = orc.fp8_attention(q, k, v, 2, 3, torch.float32)
+    assert out.shape == (2, 3, 64, 16)
+    one = orc.fp8_attention(q[4:5], k[4:5], v[4:5], 1, 1, torch.float32)
+    assert torch.equal(out[1, 1], one[0, 0])  # bh = 4 -> b = 1, h = 1 (examples/fp8_attention.py:56-57)
