@@ -31,10 +31,8 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
                                                           long ldc, const float* __restrict__ scale_a,
                                                           const float* __restrict__ scale_b, int tiles_m, int tiles_n) {
   typedef typename OutT<OUT>::T out_t;
-  __shared__ __attribute__((aligned(1024))) uint8_t sA0[T256_TILE_BYTES];
-  __shared__ __attribute__((aligned(1024))) uint8_t sA1[T256_TILE_BYTES];
-  __shared__ __attribute__((aligned(1024))) uint8_t sB0[T256_TILE_BYTES];
-  __shared__ __attribute__((aligned(1024))) uint8_t sB1[T256_TILE_BYTES];
+  // [stage][A|B][256 rows x 128 B]
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[2][2][T256_TILE_BYTES];
 
   // ---- workgroup -> tile. Workgroup i runs on XCD i%8 (each XCD has its own 4 MB L2): give every
   // XCD a contiguous range of a grouped (8 tile-rows tall) raster so concurrently resident tiles of
@@ -58,25 +56,24 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = w >> 1, wn = w & 1;
 
-  // ---- DMA addressing: wave w owns tile rows [64w, 64w+64); instruction j covers rows 64w+8j .. +7
+  // ---- DMA addressing: wave w owns tile rows [64w, 64w+64); instruction j covers rows 64w+8j .. +7.
+  // address = uniform base (row block, k-tile) + per-lane offset (row in block, swizzled chunk)
   const int lrow = lane >> 3, lpos = lane & 7;
-  const int coff0 = (lpos ^ ((lrow >> 1) & 7)) * 16;        // j even: swz = (lrow>>1)
-  const int coff1 = (lpos ^ ((4 + (lrow >> 1)) & 7)) * 16;  // j odd : swz = 4 + (lrow>>1)
-  const uint8_t* gA = A + (m0 + w * 64 + lrow) * lda;
-  const uint8_t* gB = Bt + (n0 + w * 64 + lrow) * ldb;
+  const uint32_t a_vo0 = (uint32_t)(lrow * lda + (lpos ^ ((lrow >> 1) & 7)) * 16);        // j even
+  const uint32_t a_vo1 = (uint32_t)(lrow * lda + (lpos ^ ((4 + (lrow >> 1)) & 7)) * 16);  // j odd
+  const uint32_t b_vo0 = (uint32_t)(lrow * ldb + (lpos ^ ((lrow >> 1) & 7)) * 16);
+  const uint32_t b_vo1 = (uint32_t)(lrow * ldb + (lpos ^ ((4 + (lrow >> 1)) & 7)) * 16);
+  const uint8_t* gA = A + (m0 + w * 64) * lda;   // wave-uniform
+  const uint8_t* gB = Bt + (n0 + w * 64) * ldb;  // wave-uniform
+  const uint32_t lds0 = hx_lds_addr(&smem[0][0][0]) + (uint32_t)w * 64 * 128;
 
-  auto issue = [&](int kt, uint8_t* sa, uint8_t* sb) {
+  auto issue = [&](int kt, int stage) {
     const long kb = (long)kt * T256_BK;
+    const uint32_t la = lds0 + (uint32_t)stage * 2 * T256_TILE_BYTES, lb = la + T256_TILE_BYTES;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int co = (j & 1) ? coff1 : coff0;
-      hx_g2l16(gA + (long)j * 8 * lda + kb + co, sa + (w * 64 + j * 8) * 128);
-    }
+    for (int j = 0; j < 8; ++j) hx_g2l16_s(gA + (long)j * 8 * lda + kb, (j & 1) ? a_vo1 : a_vo0, la + j * 1024);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int co = (j & 1) ? coff1 : coff0;
-      hx_g2l16(gB + (long)j * 8 * ldb + kb + co, sb + (w * 64 + j * 8) * 128);
-    }
+    for (int j = 0; j < 8; ++j) hx_g2l16_s(gB + (long)j * 8 * ldb + kb, (j & 1) ? b_vo1 : b_vo0, lb + j * 1024);
   };
 
   // ---- MFMA operand addressing
@@ -93,43 +90,73 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  auto compute = [&](const uint8_t* sa, const uint8_t* sb) {
+  // Fragments of one 64-byte k-step: 4 A blocks + 4 B blocks of 32 rows, 8 VGPRs each.
+  auto load_frags = [&](v8i(&af)[4], v8i(&bf)[4], int stage, int t) {
+    const uint8_t* sa = &smem[stage][0][0];
+    const uint8_t* sb = &smem[stage][1][0];
+    const int o0 = x ^ (t * 64), o1 = x ^ (t * 64 + 16);
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      v8i af[4], bf[4];
-      const int o0 = x ^ (t * 64), o1 = x ^ (t * 64 + 16);
+    for (int i = 0; i < 4; ++i) {
+      v4i lo = *(const v4i*)(sa + a_base + i * 4096 + o0);
+      v4i hi = *(const v4i*)(sa + a_base + i * 4096 + o1);
+      af[i] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        v4i lo = *(const v4i*)(sa + a_base + i * 4096 + o0);
-        v4i hi = *(const v4i*)(sa + a_base + i * 4096 + o1);
-        af[i] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        v4i lo = *(const v4i*)(sb + b_base + i * 4096 + o0);
-        v4i hi = *(const v4i*)(sb + b_base + i * 4096 + o1);
-        bf[i] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-      }
-#pragma unroll
-      for (int bj = 0; bj < 4; ++bj)
-#pragma unroll
-        for (int bi = 0; bi < 4; ++bi) acc[bj][bi] = hx_mfma_32x32x64_e4m3(bf[bj], af[bi], acc[bj][bi]);
+    for (int i = 0; i < 4; ++i) {
+      v4i lo = *(const v4i*)(sb + b_base + i * 4096 + o0);
+      v4i hi = *(const v4i*)(sb + b_base + i * 4096 + o1);
+      bf[i] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
     }
   };
+  auto mma = [&](v8i(&af)[4], v8i(&bf)[4]) {
+#pragma unroll
+    for (int bj = 0; bj < 4; ++bj)
+#pragma unroll
+      for (int bi = 0; bi < 4; ++bi) acc[bj][bi] = hx_mfma_32x32x64_e4m3(bf[bj], af[bi], acc[bj][bi]);
+  };
+  // two LDS reads slotted after each of the first 8 MFMAs: the 16 reads of the next k-step hide under
+  // the MFMAs and have all returned by the time the last MFMAs of the step issue
+  auto interleave = [&]() {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // 2 DS reads
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+  };
 
+  // Software pipeline.  k-tile kt lives in stage kt&1.  While the MFMAs of (kt, t=0) run, the fragments
+  // of (kt, t=1) are fetched; then one barrier says "tile kt+1 has landed in every wave's view and nobody
+  // reads stage kt&1 any more", the DMA of tile kt+2 is issued into the stage just freed, and the MFMAs
+  // of (kt, t=1) run while the fragments of (kt+1, t=0) are fetched.
   const int nk = K / T256_BK;
-  issue(0, sA0, sB0);
-  for (int kt = 0; kt < nk; kt += 2) {
+  v8i fa0[4], fb0[4], fa1[4], fb1[4];
+  issue(0, 0);
+  if (nk > 1) issue(1, 1);
+  if (nk > 1) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(16)); else HX_WAIT_VM0();
+  __syncthreads();
+  load_frags(fa0, fb0, 0, 0);
+  for (int kt = 0; kt < nk - 1; ++kt) {
+    const int stage = kt & 1;
+    load_frags(fa1, fb1, stage, 1);
+    mma(fa0, fb0);
+    interleave();
+    __builtin_amdgcn_sched_barrier(0);
     HX_WAIT_VM0();
     __syncthreads();
-    if (kt + 1 < nk) issue(kt + 1, sA1, sB1);
-    compute(sA0, sB0);
-    if (kt + 1 < nk) {
-      HX_WAIT_VM0();
-      __syncthreads();
-      if (kt + 2 < nk) issue(kt + 2, sA0, sB0);
-      compute(sA1, sB1);
-    }
+    if (kt + 2 < nk) issue(kt + 2, stage);
+    load_frags(fa0, fb0, stage ^ 1, 0);
+    mma(fa1, fb1);
+    interleave();
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  {
+    const int stage = (nk - 1) & 1;
+    load_frags(fa1, fb1, stage, 1);
+    mma(fa0, fb0);
+    interleave();
+    __builtin_amdgcn_sched_barrier(0);
+    mma(fa1, fb1);
   }
 
   // ---- epilogue: acc[bj][bi][4a+b] is C[m0 + wm*128 + bi*32 + lane%32][n0 + wn*128 + bj*32 + 8a + 4g + b]
@@ -325,7 +352,7 @@ extern "C" int hx_fp8_gemm_path(int64_t M, int64_t N, int64_t K, int64_t lda, in
                       aligned(b, 16) && K >= 128;
   if (kmajor && M <= 16 && lda >= K && ldb_n >= K) return 2;
   if (kmajor && (M % 256 == 0) && (N % 256 == 0) && (ldc % 4 == 0) && aligned(c, 16) &&
-      M * lda < (1LL << 31) && N * ldb_n < (1LL << 31))
+      lda < (1LL << 27) && ldb_n < (1LL << 27))
     return 1;
   return 0;
 }

@@ -28,6 +28,18 @@ __device__ __forceinline__ void hx_g2l16(const void* gptr, void* lds_wave_base) 
   __builtin_amdgcn_global_load_lds(HX_GLB(gptr), HX_LDS(lds_wave_base), 16, 0, 0);
 }
 
+// Same DMA, spelled in assembly with a wave-uniform 64-bit base (SGPR pair) plus a per-lane 32-bit
+// byte offset.  The compiler does not track this load: the caller orders it with HX_WAIT_VM0() and a
+// barrier before any lane reads the destination.  (Keeping it out of the compiler's sight is the
+// point: its own tracking waits for every outstanding DMA before *any* LDS read of an array it cannot
+// tell apart from the destination, which would serialise the prefetch with the MFMA loop.)
+__device__ __forceinline__ void hx_g2l16_s(const void* sbase, uint32_t voff, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_wave_base), "v"(voff), "s"(sbase) : "memory", "m0");
+}
+__device__ __forceinline__ uint32_t hx_lds_addr(const void* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t*)p;
+}
+
 // s_waitcnt encodings (gfx9): vmcnt [3:0]+[15:14], expcnt [6:4], lgkmcnt [11:8]
 #define HX_WAIT_VM0() __builtin_amdgcn_s_waitcnt(0x0F70)
 #define HX_WAIT_LGKM0() __builtin_amdgcn_s_waitcnt(0xC07F)

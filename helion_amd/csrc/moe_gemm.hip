@@ -110,10 +110,8 @@ __global__ __launch_bounds__(256) void hx_moe_tile256(const uint8_t* __restrict_
                                                      int N, int max_tiles, int tiles_n) {
   typedef typename Mfma16<BF>::T out_t;
   typedef typename Mfma16<BF>::V8 V8;
-  __shared__ __attribute__((aligned(1024))) uint8_t sA0[MOE_TILE_BYTES];
-  __shared__ __attribute__((aligned(1024))) uint8_t sA1[MOE_TILE_BYTES];
-  __shared__ __attribute__((aligned(1024))) uint8_t sW0[MOE_TILE_BYTES];
-  __shared__ __attribute__((aligned(1024))) uint8_t sW1[MOE_TILE_BYTES];
+  // [stage][A|W][32 KB]
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[2][2][MOE_TILE_BYTES];
 
   // XCD-contiguous grouped raster over (row tile, column tile), as in the fp8 GEMM
   int tile;
@@ -137,32 +135,37 @@ __global__ __launch_bounds__(256) void hx_moe_tile256(const uint8_t* __restrict_
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = w >> 1, wn = w & 1;
 
-  // ---- A DMA: wave w owns tile rows [64w, 64w+64), 8 instructions of 8 rows; rows are gathered
+  // ---- A DMA: wave w owns tile rows [64w, 64w+64), 8 instructions of 8 rows; rows are gathered, so the
+  // per-lane byte offset carries the row (A is below 4 GB, checked by the host).
   const int lrow = lane >> 3, lpos = lane & 7;
-  const int coff0 = (lpos ^ ((lrow >> 1) & 7)) * 16;
-  const int coff1 = (lpos ^ ((4 + (lrow >> 1)) & 7)) * 16;
-  const uint8_t* arow[8];
+  uint32_t a_vo[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     int lr = w * 64 + j * 8 + lrow;
     lr = lr < mt.rows ? lr : 0;  // padded rows re-read row 0 of the tile; never stored
     int r = idx[mt.row_start + lr];
     r = (r >= 0 && r < T) ? r : 0;
-    arow[j] = A + (long)r * K * 2 + ((j & 1) ? coff1 : coff0);
+    const int swz = ((j & 1) ? 4 + (lrow >> 1) : (lrow >> 1)) & 7;
+    a_vo[j] = (uint32_t)r * (uint32_t)(K * 2) + (uint32_t)((lpos ^ swz) * 16);
   }
-  // ---- W DMA: wave w owns k rows [16w, 16w+16), 8 instructions of 2 rows x 512 B
-  const uint8_t* We = W + (long)mt.expert * K * N * 2 + n0 * 2;
+  // ---- W DMA: wave w owns k rows [16w, 16w+16), 8 instructions of 2 rows x 512 B.
+  // row k = 16w + 2j + (lane>>5); chunk = (lane&31) ^ ((k&7)<<1); (k&7) = (2j + (lane>>5)) & 7
+  const uint8_t* We = W + (long)mt.expert * K * N * 2 + n0 * 2 + (long)(w * 16) * N * 2;  // wave-uniform
   const int wk_l = lane >> 5, wpos = lane & 31;
+  uint32_t w_vo[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) w_vo[j] = (uint32_t)(wk_l * N * 2 + ((wpos ^ (((2 * j + wk_l) & 7) << 1)) * 16));
+  const uint32_t lds0 = hx_lds_addr(&smem[0][0][0]);
 
-  auto issue = [&](int kt, uint8_t* sa, uint8_t* sw) {
+  auto issue = [&](int kt, int stage) {
+    const uint32_t la = lds0 + (uint32_t)stage * 2 * MOE_TILE_BYTES + (uint32_t)w * 64 * 128;
+    const uint32_t lw = lds0 + (uint32_t)stage * 2 * MOE_TILE_BYTES + MOE_TILE_BYTES + (uint32_t)w * 16 * 512;
+    const uint8_t* ak = A + (long)kt * 128;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) hx_g2l16(arow[j] + (long)kt * 128, sa + (w * 64 + j * 8) * 128);
+    for (int j = 0; j < 8; ++j) hx_g2l16_s(ak, a_vo[j], la + j * 1024);
+    const uint8_t* wk = We + (long)kt * MOE_BK * N * 2;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int k = w * 16 + j * 2 + wk_l;
-      const int chunk = wpos ^ ((k & 7) << 1);
-      hx_g2l16(We + ((long)kt * MOE_BK + k) * N * 2 + chunk * 16, sw + (w * 16 + j * 2) * 512);
-    }
+    for (int j = 0; j < 8; ++j) hx_g2l16_s(wk + (long)(2 * j) * N * 2, w_vo[j & 3], lw + j * 1024);
   };
 
   // ---- operand addressing
@@ -174,6 +177,14 @@ __global__ __launch_bounds__(256) void hx_moe_tile256(const uint8_t* __restrict_
   const int tb = lane >> 4, te = (lane >> 2) & 3, tq = lane & 3;
   const int tk = 8 * (tb >> 1) + te;                  // + 16*ks + 4*half
   const int tn_ = wn * 128 + 16 * (tb & 1) + 4 * tq;  // + 32*bj
+  // byte offset of (k = tk + 4*half, n = tn_) in the W tile.  Column block bj adds 4 to the chunk index in bits
+  // the swizzle mask and tn_>>3 leave alone, so it is an xor with 64*bj; k-step ks adds 16 rows = 8192 bytes.
+  int w_off[2];
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    const int k = tk + 4 * half;
+    w_off[half] = k * 512 + (((tn_ >> 3) ^ ((k & 7) << 1)) * 16) + (tn_ & 7) * 2;
+  }
 
   v16f acc[4][4];
 #pragma unroll
@@ -183,46 +194,64 @@ __global__ __launch_bounds__(256) void hx_moe_tile256(const uint8_t* __restrict_
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  auto compute = [&](const uint8_t* sa, const uint8_t* sw) {
+  // fragments of one k-step (16 k): 4 A blocks (one b128 each) and 4 W blocks (two transposing b64 each)
+  auto load_frags = [&](V8(&af)[4], V8(&wf)[4], int stage, int ks) {
+    const uint8_t* sa = &smem[stage][0][0];
+    const uint8_t* sw = &smem[stage][1][0];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      V8 af[4], wf[4];
+    for (int i = 0; i < 4; ++i) af[i] = *(const V8*)(sa + a_base + i * 4096 + (ax ^ (ks * 32)));
 #pragma unroll
-      for (int i = 0; i < 4; ++i) af[i] = *(const V8*)(sa + a_base + i * 4096 + (ax ^ (ks * 32)));
+    for (int bj = 0; bj < 4; ++bj) {
+      v4s part[2];
 #pragma unroll
-      for (int bj = 0; bj < 4; ++bj) {
-        v4s part[2];
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          const int k = 16 * ks + 4 * half + tk;
-          const int n = tn_ + 32 * bj;
-          const int pos = (n >> 3) ^ ((k & 7) << 1);
-          const uint8_t* p = sw + k * 512 + pos * 16 + (n & 7) * 2;
-          part[half] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3)))*)p);
-        }
-        v8s both = (v8s){part[0][0], part[0][1], part[0][2], part[0][3], part[1][0], part[1][1], part[1][2], part[1][3]};
-        wf[bj] = __builtin_bit_cast(V8, both);
+      for (int half = 0; half < 2; ++half) {
+        const int off = (w_off[half] ^ (bj * 64)) + ks * 8192;
+        part[half] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3)))*)(sw + off));
       }
-#pragma unroll
-      for (int bj = 0; bj < 4; ++bj)
-#pragma unroll
-        for (int bi = 0; bi < 4; ++bi) acc[bj][bi] = Mfma16<BF>::run(wf[bj], af[bi], acc[bj][bi]);
+      v8s both = (v8s){part[0][0], part[0][1], part[0][2], part[0][3], part[1][0], part[1][1], part[1][2], part[1][3]};
+      wf[bj] = __builtin_bit_cast(V8, both);
     }
   };
+  auto mma = [&](V8(&af)[4], V8(&wf)[4]) {
+#pragma unroll
+    for (int bj = 0; bj < 4; ++bj)
+#pragma unroll
+      for (int bi = 0; bi < 4; ++bi) acc[bj][bi] = Mfma16<BF>::run(wf[bj], af[bi], acc[bj][bi]);
+  };
+  auto interleave = [&]() {  // 12 LDS reads under the first 12 of 16 MFMAs
+#pragma unroll
+    for (int i = 0; i < 12; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+  };
 
+  // software pipeline, as in the fp8 GEMM: k-tile kt in stage kt&1, four k-steps per tile, fragments double
+  // buffered; the one barrier per tile sits before the last k-step's MFMAs.
   const int nk = K / MOE_BK;
-  issue(0, sA0, sW0);
-  for (int kt = 0; kt < nk; kt += 2) {
+  V8 fa0[4], fw0[4], fa1[4], fw1[4];
+  issue(0, 0);
+  if (nk > 1) issue(1, 1);
+  if (nk > 1) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(16)); else HX_WAIT_VM0();
+  __syncthreads();
+  load_frags(fa0, fw0, 0, 0);
+  for (int kt = 0; kt < nk - 1; ++kt) {
+    const int stage = kt & 1;
+    load_frags(fa1, fw1, stage, 1); mma(fa0, fw0); interleave(); __builtin_amdgcn_sched_barrier(0);
+    load_frags(fa0, fw0, stage, 2); mma(fa1, fw1); interleave(); __builtin_amdgcn_sched_barrier(0);
+    load_frags(fa1, fw1, stage, 3); mma(fa0, fw0); interleave(); __builtin_amdgcn_sched_barrier(0);
     HX_WAIT_VM0();
     __syncthreads();
-    if (kt + 1 < nk) issue(kt + 1, sA1, sW1);
-    compute(sA0, sW0);
-    if (kt + 1 < nk) {
-      HX_WAIT_VM0();
-      __syncthreads();
-      if (kt + 2 < nk) issue(kt + 2, sA0, sW0);
-      compute(sA1, sW1);
-    }
+    if (kt + 2 < nk) issue(kt + 2, stage);
+    load_frags(fa0, fw0, stage ^ 1, 0); mma(fa1, fw1); interleave(); __builtin_amdgcn_sched_barrier(0);
+  }
+  {
+    const int stage = (nk - 1) & 1;
+    load_frags(fa1, fw1, stage, 1); mma(fa0, fw0); interleave(); __builtin_amdgcn_sched_barrier(0);
+    load_frags(fa0, fw0, stage, 2); mma(fa1, fw1); interleave(); __builtin_amdgcn_sched_barrier(0);
+    load_frags(fa1, fw1, stage, 3); mma(fa0, fw0); interleave(); __builtin_amdgcn_sched_barrier(0);
+    mma(fa1, fw1);
   }
 
   // ---- epilogue: acc[bj][bi][4a+b] is C[idx[row_start + wm*128 + bi*32 + lane%32]][n0 + wn*128 + bj*32 + 8a + 4g + b]
@@ -320,7 +349,7 @@ template <bool BF>
 static int launch_moe(const void* A, const void* W, void* C, const int32_t* counts, const int32_t* offsets, const int32_t* idx,
                       int64_t T, int64_t K, int64_t N, int64_t E, void* ws, hipStream_t s) {
   typedef typename Mfma16<BF>::T T16;
-  const bool fast = (K % MOE_BK == 0) && (N % MOE_BN == 0) && K >= MOE_BK && (((uintptr_t)A | (uintptr_t)W | (uintptr_t)C) & 15) == 0;
+  const bool fast = (K % MOE_BK == 0) && (N % MOE_BN == 0) && K >= MOE_BK && (T * K * 2 < (1LL << 32)) && (N * 4 < (1LL << 31)) && (((uintptr_t)A | (uintptr_t)W | (uintptr_t)C) & 15) == 0;
   const int bm = fast ? MOE_BM : 64;
   const int max_tiles = (int)moe_max_tiles(T, E, bm);
   int* num_tiles = (int*)ws;
