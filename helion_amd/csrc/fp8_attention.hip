@@ -19,12 +19,22 @@
 #define ATT_BN 64      // keys per tile
 #define ATT_WAVES 4
 #define ATT_BM (32 * ATT_WAVES)
+#define ATT_NS 4       // LDS stages: tiles j .. j+2 are in flight while tile j is consumed
+#define ATT_LEAD (ATT_NS - 1)
 
 // K tile: [64 keys][D bytes]; V tile: [D rows][64 bytes].  Rows are 16-byte chunks, swizzled:
 //   row bytes 128: pos = chunk ^ ((row >> 1) & 7);   row bytes 64: pos = chunk ^ ((row >> 2) & 3)
 template <int RB>
 __device__ __forceinline__ int att_swz(int row) {
   return RB == 128 ? ((row >> 1) & 7) : ((row >> 2) & 3);
+}
+
+// wait until at most `newer` tiles' worth of this wave's DMA instructions (IPT per tile) are outstanding
+template <int IPT>
+__device__ __forceinline__ void att_wait_tiles(int newer) {
+  if (newer >= 2) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(2 * IPT));
+  else if (newer == 1) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(IPT));
+  else __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(0));
 }
 
 template <int D, int OUT, bool EXACT>
@@ -34,23 +44,20 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
   constexpr int KSTEPS = D / 64;  // MFMA k-steps for S = K Q^T
   constexpr int DB = D / 32;      // 32-row blocks of O^T
   constexpr int KROWS_PER_DMA = 1024 / D;
-  constexpr int K_DMAS = ATT_BN / KROWS_PER_DMA;  // per tile
-  constexpr int V_DMAS = D / 16;                  // 16 rows of 64 B per DMA
-  __shared__ __attribute__((aligned(1024))) uint8_t sK0[ATT_BN * D];
-  __shared__ __attribute__((aligned(1024))) uint8_t sK1[ATT_BN * D];
-  __shared__ __attribute__((aligned(1024))) uint8_t sV0[D * ATT_BN];
-  __shared__ __attribute__((aligned(1024))) uint8_t sV1[D * ATT_BN];
+  constexpr int KPW = (ATT_BN / KROWS_PER_DMA) / ATT_WAVES;  // K DMA instructions per wave per tile
+  constexpr int VPW = (D / 16) / ATT_WAVES;                  // V DMA instructions per wave per tile (16 rows x 64 B each)
+  constexpr int TILE = ATT_BN * D;                           // bytes of a K tile == bytes of a V tile
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[ATT_NS][2][TILE];
 
   // workgroup -> (head, query tile): XCD x (= id%8) takes heads x, x+8, ...; the query tiles of a head
   // are consecutive on that XCD so its K/V stay in that XCD's L2.
   int bh, qt;
   {
     const int id = blockIdx.x, xcd = id & 7, loc = id >> 3;
-    const int hpx = (BH + 7) >> 3;  // heads per xcd (upper bound)
     const int hl = loc / qtiles;
     qt = loc % qtiles;
     bh = xcd + 8 * hl;
-    if (hl >= hpx || bh >= BH) return;  // whole workgroup exits together
+    if (bh >= BH) return;  // whole workgroup exits together
   }
   const int tid = threadIdx.x, lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -74,24 +81,27 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
     }
   }
 
-  // ---- DMA addressing.  K: one instruction = KROWS_PER_DMA rows of D bytes.
+  // ---- DMA addressing: wave w issues K instructions j = w, w+4, ... (KROWS_PER_DMA rows of D bytes each) and
+  // V instructions j = w, w+4, ... (16 rows of 64 bytes each).  The swizzle of a lane's row does not depend on
+  // which of the wave's instructions it is, so one per-lane offset serves all of them.
   constexpr int KCPR = D / 16;  // chunks per K row
   const int k_lrow = lane / KCPR, k_lpos = lane % KCPR;
-  auto issue_k = [&](int tile, uint8_t* sk) {
+  const uint32_t k_vo = (uint32_t)(k_lrow * D + ((k_lpos ^ att_swz<D>(w * KROWS_PER_DMA + k_lrow)) * 16));
+  const int v_lrow = lane >> 2, v_lpos = lane & 3;
+  const uint32_t v_vo = (uint32_t)(v_lrow * S + ((v_lpos ^ att_swz<64>(v_lrow)) * 16));
+  const uint32_t lds0 = hx_lds_addr(&smem[0][0][0]);
+  auto issue_k = [&](int tile, int stage) {
 #pragma unroll
-    for (int j = w; j < K_DMAS; j += ATT_WAVES) {
-      const int row = j * KROWS_PER_DMA + k_lrow;
-      const int chunk = k_lpos ^ att_swz<D>(row);
-      hx_g2l16(Kh + (long)(tile * ATT_BN + row) * D + chunk * 16, sk + j * 1024);
+    for (int jj = 0; jj < KPW; ++jj) {
+      const int j = w + ATT_WAVES * jj;
+      hx_g2l16_s(Kh + ((long)tile * ATT_BN + j * KROWS_PER_DMA) * D, k_vo, lds0 + (uint32_t)stage * 2 * TILE + j * 1024);
     }
   };
-  const int v_lrow = lane >> 2, v_lpos = lane & 3;
-  auto issue_v = [&](int tile, uint8_t* sv) {
+  auto issue_v = [&](int tile, int stage) {
 #pragma unroll
-    for (int j = w; j < V_DMAS; j += ATT_WAVES) {
-      const int row = j * 16 + v_lrow;
-      const int chunk = v_lpos ^ att_swz<64>(row);
-      hx_g2l16(Vh + (long)row * S + tile * ATT_BN + chunk * 16, sv + j * 1024);
+    for (int jj = 0; jj < VPW; ++jj) {
+      const int j = w + ATT_WAVES * jj;
+      hx_g2l16_s(Vh + (long)(j * 16) * S + (long)tile * ATT_BN, v_vo, lds0 + (uint32_t)stage * 2 * TILE + TILE + j * 1024);
     }
   };
 
@@ -115,7 +125,7 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
   const float c = (float)((1.0 / __builtin_sqrt((double)D)) * 1.44269504);
   const int ntiles = S / ATT_BN;
 
-  auto scores = [&](const uint8_t* sk, v16f (&s)[2]) {
+  auto scores = [&](const uint8_t* sk, v16f(&s)[2]) {
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
@@ -130,41 +140,49 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
     }
   };
 
-  float m_run = -__builtin_inff();  // scaled-domain row max
+  // The Q loads above are the only memory operations the compiler tracks; retire them here so that it has no
+  // reason to put a vmcnt wait (which would also wait for every DMA in flight) inside the key loops.
+  HX_WAIT_VM0();
 
+  float neg_m = __builtin_inff();  // minus the scaled-domain row max
+
+  // Both key loops are software pipelined by one tile: the score MFMAs of tile j+1 are issued before the
+  // VALU work on tile j's scores, so the matrix pipe runs under the softmax arithmetic.
+  // LDS slots: tile t lives in slot t % 4.  At iteration j the wave reads K of tile j+1 and V of tile j while
+  // tiles j+2 and j+3 are in flight; the barrier at the top of iteration j is what frees slot (j+3) % 4.
   if (EXACT) {
-    // ---------------- pass 1: exact row max of the raw scores
-    float smax = -__builtin_inff();
-    issue_k(0, sK0);
-    for (int j = 0; j < ntiles; j += 2) {
-      HX_WAIT_VM0();
-      __syncthreads();
-      if (j + 1 < ntiles) issue_k(j + 1, sK1);
+    // ---------------- pass 1: exact row max of the raw scores (K tiles only)
+    float smax0 = -__builtin_inff(), smax1 = -__builtin_inff();
+    for (int t = 0; t < ATT_LEAD && t < ntiles; ++t) issue_k(t, t % ATT_NS);
+    att_wait_tiles<KPW>(min(ATT_LEAD - 1, ntiles - 1));
+    __syncthreads();
+    // one tile: sync, prefetch, issue the score MFMAs of tile j+1 into `next`, then reduce tile j's scores (`cur`)
+    auto step1 = [&](v16f(&cur)[2], v16f(&next)[2], int j) {
+      if (j + 2 < ntiles) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(KPW));  // tile j+1 landed, tile j+2 may be in flight
+      else HX_WAIT_VM0();
+      __syncthreads();  // tile j+1 visible to every wave; every wave is done with tile j-1
+      if (j + ATT_LEAD < ntiles) issue_k(j + ATT_LEAD, (j + ATT_LEAD) % ATT_NS);
       if (active) {
-        v16f s[2];
-        scores(sK0, s);
+        if (j + 1 < ntiles) scores(&smem[(j + 1) % ATT_NS][0][0], next);
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) smax = fmaxf(smax, s[kb][r]);
-      }
-      if (j + 1 < ntiles) {
-        HX_WAIT_VM0();
-        __syncthreads();
-        if (j + 2 < ntiles) issue_k(j + 2, sK0);
-        if (active) {
-          v16f s[2];
-          scores(sK1, s);
-#pragma unroll
-          for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) smax = fmaxf(smax, s[kb][r]);
+        for (int r = 0; r < 16; r += 2) {
+          smax0 = fmaxf(fmaxf(smax0, cur[0][r]), cur[0][r + 1]);
+          smax1 = fmaxf(fmaxf(smax1, cur[1][r]), cur[1][r + 1]);
         }
       }
+    };
+    v16f sa[2], sb[2];
+    if (active) scores(&smem[0][0][0], sa);
+    int j = 0;
+    for (; j + 1 < ntiles; j += 2) {
+      step1(sa, sb, j);
+      step1(sb, sa, j + 1);
     }
+    if (j < ntiles) step1(sa, sb, j);
+    float smax = fmaxf(smax0, smax1);
     smax = fmaxf(smax, __shfl_xor(smax, 32));
-    m_run = smax * c;  // max(s*c) == max(s)*c for c > 0 (rounding is monotone)
-    __syncthreads();   // all waves done with sK0/sK1 before pass 2 overwrites them
+    neg_m = -(smax * c);  // max(s*c) == max(s)*c for c > 0 (rounding is monotone)
+    __syncthreads();      // all waves done with the last K tiles before pass 2 overwrites the slots
   }
 
   // ---------------- pass 2 (or the only pass)
@@ -173,45 +191,46 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
   for (int d = 0; d < DB; ++d)
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[d][r] = 0.f;
-  float l_lane = 0.f;
+  float l4[4] = {0.f, 0.f, 0.f, 0.f};  // four independent partial row sums per lane
+  v8i pf = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  auto tile_step = [&](const uint8_t* sk, const uint8_t* sv) {
-    v16f s[2];
-    scores(sk, s);
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) s[kb][r] = __fmul_rn(s[kb][r], c);
+  auto softmax_pv = [&](v16f(&s)[2], const uint8_t* sv) {
     if (!EXACT) {
-      float tmax = s[0][0];
+      float t0 = s[0][0], t1 = s[1][0];
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s[kb][r]);
+      for (int r = 0; r < 16; r += 2) {
+        t0 = fmaxf(fmaxf(t0, s[0][r]), s[0][r + 1]);
+        t1 = fmaxf(fmaxf(t1, s[1][r]), s[1][r + 1]);
+      }
+      float tmax = fmaxf(t0, t1);
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-      const float m_new = fmaxf(m_run, tmax);
-      const float alpha = __builtin_amdgcn_exp2f(__fsub_rn(m_run, m_new));
-      l_lane *= alpha;
+      const float neg_new = fminf(neg_m, -(tmax * c));
+      const float alpha = __builtin_amdgcn_exp2f(neg_new - neg_m);  // exp2(m_old - m_new); first tile: exp2(-inf) = 0
+      if (__builtin_amdgcn_ballot_w64(neg_new != neg_m)) {  // wave-uniform: most tiles leave every row max alone
 #pragma unroll
-      for (int d = 0; d < DB; ++d)
+        for (int i = 0; i < 4; ++i) l4[i] *= alpha;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o[d][r] *= alpha;
-      m_run = m_new;
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[d][r] *= alpha;
+      }
+      neg_m = neg_new;
     }
-    v8i pf;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
       float p[16];
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        p[r] = __builtin_amdgcn_exp2f(__fsub_rn(s[kb][r], m_run));
-        l_lane += p[r];
+        // s*c - m fused into one rounding: the score already carries the fp8 MFMA's accumulation rounding,
+        // three orders of magnitude above the difference between one and two roundings here
+        p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][r], c, neg_m));
+        l4[r & 3] += p[r];
       }
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        int dw = HX_CVT_PK_E4M3(p[4 * j], p[4 * j + 1], 0, false);
-        dw = HX_CVT_PK_E4M3(p[4 * j + 2], p[4 * j + 3], dw, true);
-        pf[kb * 4 + j] = dw;
+        // both halves of the dword are overwritten, so the previous tile's value serves as the tied operand
+        int dw = HX_CVT_PK_E4M3(p[4 * j], p[4 * j + 1], pf[kb * 4 + j], false);
+        pf[kb * 4 + j] = HX_CVT_PK_E4M3(p[4 * j + 2], p[4 * j + 3], dw, true);
       }
     }
 #pragma unroll
@@ -223,26 +242,36 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
     }
   };
 
-  issue_k(0, sK0);
-  issue_v(0, sV0);
-  for (int j = 0; j < ntiles; j += 2) {
-    HX_WAIT_VM0();
-    __syncthreads();
-    if (j + 1 < ntiles) {
-      issue_k(j + 1, sK1);
-      issue_v(j + 1, sV1);
-    }
-    if (active) tile_step(sK0, sV0);
-    if (j + 1 < ntiles) {
-      HX_WAIT_VM0();
-      __syncthreads();
-      if (j + 2 < ntiles) {
-        issue_k(j + 2, sK0);
-        issue_v(j + 2, sV0);
-      }
-      if (active) tile_step(sK1, sV1);
-    }
+  for (int t = 0; t < ATT_LEAD && t < ntiles; ++t) {
+    issue_k(t, t % ATT_NS);
+    issue_v(t, t % ATT_NS);
   }
+  att_wait_tiles<KPW + VPW>(min(ATT_LEAD - 1, ntiles - 1));
+  __syncthreads();
+  {
+    auto step2 = [&](v16f(&cur)[2], v16f(&next)[2], int j) {
+      if (j + 2 < ntiles) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(KPW + VPW));
+      else HX_WAIT_VM0();
+      __syncthreads();
+      if (j + ATT_LEAD < ntiles) {
+        issue_k(j + ATT_LEAD, (j + ATT_LEAD) % ATT_NS);
+        issue_v(j + ATT_LEAD, (j + ATT_LEAD) % ATT_NS);
+      }
+      if (active) {
+        if (j + 1 < ntiles) scores(&smem[(j + 1) % ATT_NS][0][0], next);
+        softmax_pv(cur, &smem[j % ATT_NS][1][0]);
+      }
+    };
+    v16f sa[2], sb[2];
+    if (active) scores(&smem[0][0][0], sa);
+    int j = 0;
+    for (; j + 1 < ntiles; j += 2) {
+      step2(sa, sb, j);
+      step2(sb, sa, j + 1);
+    }
+    if (j < ntiles) step2(sa, sb, j);
+  }
+  const float l_lane = (l4[0] + l4[1]) + (l4[2] + l4[3]);
 
   if (!active) return;
   // ---------------- epilogue: o[db][4a+b] is O[q0 + lane%32][32 db + 8a + 4G + b]
@@ -316,7 +345,7 @@ extern "C" int hx_fp8_attention(const void* q, const void* k, const void* v, voi
     hx_set_error("hx_fp8_attention: pointers must be 16-byte aligned");
     return HX_ERR_UNSUPPORTED;
   }
-  if (BH * S * D >= (1LL << 40)) {
+  if (BH * S * D >= (1LL << 40) || S * D >= (1LL << 31)) {
     hx_set_error("hx_fp8_attention: problem too large");
     return HX_ERR_UNSUPPORTED;
   }

@@ -68,7 +68,9 @@ def test_uniform_scores_give_mean_of_v_and_single_hot_key():
     q2 = torch.zeros(1, s, d); k2 = torch.zeros(1, s, d)
     q2[0, :, 0] = 16.0; k2[0, 37, 0] = 448.0
     out2 = _run(q2.to(E4M3), k2.to(E4M3), v, 1, 1, out_dtype=torch.float32)[0, 0].cpu()
-    assert torch.allclose(out2, orc.dq(v)[0][:, 37].expand(s, d), rtol=0, atol=1e-6)
+    # the kernel forms s*c - m with one rounding where the reference has two: with scores this large (2^10)
+    # the winning key's p is 1 +- 2e-5 instead of exactly 1
+    assert torch.allclose(out2, orc.dq(v)[0][:, 37].expand(s, d), rtol=1e-4, atol=1e-6)
 
 
 def test_tritonbench_thunk_and_layout():
