@@ -4,8 +4,9 @@
 // Three kernels:
 //   hx_fp8_gemm_tile256 : 256x256x128 workgroup tile, 4 waves (2x2) of 128x128, 32x32x64 fp8 MFMA,
 //                         A/B k-tiles DMA'd global->LDS (double buffered, XOR-swizzled 16B chunks).
-//   hx_fp8_gemm_skinny  : M <= 16; HBM-bound streaming of B through 16x16x128 MFMA, K split across
-//                         the 8 waves of a workgroup, wave partials reduced through LDS.
+//   hx_fp8_gemm_skinny_direct : M <= 16, K <= 8192; HBM-bound streaming of B^T through registers into
+//                         16x16x128 MFMA, K split across the 8 waves of a workgroup, partials summed in LDS.
+//   hx_fp8_gemm_skinny  : M <= 16, larger K; same split, A panel staged through LDS in 8 KB chunks of K.
 //   hx_fp8_gemm_general : bounds-checked, arbitrary strides (fallback for ragged/unaligned inputs).
 #include "hx_common.h"
 
@@ -294,6 +295,111 @@ __global__ __launch_bounds__(512) void hx_fp8_gemm_skinny(const uint8_t* __restr
 }
 
 // ------------------------------------------------------------------------------------------
+// skinny, direct variant (M <= 16, K <= 8192): the bandwidth path.  No LDS on the load path.
+// Each of the 8 waves owns k-steps w, w+8, ... (at most 8) of every column group and keeps the matching A
+// fragments in registers for the whole kernel.  B^T goes straight to VGPRs with loads that cover whole
+// 128-byte lines: one instruction reads 8 rows x 128 B, lane (j = lane%16, g = lane/16) taking row j>>1,
+// chunk 2g + (j&1); a second instruction does rows 8..15 with the chunk parity flipped.  One exchange
+// between neighbouring lanes (DPP quad_perm [1,0,3,2]) then leaves lane (j, g) with chunks 2g and 2g+1 of
+// row (j>>1) + 8*(j&1): an MFMA B operand whose column j is that row.  (A lane must supply 32 bytes of ONE
+// row to the MFMA, and loads of 16 rows x 64 B per instruction run ~15 % slower than whole lines.)
+// The registers of a k-step are refilled with the same k-step of the next column group as soon as the MFMA
+// operand has been built from them, so about one column group per wave (128 KB per CU) is always in flight,
+// also across the barrier that sums the eight wave partials.
+// ------------------------------------------------------------------------------------------
+#define SKD_MAXS 8
+template <int OUT, bool FULL>  // FULL: K == 8192, every wave owns exactly 8 k-steps (no per-step predicates)
+__global__ __launch_bounds__(512) void hx_fp8_gemm_skinny_direct(const uint8_t* __restrict__ A, const uint8_t* __restrict__ Bt,
+                                                                typename OutT<OUT>::T* __restrict__ C, int M, int N, int K,
+                                                                long lda, long ldb, long ldc, const float* __restrict__ scale_a,
+                                                                const float* __restrict__ scale_b) {
+  typedef typename OutT<OUT>::T out_t;
+  __shared__ __attribute__((aligned(16))) float red[2][SK_WAVES][4][64];  // [parity][wave][r][lane]
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int j = lane & 15, g = lane >> 4, odd = j & 1;
+  const int steps = K >> 7;
+  const int nmine = FULL ? SKD_MAXS : (steps - w + SK_WAVES - 1) / SK_WAVES;  // this wave's k-steps (wave-uniform)
+
+  const int ncg = (N + 15) >> 4;
+  const int my_groups = (ncg - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+
+  // per-lane source pointers of a column group (rows clamp to N-1: those columns are never stored)
+  const int c_lo = (2 * g + odd) * 16, c_hi = (2 * g + (odd ^ 1)) * 16;
+  const uint8_t *p0 = Bt, *p1 = Bt;
+  auto point_at = [&](int gi) {
+    const int cg = blockIdx.x + gi * gridDim.x;
+    p0 = Bt + (long)min(cg * 16 + (j >> 1), N - 1) * ldb + c_lo + (long)w * 128;
+    p1 = Bt + (long)min(cg * 16 + 8 + (j >> 1), N - 1) * ldb + c_hi + (long)w * 128;
+  };
+  v4i x0[SKD_MAXS], x1[SKD_MAXS];
+  auto load_step = [&](int s) {
+    x0[s] = __builtin_nontemporal_load((const v4i*)(p0 + (long)s * SK_WAVES * 128));
+    x1[s] = __builtin_nontemporal_load((const v4i*)(p1 + (long)s * SK_WAVES * 128));
+  };
+  // the B stream starts before anything else touches memory
+  if (my_groups > 0) {
+    point_at(0);
+#pragma unroll
+    for (int s = 0; s < SKD_MAXS; ++s)
+      if (FULL || s < nmine) load_step(s);
+  }
+
+  // ---- A fragments: lane (m = j, g) holds A[m][128*(w + 8s) + 32g .. +31]
+  v8i af[SKD_MAXS];
+  {
+    const uint8_t* ap = A + (long)min(j, M - 1) * lda + g * 32 + (long)w * 128;
+#pragma unroll
+    for (int s = 0; s < SKD_MAXS; ++s)
+      if (FULL || s < nmine) {
+        const v4i* p = (const v4i*)(ap + (long)s * SK_WAVES * 128);
+        v4i lo = p[0], hi = p[1];
+        af[s] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      }
+  }
+  float alpha = 1.f;
+  if (scale_a) alpha = *scale_a;
+  if (scale_b) alpha = alpha * *scale_b;
+
+  int parity = 0;
+  for (int gi = 0; gi < my_groups; ++gi) {
+    const bool more = gi + 1 < my_groups;
+    if (more) point_at(gi + 1);
+    v4f acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < SKD_MAXS; ++s)
+      if (FULL || s < nmine) {
+        v8i bf;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          const int lo = odd ? x1[s][d] : x0[s][d];
+          const int send = odd ? x0[s][d] : x1[s][d];
+          bf[d] = lo;
+          bf[4 + d] = __builtin_amdgcn_mov_dpp(send, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]: lane ^ 1
+        }
+        if (more) load_step(s);  // the registers just consumed take this k-step of the next column group
+        acc = hx_mfma_16x16x128_e4m3(af[s], bf, acc);
+      }
+    // ---- sum the 8 wave partials: acc[r] is C[4g + r][column of lane j = cg*16 + (j>>1) + 8*(j&1)]
+    const int cg = blockIdx.x + gi * gridDim.x;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[parity][w][r][lane] = acc[r];
+    __syncthreads();
+    if (tid < 256) {
+      const int l2 = tid & 63, r = tid >> 6;
+      float sum = 0.f;
+#pragma unroll
+      for (int ww = 0; ww < SK_WAVES; ++ww) sum += red[parity][ww][r][l2];
+      const int j2 = l2 & 15;
+      const int m = 4 * (l2 >> 4) + r, n = cg * 16 + (j2 >> 1) + 8 * (j2 & 1);
+      if (m < M && n < N) C[(long)m * ldc + n] = (out_t)(sum * alpha);
+    }
+    parity ^= 1;  // the next group writes the other buffer, so one barrier per group is enough
+  }
+}
+
+// ------------------------------------------------------------------------------------------
 // general: 64x64 tile, 256 threads, 4x4 outputs per thread, fp32 FMAs on decoded e4m3.
 // ------------------------------------------------------------------------------------------
 template <int OUT>
@@ -372,8 +478,15 @@ static int launch_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int
     (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     const int ncg = (int)((N + 15) / 16);
     const int grid = ncg < cus ? ncg : cus;
-    hipLaunchKernelGGL(hx_fp8_gemm_skinny<OUT>, dim3(grid), dim3(512), 0, stream, (const uint8_t*)a, (const uint8_t*)b,
-                       (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb_n, (long)ldc, sa, sb);
+    if (K == 8192)
+      hipLaunchKernelGGL((hx_fp8_gemm_skinny_direct<OUT, true>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
+                         (const uint8_t*)b, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb_n, (long)ldc, sa, sb);
+    else if (K < 8192)
+      hipLaunchKernelGGL((hx_fp8_gemm_skinny_direct<OUT, false>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
+                         (const uint8_t*)b, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb_n, (long)ldc, sa, sb);
+    else
+      hipLaunchKernelGGL(hx_fp8_gemm_skinny<OUT>, dim3(grid), dim3(512), 0, stream, (const uint8_t*)a, (const uint8_t*)b,
+                         (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb_n, (long)ldc, sa, sb);
   } else {
     dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
     hipLaunchKernelGGL(hx_fp8_gemm_general<OUT>, grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)b, (out_t*)c,
