@@ -68,13 +68,16 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
   const uint8_t* gB = Bt + (n0 + w * 64) * ldb;  // wave-uniform
   const uint32_t lds0 = hx_lds_addr(&smem[0][0][0]) + (uint32_t)w * 64 * 128;
 
-  auto issue = [&](int kt, int stage) {
+  // DMA instruction i (0..15) of a k-tile: i < 8 -> A rows 64w + 8i .., else B rows 64w + 8(i-8) ..
+  auto issue_one = [&](int kt, int stage, int i) {
     const long kb = (long)kt * T256_BK;
     const uint32_t la = lds0 + (uint32_t)stage * 2 * T256_TILE_BYTES, lb = la + T256_TILE_BYTES;
+    if (i < 8) hx_g2l16_s(gA + (long)i * 8 * lda + kb, (i & 1) ? a_vo1 : a_vo0, la + i * 1024);
+    else hx_g2l16_s(gB + (long)(i - 8) * 8 * ldb + kb, (i & 1) ? b_vo1 : b_vo0, lb + (i - 8) * 1024);
+  };
+  auto issue = [&](int kt, int stage) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) hx_g2l16_s(gA + (long)j * 8 * lda + kb, (j & 1) ? a_vo1 : a_vo0, la + j * 1024);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) hx_g2l16_s(gB + (long)j * 8 * ldb + kb, (j & 1) ? b_vo1 : b_vo0, lb + j * 1024);
+    for (int i = 0; i < 16; ++i) issue_one(kt, stage, i);
   };
 
   // ---- MFMA operand addressing
@@ -91,74 +94,55 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // Fragments of one 64-byte k-step: 4 A blocks + 4 B blocks of 32 rows, 8 VGPRs each.
-  auto load_frags = [&](v8i(&af)[4], v8i(&bf)[4], int stage, int t) {
-    const uint8_t* sa = &smem[stage][0][0];
-    const uint8_t* sb = &smem[stage][1][0];
-    const int o0 = x ^ (t * 64), o1 = x ^ (t * 64 + 16);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      v4i lo = *(const v4i*)(sa + a_base + i * 4096 + o0);
-      v4i hi = *(const v4i*)(sa + a_base + i * 4096 + o1);
-      af[i] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      v4i lo = *(const v4i*)(sb + b_base + i * 4096 + o0);
-      v4i hi = *(const v4i*)(sb + b_base + i * 4096 + o1);
-      bf[i] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-    }
+  // fragment f (0..7) of the 64-byte k-step t of a stage: f < 4 -> A rows 32f.. of this wave, else B rows 32(f-4)..
+  auto load_frag = [&](v8i(&af)[4], v8i(&bf)[4], int stage, int t, int f) {
+    const uint8_t* base = (f < 4) ? &smem[stage][0][0] + a_base + f * 4096 : &smem[stage][1][0] + b_base + (f - 4) * 4096;
+    v4i lo = *(const v4i*)(base + (x ^ (t * 64)));
+    v4i hi = *(const v4i*)(base + (x ^ (t * 64 + 16)));
+    v8i v = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    if (f < 4) af[f] = v; else bf[f - 4] = v;
   };
-  auto mma = [&](v8i(&af)[4], v8i(&bf)[4]) {
+  // One k-step: 16 MFMAs on the current fragments.  Slotted between them, in program order pinned by scheduling
+  // barriers: the 8 fragment loads of the next k-step (under the first 8 MFMAs) and, when DMA is set, the 16 DMA
+  // instructions of a later k-tile, one per MFMA.  Spreading the DMA keeps the wave's in-order instruction stream
+  // from stalling behind a burst of 64 address-coalescing requests (4 waves x 16) right after the barrier.
+  auto kstep = [&](v8i(&ca)[4], v8i(&cb)[4], v8i(&na)[4], v8i(&nb)[4], int nstage, int nt, bool load_next, bool dma, int dkt,
+                   int dstage) {
 #pragma unroll
-    for (int bj = 0; bj < 4; ++bj)
-#pragma unroll
-      for (int bi = 0; bi < 4; ++bi) acc[bj][bi] = hx_mfma_32x32x64_e4m3(bf[bj], af[bi], acc[bj][bi]);
-  };
-  // two LDS reads slotted after each of the first 8 MFMAs: the 16 reads of the next k-step hide under
-  // the MFMAs and have all returned by the time the last MFMAs of the step issue
-  auto interleave = [&]() {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // 2 DS reads
+    for (int i = 0; i < 16; ++i) {
+      if (load_next && i < 8) load_frag(na, nb, nstage, nt, i);
+      acc[i >> 2][i & 3] = hx_mfma_32x32x64_e4m3(cb[i >> 2], ca[i & 3], acc[i >> 2][i & 3]);
+      if (dma) issue_one(dkt, dstage, i);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
   };
 
-  // Software pipeline.  k-tile kt lives in stage kt&1.  While the MFMAs of (kt, t=0) run, the fragments
-  // of (kt, t=1) are fetched; then one barrier says "tile kt+1 has landed in every wave's view and nobody
-  // reads stage kt&1 any more", the DMA of tile kt+2 is issued into the stage just freed, and the MFMAs
-  // of (kt, t=1) run while the fragments of (kt+1, t=0) are fetched.
+  // Software pipeline.  k-tile kt lives in stage kt&1.  While the MFMAs of (kt, t=0) run, the fragments of
+  // (kt, t=1) are fetched; then one barrier says "tile kt+1 has landed in every wave's view and nobody reads
+  // stage kt&1 any more"; under the MFMAs of (kt, t=1) the fragments of (kt+1, t=0) are fetched and the DMA of
+  // tile kt+2 goes out into the stage just freed.  (Past the end the DMA re-fetches the last tile into the free
+  // stage: harmless, and it keeps the loop free of branches around the accumulators.)
   const int nk = K / T256_BK;
   v8i fa0[4], fb0[4], fa1[4], fb1[4];
   issue(0, 0);
   if (nk > 1) issue(1, 1);
   if (nk > 1) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(16)); else HX_WAIT_VM0();
   __syncthreads();
-  load_frags(fa0, fb0, 0, 0);
+#pragma unroll
+  for (int f = 0; f < 8; ++f) load_frag(fa0, fb0, 0, 0, f);
   for (int kt = 0; kt < nk - 1; ++kt) {
     const int stage = kt & 1;
-    load_frags(fa1, fb1, stage, 1);
-    mma(fa0, fb0);
-    interleave();
-    __builtin_amdgcn_sched_barrier(0);
+    kstep(fa0, fb0, fa1, fb1, stage, 1, true, false, 0, 0);
     HX_WAIT_VM0();
     __syncthreads();
-    if (kt + 2 < nk) issue(kt + 2, stage);
-    load_frags(fa0, fb0, stage ^ 1, 0);
-    mma(fa1, fb1);
-    interleave();
-    __builtin_amdgcn_sched_barrier(0);
+    kstep(fa1, fb1, fa0, fb0, stage ^ 1, 0, true, true, min(kt + 2, nk - 1), stage);
   }
   {
     const int stage = (nk - 1) & 1;
-    load_frags(fa1, fb1, stage, 1);
-    mma(fa0, fb0);
-    interleave();
-    __builtin_amdgcn_sched_barrier(0);
-    mma(fa1, fb1);
+    kstep(fa0, fb0, fa1, fb1, stage, 1, true, false, 0, 0);
+    kstep(fa1, fb1, fa0, fb0, 0, 0, false, false, 0, 0);
   }
+  HX_WAIT_VM0();  // the trailing re-fetch must have landed before the workgroup's LDS is released
 
   // ---- epilogue: acc[bj][bi][4a+b] is C[m0 + wm*128 + bi*32 + lane%32][n0 + wn*128 + bj*32 + 8a + 4g + b]
   float alpha = 1.f;
