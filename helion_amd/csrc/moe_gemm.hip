@@ -157,15 +157,16 @@ __global__ __launch_bounds__(256) void hx_moe_tile256(const uint8_t* __restrict_
   for (int j = 0; j < 4; ++j) w_vo[j] = (uint32_t)(wk_l * N * 2 + ((wpos ^ (((2 * j + wk_l) & 7) << 1)) * 16));
   const uint32_t lds0 = hx_lds_addr(&smem[0][0][0]);
 
-  auto issue = [&](int kt, int stage) {
+  // DMA instruction i (0..15) of a k-tile: i < 8 -> gathered A rows 64w + 8i .., else W k-rows 16w + 2(i-8), +1
+  auto issue_one = [&](int kt, int stage, int i) {
     const uint32_t la = lds0 + (uint32_t)stage * 2 * MOE_TILE_BYTES + (uint32_t)w * 64 * 128;
     const uint32_t lw = lds0 + (uint32_t)stage * 2 * MOE_TILE_BYTES + MOE_TILE_BYTES + (uint32_t)w * 16 * 512;
-    const uint8_t* ak = A + (long)kt * 128;
+    if (i < 8) hx_g2l16_s(A + (long)kt * 128, a_vo[i], la + i * 1024);
+    else hx_g2l16_s(We + (long)kt * MOE_BK * N * 2 + (long)(2 * (i - 8)) * N * 2, w_vo[(i - 8) & 3], lw + (i - 8) * 1024);
+  };
+  auto issue = [&](int kt, int stage) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) hx_g2l16_s(ak, a_vo[j], la + j * 1024);
-    const uint8_t* wk = We + (long)kt * MOE_BK * N * 2;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) hx_g2l16_s(wk + (long)(2 * j) * N * 2, w_vo[j & 3], lw + j * 1024);
+    for (int i = 0; i < 16; ++i) issue_one(kt, stage, i);
   };
 
   // ---- operand addressing
@@ -194,65 +195,67 @@ __global__ __launch_bounds__(256) void hx_moe_tile256(const uint8_t* __restrict_
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // fragments of one k-step (16 k): 4 A blocks (one b128 each) and 4 W blocks (two transposing b64 each)
-  auto load_frags = [&](V8(&af)[4], V8(&wf)[4], int stage, int ks) {
-    const uint8_t* sa = &smem[stage][0][0];
-    const uint8_t* sw = &smem[stage][1][0];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) af[i] = *(const V8*)(sa + a_base + i * 4096 + (ax ^ (ks * 32)));
-#pragma unroll
-    for (int bj = 0; bj < 4; ++bj) {
+  // fragment f (0..7) of k-step ks (16 k) of a stage: f < 4 -> A rows 32f.. (one b128), else W columns 32(f-4)..
+  // (two transposing b64 reads)
+  auto load_frag = [&](V8(&af)[4], V8(&wf)[4], int stage, int ks, int f) {
+    if (f < 4) {
+      af[f] = *(const V8*)(&smem[stage][0][0] + a_base + f * 4096 + (ax ^ (ks * 32)));
+    } else {
+      const uint8_t* sw = &smem[stage][1][0];
       v4s part[2];
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
-        const int off = (w_off[half] ^ (bj * 64)) + ks * 8192;
+        const int off = (w_off[half] ^ ((f - 4) * 64)) + ks * 8192;
         part[half] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3)))*)(sw + off));
       }
       v8s both = (v8s){part[0][0], part[0][1], part[0][2], part[0][3], part[1][0], part[1][1], part[1][2], part[1][3]};
-      wf[bj] = __builtin_bit_cast(V8, both);
+      wf[f - 4] = __builtin_bit_cast(V8, both);
     }
   };
-  auto mma = [&](V8(&af)[4], V8(&wf)[4]) {
+  // One k-step: 16 MFMAs on the current fragments; pinned between them the 8 fragment loads of the next k-step and,
+  // when DMA is set, NDMA DMA instructions starting at number D0 (one per MFMA), as in the fp8 GEMM.
+  auto kstep = [&](V8(&ca)[4], V8(&cw)[4], V8(&na)[4], V8(&nw)[4], int nstage, int nks, bool load_next, bool dma, int dkt,
+                   int dstage, int d0) {
 #pragma unroll
-    for (int bj = 0; bj < 4; ++bj)
-#pragma unroll
-      for (int bi = 0; bi < 4; ++bi) acc[bj][bi] = Mfma16<BF>::run(wf[bj], af[bi], acc[bj][bi]);
-  };
-  auto interleave = [&]() {  // 12 LDS reads under the first 12 of 16 MFMAs
-#pragma unroll
-    for (int i = 0; i < 12; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    for (int i = 0; i < 16; ++i) {
+      if (load_next && i < 8) load_frag(na, nw, nstage, nks, i);
+      acc[i >> 2][i & 3] = Mfma16<BF>::run(cw[i >> 2], ca[i & 3], acc[i >> 2][i & 3]);
+      if (dma && (i & 1)) issue_one(dkt, dstage, d0 + (i >> 1));
+      __builtin_amdgcn_sched_barrier(0);
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
   };
 
   // software pipeline, as in the fp8 GEMM: k-tile kt in stage kt&1, four k-steps per tile, fragments double
-  // buffered; the one barrier per tile sits before the last k-step's MFMAs.
+  // buffered; the one barrier per tile sits before the last k-step's MFMAs; the 16 DMA instructions of tile kt+2 go
+  // out under the MFMAs of (kt, ks=3) and (kt+1, ks=0), one every other MFMA.
   const int nk = K / MOE_BK;
   V8 fa0[4], fw0[4], fa1[4], fw1[4];
   issue(0, 0);
   if (nk > 1) issue(1, 1);
   if (nk > 1) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(16)); else HX_WAIT_VM0();
   __syncthreads();
-  load_frags(fa0, fw0, 0, 0);
+#pragma unroll
+  for (int f = 0; f < 8; ++f) load_frag(fa0, fw0, 0, 0, f);
   for (int kt = 0; kt < nk - 1; ++kt) {
     const int stage = kt & 1;
-    load_frags(fa1, fw1, stage, 1); mma(fa0, fw0); interleave(); __builtin_amdgcn_sched_barrier(0);
-    load_frags(fa0, fw0, stage, 2); mma(fa1, fw1); interleave(); __builtin_amdgcn_sched_barrier(0);
-    load_frags(fa1, fw1, stage, 3); mma(fa0, fw0); interleave(); __builtin_amdgcn_sched_barrier(0);
+    // (kt, ks=0): second half of tile kt+1's DMA (its first half went out under (kt-1, ks=3)); stage^1 is free
+    // since the last barrier, and both halves are complete at this iteration's barrier
+    kstep(fa0, fw0, fa1, fw1, stage, 1, true, kt > 0, min(kt + 1, nk - 1), stage ^ 1, 8);
+    kstep(fa1, fw1, fa0, fw0, stage, 2, true, false, 0, 0, 0);
+    kstep(fa0, fw0, fa1, fw1, stage, 3, true, false, 0, 0, 0);
     HX_WAIT_VM0();
     __syncthreads();
-    if (kt + 2 < nk) issue(kt + 2, stage);
-    load_frags(fa0, fw0, stage ^ 1, 0); mma(fa1, fw1); interleave(); __builtin_amdgcn_sched_barrier(0);
+    // (kt, ks=3): first half of tile kt+2's DMA into the stage just freed
+    kstep(fa1, fw1, fa0, fw0, stage ^ 1, 0, true, true, min(kt + 2, nk - 1), stage, 0);
   }
   {
     const int stage = (nk - 1) & 1;
-    load_frags(fa1, fw1, stage, 1); mma(fa0, fw0); interleave(); __builtin_amdgcn_sched_barrier(0);
-    load_frags(fa0, fw0, stage, 2); mma(fa1, fw1); interleave(); __builtin_amdgcn_sched_barrier(0);
-    load_frags(fa1, fw1, stage, 3); mma(fa0, fw0); interleave(); __builtin_amdgcn_sched_barrier(0);
-    mma(fa1, fw1);
+    kstep(fa0, fw0, fa1, fw1, stage, 1, true, nk > 1, nk - 1, stage ^ 1, 8);
+    kstep(fa1, fw1, fa0, fw0, stage, 2, true, false, 0, 0, 0);
+    kstep(fa0, fw0, fa1, fw1, stage, 3, true, false, 0, 0, 0);
+    kstep(fa1, fw1, fa0, fw0, 0, 0, false, false, 0, 0, 0);
   }
+  HX_WAIT_VM0();  // trailing re-fetches must land before the workgroup's LDS is released
 
   // ---- epilogue: acc[bj][bi][4a+b] is C[idx[row_start + wm*128 + bi*32 + lane%32]][n0 + wn*128 + bj*32 + 8a + 4g + b]
 #pragma unroll
