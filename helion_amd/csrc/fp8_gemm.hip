@@ -26,10 +26,12 @@
 #define T256_BK 128
 #define T256_TILE_BYTES (256 * 128)
 
-template <int OUT>
+// EDGE: M and/or N are not multiples of 256.  Rows past the end are clamped to the last row on load (their
+// products land in accumulators that are never stored) and the stores are guarded.
+template <int OUT, bool EDGE>
 __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __restrict__ A, const uint8_t* __restrict__ Bt,
-                                                          typename OutT<OUT>::T* __restrict__ C, int K, long lda, long ldb,
-                                                          long ldc, const float* __restrict__ scale_a,
+                                                          typename OutT<OUT>::T* __restrict__ C, int M, int N, int K, long lda,
+                                                          long ldb, long ldc, const float* __restrict__ scale_a,
                                                           const float* __restrict__ scale_b, int tiles_m, int tiles_n) {
   typedef typename OutT<OUT>::T out_t;
   // [stage][A|B][256 rows x 128 B]
@@ -72,8 +74,19 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
   auto issue_one = [&](int kt, int stage, int i) {
     const long kb = (long)kt * T256_BK;
     const uint32_t la = lds0 + (uint32_t)stage * 2 * T256_TILE_BYTES, lb = la + T256_TILE_BYTES;
-    if (i < 8) hx_g2l16_s(gA + (long)i * 8 * lda + kb, (i & 1) ? a_vo1 : a_vo0, la + i * 1024);
-    else hx_g2l16_s(gB + (long)(i - 8) * 8 * ldb + kb, (i & 1) ? b_vo1 : b_vo0, lb + (i - 8) * 1024);
+    if (!EDGE) {
+      if (i < 8) hx_g2l16_s(gA + (long)i * 8 * lda + kb, (i & 1) ? a_vo1 : a_vo0, la + i * 1024);
+      else hx_g2l16_s(gB + (long)(i - 8) * 8 * ldb + kb, (i & 1) ? b_vo1 : b_vo0, lb + (i - 8) * 1024);
+    } else {  // per-lane clamped row; the whole matrix is below 4 GB (checked by the host), so the offset fits 32 bits
+      const int swz = (((i & 1) ? 4 : 0) + (lrow >> 1)) & 7;
+      if (i < 8) {
+        const uint32_t row = (uint32_t)min((int)m0 + w * 64 + i * 8 + lrow, M - 1);
+        hx_g2l16_s(A + kb, row * (uint32_t)lda + (uint32_t)((lpos ^ swz) * 16), la + i * 1024);
+      } else {
+        const uint32_t row = (uint32_t)min((int)n0 + w * 64 + (i - 8) * 8 + lrow, N - 1);
+        hx_g2l16_s(Bt + kb, row * (uint32_t)ldb + (uint32_t)((lpos ^ swz) * 16), lb + (i - 8) * 1024);
+      }
+    }
   };
   auto issue = [&](int kt, int stage) {
 #pragma unroll
@@ -150,7 +163,9 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
   if (scale_b) alpha = alpha * *scale_b;
 #pragma unroll
   for (int bi = 0; bi < 4; ++bi) {
-    out_t* crow = C + (m0 + wm * 128 + bi * 32 + r31) * ldc + n0 + wn * 128 + 4 * g;
+    const long m = m0 + wm * 128 + bi * 32 + r31;
+    out_t* crow = C + m * ldc + n0 + wn * 128 + 4 * g;
+    if (EDGE && m >= M) continue;
 #pragma unroll
     for (int bj = 0; bj < 4; ++bj)
 #pragma unroll
@@ -159,8 +174,36 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
         ov4 o;
 #pragma unroll
         for (int b = 0; b < 4; ++b) o[b] = (out_t)(acc[bj][bi][4 * a + b] * alpha);
-        *(ov4*)(crow + bj * 32 + 8 * a) = o;
+        if (!EDGE) {
+          *(ov4*)(crow + bj * 32 + 8 * a) = o;
+        } else {
+          const long n = n0 + wn * 128 + 4 * g + bj * 32 + 8 * a;
+          if (n + 4 <= N && ((uintptr_t)(crow + bj * 32 + 8 * a) & (sizeof(ov4) - 1)) == 0) *(ov4*)(crow + bj * 32 + 8 * a) = o;
+          else
+            for (int b = 0; b < 4; ++b)
+              if (n + b < N) crow[bj * 32 + 8 * a + b] = o[b];
+        }
       }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// byte transpose: src[K][N] (row stride lds_, N contiguous) -> dst[N][K] contiguous.  Turns a row-major B into
+// the K-contiguous layout the MFMA kernels read; 64x64 tiles through LDS.
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void hx_transpose_u8(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, int K, int N,
+                                                      long src_ld) {
+  __shared__ uint8_t t[64][64 + 4];
+  const int k0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int r = ty; r < 64; r += 4) {
+    const int k = k0 + r, n = n0 + tx;
+    t[r][tx] = (k < K && n < N) ? src[(long)k * src_ld + n] : (uint8_t)0;
+  }
+  __syncthreads();
+  for (int r = ty; r < 64; r += 4) {
+    const int n = n0 + r, k = k0 + tx;
+    if (n < N && k < K) dst[(long)n * K + k] = t[tx][r];
   }
 }
 
@@ -436,27 +479,39 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_general(const uint8_t* __rest
 // ------------------------------------------------------------------------------------------
 static inline bool aligned(const void* p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
+// 0 general, 1 tile256, 2 skinny, 3 tile256 with edge tiles (M or N not a multiple of 256)
+static int gemm_path_kmajor(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, const void* a, const void* b,
+                            const void* c) {
+  const bool ok = (lda % 16 == 0) && (ldb % 16 == 0) && (K % 128 == 0) && aligned(a, 16) && aligned(b, 16) && K >= 128;
+  if (!ok) return 0;
+  if (M <= 16 && lda >= K && ldb >= K) return 2;
+  if (lda >= (1LL << 27) || ldb >= (1LL << 27)) return 0;
+  if ((M % 256 == 0) && (N % 256 == 0) && (ldc % 4 == 0) && aligned(c, 16)) return 1;
+  if (M * lda < (1LL << 32) && N * ldb < (1LL << 32)) return 3;
+  return 0;
+}
+
 extern "C" int hx_fp8_gemm_path(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
                                 const void* a, const void* b, const void* c) {
-  const bool kmajor = (ldb_k == 1) && (lda % 16 == 0) && (ldb_n % 16 == 0) && (K % 128 == 0) && aligned(a, 16) &&
-                      aligned(b, 16) && K >= 128;
-  if (kmajor && M <= 16 && lda >= K && ldb_n >= K) return 2;
-  if (kmajor && (M % 256 == 0) && (N % 256 == 0) && (ldc % 4 == 0) && aligned(c, 16) &&
-      lda < (1LL << 27) && ldb_n < (1LL << 27))
-    return 1;
+  if (ldb_k == 1) return gemm_path_kmajor(M, N, K, lda, ldb_n, ldc, a, b, c);
   return 0;
 }
 
 template <int OUT>
-static int launch_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k,
-                           int64_t ldb_n, int64_t ldc, const float* sa, const float* sb, hipStream_t stream) {
+static void launch_kmajor(int path, const void* a, const void* bt, void* c, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                          int64_t ldc, const float* sa, const float* sb, hipStream_t stream) {
   typedef typename OutT<OUT>::T out_t;
-  const int path = hx_fp8_gemm_path(M, N, K, lda, ldb_k, ldb_n, ldc, a, b, c);
-  if (path == 1) {
-    const int tiles_m = (int)(M / 256), tiles_n = (int)(N / 256);
-    hipLaunchKernelGGL(hx_fp8_gemm_tile256<OUT>, dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
-                       (const uint8_t*)b, (out_t*)c, (int)K, (long)lda, (long)ldb_n, (long)ldc, sa, sb, tiles_m, tiles_n);
-  } else if (path == 2) {
+  if (path == 1 || path == 3) {
+    const int tiles_m = (int)((M + 255) / 256), tiles_n = (int)((N + 255) / 256);
+    if (path == 1)
+      hipLaunchKernelGGL((hx_fp8_gemm_tile256<OUT, false>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
+                         (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m,
+                         tiles_n);
+    else
+      hipLaunchKernelGGL((hx_fp8_gemm_tile256<OUT, true>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
+                         (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m,
+                         tiles_n);
+  } else {  // path == 2
     int dev = 0, cus = 256;
     (void)hipGetDevice(&dev);
     (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
@@ -464,17 +519,38 @@ static int launch_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int
     const int grid = ncg < cus ? ncg : cus;
     if (K == 8192)
       hipLaunchKernelGGL((hx_fp8_gemm_skinny_direct<OUT, true>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
-                         (const uint8_t*)b, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb_n, (long)ldc, sa, sb);
+                         (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb);
     else if (K < 8192)
       hipLaunchKernelGGL((hx_fp8_gemm_skinny_direct<OUT, false>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
-                         (const uint8_t*)b, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb_n, (long)ldc, sa, sb);
+                         (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb);
     else
-      hipLaunchKernelGGL(hx_fp8_gemm_skinny<OUT>, dim3(grid), dim3(512), 0, stream, (const uint8_t*)a, (const uint8_t*)b,
-                         (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb_n, (long)ldc, sa, sb);
+      hipLaunchKernelGGL(hx_fp8_gemm_skinny<OUT>, dim3(grid), dim3(512), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
+                         (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb);
+  }
+}
+
+template <int OUT>
+static int launch_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k,
+                           int64_t ldb_n, int64_t ldc, const float* sa, const float* sb, void* ws, size_t ws_bytes,
+                           hipStream_t stream) {
+  typedef typename OutT<OUT>::T out_t;
+  int path = hx_fp8_gemm_path(M, N, K, lda, ldb_k, ldb_n, ldc, a, b, c);
+  if (path != 0) {
+    launch_kmajor<OUT>(path, a, b, c, M, N, K, lda, ldb_n, ldc, sa, sb, stream);
   } else {
-    dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
-    hipLaunchKernelGGL(hx_fp8_gemm_general<OUT>, grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)b, (out_t*)c,
-                       (int)M, (int)N, (int)K, (long)lda, (long)ldb_k, (long)ldb_n, (long)ldc, sa, sb);
+    // row-major B with a workspace: transpose it once into K-contiguous form, then take a fast path
+    int tpath = 0;
+    if (ldb_n == 1 && ldb_k >= N && ws && ws_bytes >= (size_t)(N * K) && aligned(ws, 16))
+      tpath = gemm_path_kmajor(M, N, K, lda, K, ldc, a, ws, c);
+    if (tpath != 0) {
+      dim3 tg((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64));
+      hipLaunchKernelGGL(hx_transpose_u8, tg, dim3(256), 0, stream, (const uint8_t*)b, (uint8_t*)ws, (int)K, (int)N, (long)ldb_k);
+      launch_kmajor<OUT>(tpath, a, ws, c, M, N, K, lda, K, ldc, sa, sb, stream);
+    } else {
+      dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
+      hipLaunchKernelGGL(hx_fp8_gemm_general<OUT>, grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)b, (out_t*)c,
+                         (int)M, (int)N, (int)K, (long)lda, (long)ldb_k, (long)ldb_n, (long)ldc, sa, sb);
+    }
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
@@ -484,11 +560,15 @@ static int launch_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int
   return 0;
 }
 
-extern "C" size_t hx_fp8_gemm_workspace_bytes(int64_t, int64_t, int64_t) { return 0; }
+extern "C" size_t hx_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t ldb_k, int64_t ldb_n) {
+  // only a row-major B (N contiguous) that could take a fast path after a transpose needs scratch: N*K bytes
+  if (M <= 0 || N <= 0 || K <= 0 || ldb_k == 1 || ldb_n != 1 || K % 128 != 0) return 0;
+  return (size_t)(N * K);
+}
 
 extern "C" int hx_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k,
                            int64_t ldb_n, int64_t ldc, const float* scale_a, const float* scale_b, int out_dtype,
-                           void* /*workspace*/, size_t /*workspace_bytes*/, void* stream) {
+                           void* workspace, size_t workspace_bytes, void* stream) {
   if (M < 0 || N < 0 || K < 0) {
     hx_set_error("hx_fp8_gemm: negative size M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
     return HX_ERR_BAD_ARG;
@@ -509,9 +589,9 @@ extern "C" int hx_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int
   }
   hipStream_t s = (hipStream_t)stream;
   switch (out_dtype) {
-    case HX_F16: return launch_fp8_gemm<HX_F16>(a, b, c, M, N, K, lda, ldb_k, ldb_n, ldc, scale_a, scale_b, s);
-    case HX_BF16: return launch_fp8_gemm<HX_BF16>(a, b, c, M, N, K, lda, ldb_k, ldb_n, ldc, scale_a, scale_b, s);
-    case HX_F32: return launch_fp8_gemm<HX_F32>(a, b, c, M, N, K, lda, ldb_k, ldb_n, ldc, scale_a, scale_b, s);
+    case HX_F16: return launch_fp8_gemm<HX_F16>(a, b, c, M, N, K, lda, ldb_k, ldb_n, ldc, scale_a, scale_b, workspace, workspace_bytes, s);
+    case HX_BF16: return launch_fp8_gemm<HX_BF16>(a, b, c, M, N, K, lda, ldb_k, ldb_n, ldc, scale_a, scale_b, workspace, workspace_bytes, s);
+    case HX_F32: return launch_fp8_gemm<HX_F32>(a, b, c, M, N, K, lda, ldb_k, ldb_n, ldc, scale_a, scale_b, workspace, workspace_bytes, s);
     default:
       hx_set_error("hx_fp8_gemm: unknown out_dtype tag %d", out_dtype);
       return HX_ERR_BAD_ARG;

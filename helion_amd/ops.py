@@ -51,10 +51,12 @@ def fp8_gemm_op(x: torch.Tensor, y: torch.Tensor, scale_a: torch.Tensor | None, 
     ldb_k = y.stride(0) if k > 1 else 1
     ldb_n = y.stride(1) if n > 1 else max(k, 1)
     lib = _lib.load()
+    ws_bytes = lib.hx_fp8_gemm_workspace_bytes(m, n, k, ldb_k, ldb_n)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
     rc = lib.hx_fp8_gemm(x.data_ptr(), y.data_ptr(), out.data_ptr(), m, n, k, lda, ldb_k, ldb_n, n,
                          scale_a.data_ptr() if scale_a is not None else None,
                          scale_b.data_ptr() if scale_b is not None else None,
-                         _DT[out_dtype], None, 0, _stream_ptr(x.device))
+                         _DT[out_dtype], ws.data_ptr() if ws is not None else None, ws_bytes, _stream_ptr(x.device))
     _lib.check(rc, "hx_fp8_gemm")
     return out
 

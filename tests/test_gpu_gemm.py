@@ -25,7 +25,8 @@ def _path(m, n, k):
 @pytest.mark.parametrize("m,n,k,path", [
     (256, 256, 256, 1), (512, 512, 512, 1), (1024, 1024, 1024, 1), (256, 768, 128, 1), (768, 256, 1152, 1),
     (16, 512, 1024, 2), (1, 16, 128, 2), (5, 48, 256, 2), (16, 1000, 384, 2), (9, 33, 8192 + 128, 2), (16, 64, 16384, 2),
-    (100, 70, 50, 0), (17, 256, 256, 0), (256, 256, 200, 0), (3, 5, 7, 0), (64, 64, 0, 0),
+    (1000, 1000, 1024, 3), (300, 200, 256, 3), (257, 255, 128, 3), (17, 256, 256, 3), (255, 1, 128, 3),
+    (100, 70, 50, 0), (256, 256, 200, 0), (3, 5, 7, 0), (64, 64, 0, 0),
 ])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_shapes_vs_oracle(m, n, k, path, out_dtype):
@@ -35,6 +36,21 @@ def test_shapes_vs_oracle(m, n, k, path, out_dtype):
     assert out.dtype == out_dtype and out.shape == (m, n)
     ref = orc.fp8_gemm(a, b, sa, sb, out_dtype)
     assert rel_err(out, ref) <= (1e-2 if out_dtype != torch.float32 else 1e-4)
+
+
+@pytest.mark.parametrize("m,k,n", [(256, 384, 512), (300, 256, 200), (16, 1024, 512), (64, 100, 48)])
+def test_row_major_b_goes_through_the_transpose_workspace(m, k, n):
+    g = torch.Generator().manual_seed(m + n)
+    x = torch.randn(m, k, generator=g).to(E4M3); y = torch.randn(k, n, generator=g).to(E4M3)  # y row-major
+    lib = _lib.load()
+    want = n * k if k % 128 == 0 else 0
+    assert lib.hx_fp8_gemm_workspace_bytes(m, n, k, n, 1) == want
+    out = hx.fp8_gemm(x.to(DEV), y.to(DEV), out_dtype=torch.float32)
+    assert rel_err(out, orc.fp8_gemm(x, y, out_dtype=torch.float32)) <= 1e-4
+    # a strided (non-compact) row-major view works too
+    ybig = torch.randn(k, n + 16, generator=g).to(E4M3)
+    out2 = hx.fp8_gemm(x.to(DEV), ybig.to(DEV)[:, :n], out_dtype=torch.float32)
+    assert rel_err(out2, orc.fp8_gemm(x, ybig[:, :n].contiguous(), out_dtype=torch.float32)) <= 1e-4
 
 
 def test_reference_call_form_and_defaults():
