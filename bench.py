@@ -47,14 +47,14 @@ def _time_launches(fn, steps, warmup):
 
 
 def _traffic(name):
-    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE), if a summary of such
-    a run has been recorded under profiles/."""
-    f = ROOT / "profiles" / "traffic.json"
+    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE, scaled by a copy of known
+    size), read from the `traffic_bytes <name> <bytes>` lines of the summary recorded under profiles/."""
+    f = ROOT / "profiles" / "hbm_traffic_fetch_write_size.txt"
     if f.exists():
-        try:
-            return json.loads(f.read_text()).get(name)
-        except Exception:
-            return None
+        for line in f.read_text().splitlines():
+            parts = line.split()
+            if len(parts) == 3 and parts[0] == "traffic_bytes" and parts[1] == name:
+                return int(parts[2])
     return None
 
 
@@ -99,7 +99,7 @@ def bench_c3(steps, warmup):
         "workload": "C3 decode fp8_gemm M16 N28672 K8192 bf16 out, 6 rotating weight buffers (HBM-cold)",
         "ms_per_launch": ms, "value": gbs, "unit": "GB/s",
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
-                     "traffic": _traffic("fp8_gemm_skinny_c3"), "kernel": "hx_fp8_gemm_skinny", "avg_launch_ms": ms,
+                     "traffic": _traffic("fp8_gemm_skinny_c3"), "kernel": "hx_fp8_gemm_skinny_direct", "avg_launch_ms": ms,
                      "algorithmic_bytes_per_launch": nbytes},
     }
 
