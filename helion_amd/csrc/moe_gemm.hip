@@ -78,11 +78,17 @@ __global__ void hx_moe_zero_rows(T16* __restrict__ C, long ldc, int T, int N, co
 // tile256: 256 gathered rows x 256 columns x 64 k per step; 4 waves (2x2) of 128x128; 32x32x16 MFMA.
 //   A tile  [256 rows][128 B]  : same chunk-swizzled layout as the fp8 GEMM; the DMA gathers rows
 //                                through idx, so the gather costs nothing extra.
-//   W tile  [64 k][512 B]      : row = k, 32 chunks of 8 columns; chunk stored at pos = chunk ^ ((k&7)<<1).
+//   W tile  [64 k][512 B]      : row = k, 32 chunks of 8 columns; chunk stored at pos = chunk ^ (moe_wswz(k)<<1).
 //                                The MFMA wants 8 consecutive k per lane for one column, W has the
 //                                columns contiguous: ds_read_b64_tr_b16 transposes 4(k) x 16(n) blocks
 //                                on the way out of LDS (two reads per operand).
 // ------------------------------------------------------------------------------------------
+// Swizzle of a W-tile row, in units of 32 bytes (a pair of chunks).  One transposing read has the 32 lanes
+// that the LDS serves together fetch 4 consecutive k rows x two adjacent 32-byte column groups; rows are 512 B
+// apart (the same banks), so the 8 (row, group) combinations must land in 8 different 32-byte bank groups:
+// k&3 goes to bits 2:1 and bit 2 of k to bit 0, which the column-group bit then flips.
+__device__ __forceinline__ int moe_wswz(int k) { return ((k & 3) << 1) | ((k >> 2) & 1); }
+
 template <bool BF>
 struct Mfma16;
 template <>
@@ -149,12 +155,12 @@ __global__ __launch_bounds__(256) void hx_moe_tile256(const uint8_t* __restrict_
     a_vo[j] = (uint32_t)r * (uint32_t)(K * 2) + (uint32_t)((lpos ^ swz) * 16);
   }
   // ---- W DMA: wave w owns k rows [16w, 16w+16), 8 instructions of 2 rows x 512 B.
-  // row k = 16w + 2j + (lane>>5); chunk = (lane&31) ^ ((k&7)<<1); (k&7) = (2j + (lane>>5)) & 7
+  // row k = 16w + 2j + (lane>>5); chunk = (lane&31) ^ (moe_wswz(k)<<1); k&7 = (2j + (lane>>5)) & 7
   const uint8_t* We = W + (long)mt.expert * K * N * 2 + n0 * 2 + (long)(w * 16) * N * 2;  // wave-uniform
   const int wk_l = lane >> 5, wpos = lane & 31;
   uint32_t w_vo[4];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) w_vo[j] = (uint32_t)(wk_l * N * 2 + ((wpos ^ (((2 * j + wk_l) & 7) << 1)) * 16));
+  for (int j = 0; j < 4; ++j) w_vo[j] = (uint32_t)(wk_l * N * 2 + ((wpos ^ (moe_wswz(2 * j + wk_l) << 1)) * 16));
   const uint32_t lds0 = hx_lds_addr(&smem[0][0][0]);
 
   // DMA instruction i (0..15) of a k-tile: i < 8 -> gathered A rows 64w + 8i .., else W k-rows 16w + 2(i-8), +1
@@ -184,7 +190,7 @@ __global__ __launch_bounds__(256) void hx_moe_tile256(const uint8_t* __restrict_
 #pragma unroll
   for (int half = 0; half < 2; ++half) {
     const int k = tk + 4 * half;
-    w_off[half] = k * 512 + (((tn_ >> 3) ^ ((k & 7) << 1)) * 16) + (tn_ & 7) * 2;
+    w_off[half] = k * 512 + (((tn_ >> 3) ^ (moe_wswz(k) << 1)) * 16) + (tn_ & 7) * 2;
   }
 
   v16f acc[4][4];
