@@ -38,6 +38,18 @@ _SIGNATURES = {
          _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int, _c.c_void_p, _c.c_size_t, _c.c_void_p],
     ),
     "hx_moe_workspace_bytes": (_c.c_size_t, [_c.c_int64, _c.c_int64]),
+    "hx_moe_routing": (
+        _c.c_int,
+        [_c.c_void_p, _c.c_int, _c.c_int64, _c.c_int64, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,
+         _c.c_size_t, _c.c_void_p],
+    ),
+    "hx_moe_routing_workspace_bytes": (_c.c_size_t, [_c.c_int64, _c.c_int64]),
+    "hx_moe_topk_matmul": (
+        _c.c_int,
+        [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64,
+         _c.c_int64, _c.c_int, _c.c_void_p, _c.c_size_t, _c.c_void_p],
+    ),
+    "hx_moe_topk_workspace_bytes": (_c.c_size_t, [_c.c_int64, _c.c_int64, _c.c_int64]),
 }
 
 

@@ -113,7 +113,7 @@ template <bool BF>
 __global__ __launch_bounds__(256) void hx_moe_tile256(const uint8_t* __restrict__ A, const uint8_t* __restrict__ W,
                                                      typename Mfma16<BF>::T* __restrict__ C, const int* __restrict__ num_tiles,
                                                      const MoeTile* __restrict__ table, const int32_t* __restrict__ idx, int T, int K,
-                                                     int N, int max_tiles, int tiles_n) {
+                                                     int N, int max_tiles, int tiles_n, int a_div) {
   typedef typename Mfma16<BF>::T out_t;
   typedef typename Mfma16<BF>::V8 V8;
   // [stage][A|W][32 KB]
@@ -152,7 +152,8 @@ __global__ __launch_bounds__(256) void hx_moe_tile256(const uint8_t* __restrict_
     int r = idx[mt.row_start + lr];
     r = (r >= 0 && r < T) ? r : 0;
     const int swz = ((j & 1) ? 4 + (lrow >> 1) : (lrow >> 1)) & 7;
-    a_vo[j] = (uint32_t)r * (uint32_t)(K * 2) + (uint32_t)((lpos ^ swz) * 16);
+    // a_div > 1: C row r is the product of A row r / a_div (top-k routing without a replicated A)
+    a_vo[j] = (uint32_t)(r / a_div) * (uint32_t)(K * 2) + (uint32_t)((lpos ^ swz) * 16);
   }
   // ---- W DMA: wave w owns k rows [16w, 16w+16), 8 instructions of 2 rows x 512 B.
   // row k = 16w + 2j + (lane>>5); chunk = (lane&31) ^ (moe_wswz(k)<<1); k&7 = (2j + (lane>>5)) & 7
@@ -292,7 +293,7 @@ __global__ __launch_bounds__(256) void hx_moe_tile256(const uint8_t* __restrict_
 template <typename T16>
 __global__ __launch_bounds__(256) void hx_moe_general(const T16* __restrict__ A, const T16* __restrict__ W, T16* __restrict__ C,
                                                      const int* __restrict__ num_tiles, const MoeTile* __restrict__ table,
-                                                     const int32_t* __restrict__ idx, int T, int K, int N) {
+                                                     const int32_t* __restrict__ idx, int T, int K, int N, int a_div) {
   const int tm = blockIdx.x;
   if (tm >= *num_tiles) return;
   const MoeTile mt = table[tm];
@@ -313,7 +314,7 @@ __global__ __launch_bounds__(256) void hx_moe_general(const T16* __restrict__ A,
       const int kk = e & 15, r = e >> 4;
       const int row = srow[r];
       const long k = k0 + kk;
-      sa[kk][r] = (row >= 0 && k < K) ? (float)A[(long)row * K + k] : 0.f;
+      sa[kk][r] = (row >= 0 && k < K) ? (float)A[(long)(row / a_div) * K + k] : 0.f;
     }
     for (int e = tid; e < 64 * 16; e += 256) {
       const int c = e & 63, kk = e >> 6;
@@ -356,9 +357,9 @@ extern "C" size_t hx_moe_workspace_bytes(int64_t T, int64_t E) {
 
 template <bool BF>
 static int launch_moe(const void* A, const void* W, void* C, const int32_t* counts, const int32_t* offsets, const int32_t* idx,
-                      int64_t T, int64_t K, int64_t N, int64_t E, void* ws, hipStream_t s) {
+                      int64_t T, int64_t K, int64_t N, int64_t E, int64_t a_div, void* ws, hipStream_t s) {
   typedef typename Mfma16<BF>::T T16;
-  const bool fast = (K % MOE_BK == 0) && (N % MOE_BN == 0) && K >= MOE_BK && (T * K * 2 < (1LL << 32)) && (N * 4 < (1LL << 31)) && (((uintptr_t)A | (uintptr_t)W | (uintptr_t)C) & 15) == 0;
+  const bool fast = (K % MOE_BK == 0) && (N % MOE_BN == 0) && K >= MOE_BK && (((T + a_div - 1) / a_div) * K * 2 < (1LL << 32)) && (N * 4 < (1LL << 31)) && (((uintptr_t)A | (uintptr_t)W | (uintptr_t)C) & 15) == 0;
   const int bm = fast ? MOE_BM : 64;
   const int max_tiles = (int)moe_max_tiles(T, E, bm);
   int* num_tiles = (int*)ws;
@@ -375,11 +376,11 @@ static int launch_moe(const void* A, const void* W, void* C, const int32_t* coun
   if (fast) {
     const int tiles_n = (int)(N / MOE_BN);
     hipLaunchKernelGGL(hx_moe_tile256<BF>, dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W, (T16*)C,
-                       (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, max_tiles, tiles_n);
+                       (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, max_tiles, tiles_n, (int)a_div);
   } else {
     dim3 grid((unsigned)max_tiles, (unsigned)((N + 63) / 64));
     hipLaunchKernelGGL(hx_moe_general<T16>, grid, dim3(256), 0, s, (const T16*)A, (const T16*)W, (T16*)C, (const int*)num_tiles,
-                       (const MoeTile*)table, idx, (int)T, (int)K, (int)N);
+                       (const MoeTile*)table, idx, (int)T, (int)K, (int)N, (int)a_div);
   }
   hipLaunchKernelGGL(hx_moe_zero_rows<T16>, dim3((unsigned)T), dim3(256), 0, s, (T16*)C, (long)N, (int)T, (int)N, (const uint8_t*)flags);
   hipError_t e = hipGetLastError();
@@ -416,6 +417,68 @@ extern "C" int hx_moe_grouped_gemm(const void* A, const void* W, void* C, const 
     return HX_ERR_WORKSPACE;
   }
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == HX_BF16) return launch_moe<true>(A, W, C, counts, offsets, idx, T, K, N, E, workspace, s);
-  return launch_moe<false>(A, W, C, counts, offsets, idx, T, K, N, E, workspace, s);
+  if (dtype == HX_BF16) return launch_moe<true>(A, W, C, counts, offsets, idx, T, K, N, E, 1, workspace, s);
+  return launch_moe<false>(A, W, C, counts, offsets, idx, T, K, N, E, 1, workspace, s);
+}
+
+// ------------------------------------------------------------------------------------------
+// top-k entry: routing on the device + grouped GEMM that gathers A rows as (sorted row / top_k)
+// ------------------------------------------------------------------------------------------
+extern "C" int hx_moe_routing(const void* expert_ids, int ids_are_int64, int64_t T, int64_t E, int32_t* counts, int32_t* offsets,
+                              int32_t* idx, int32_t* max_count, void* workspace, size_t workspace_bytes, void* stream);
+extern "C" size_t hx_moe_routing_workspace_bytes(int64_t T, int64_t E);
+
+static inline size_t moe_topk_tables_bytes(int64_t T, int64_t E) {
+  // counts[E] | offsets[E+1] | max_count | idx[T] | scratch of the routing kernels
+  size_t b = (size_t)(2 * E + 2) * 4 + (size_t)T * 4 + hx_moe_routing_workspace_bytes(T, E);
+  return (b + 255) & ~(size_t)255;
+}
+
+extern "C" size_t hx_moe_topk_workspace_bytes(int64_t T_tok, int64_t top_k, int64_t E) {
+  if (T_tok < 0 || top_k < 1 || E < 0) return 0;
+  const int64_t T = T_tok * top_k;
+  return moe_topk_tables_bytes(T, E) + hx_moe_workspace_bytes(T, E);
+}
+
+extern "C" int hx_moe_topk_matmul(const void* A_tok, const void* W, void* C, const void* expert_ids, int ids_are_int64,
+                                  int64_t T_tok, int64_t top_k, int64_t K, int64_t N, int64_t E, int dtype, void* workspace,
+                                  size_t workspace_bytes, void* stream) {
+  if (T_tok < 0 || K < 0 || N < 0 || E < 0 || top_k < 1) {
+    hx_set_error("hx_moe_topk_matmul: negative size or top_k < 1");
+    return HX_ERR_BAD_ARG;
+  }
+  if (dtype != HX_BF16 && dtype != HX_F16) {
+    hx_set_error("hx_moe_topk_matmul: dtype must be HX_BF16 or HX_F16, got %d", dtype);
+    return HX_ERR_BAD_ARG;
+  }
+  if (T_tok >= (1LL << 31) / top_k) {
+    hx_set_error("hx_moe_topk_matmul: dimension too large");
+    return HX_ERR_UNSUPPORTED;
+  }
+  const int64_t T = T_tok * top_k;
+  if (T == 0 || N == 0) return 0;
+  if (!A_tok || !C || !expert_ids || (E > 0 && !W)) {
+    hx_set_error("hx_moe_topk_matmul: null pointer");
+    return HX_ERR_BAD_ARG;
+  }
+  if (T >= (1LL << 31) || K >= (1LL << 31) || N >= (1LL << 31) || E >= (1LL << 24) || N > 65535LL * 64) {
+    hx_set_error("hx_moe_topk_matmul: dimension too large");
+    return HX_ERR_UNSUPPORTED;
+  }
+  if (!workspace || workspace_bytes < hx_moe_topk_workspace_bytes(T_tok, top_k, E) || ((uintptr_t)workspace & 15)) {
+    hx_set_error("hx_moe_topk_matmul: workspace must be 16-byte aligned and at least %zu bytes (got %zu)",
+                 hx_moe_topk_workspace_bytes(T_tok, top_k, E), workspace_bytes);
+    return HX_ERR_WORKSPACE;
+  }
+  int32_t* counts = (int32_t*)workspace;
+  int32_t* offsets = counts + E;
+  int32_t* max_count = offsets + E + 1;
+  int32_t* idx = max_count + 1;
+  void* ws2 = (uint8_t*)workspace + moe_topk_tables_bytes(T, E);
+  int rc = hx_moe_routing(expert_ids, ids_are_int64, T, E, counts, offsets, idx, max_count, idx + T, hx_moe_routing_workspace_bytes(T, E),
+                          stream);
+  if (rc != 0) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == HX_BF16) return launch_moe<true>(A_tok, W, C, counts, offsets, idx, T, K, N, E, top_k, ws2, s);
+  return launch_moe<false>(A_tok, W, C, counts, offsets, idx, T, K, N, E, top_k, ws2, s);
 }

@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import torch
 
-from .ops import moe_matmul_ogs_op
+from .ops import moe_matmul_ogs_op, moe_matmul_topk_op, moe_routing_op
 
 
 def moe_matmul_ogs(A: torch.Tensor, W: torch.Tensor, expert_token_counts: torch.Tensor,
@@ -17,9 +17,14 @@ def moe_matmul_ogs(A: torch.Tensor, W: torch.Tensor, expert_token_counts: torch.
 
 
 def moe_matmul_ogs_helion_kernel_args_gen(A: torch.Tensor, W: torch.Tensor, top1_expert_per_token: torch.Tensor):
-    """examples/moe_matmul_ogs.py:84-121: stable sort of rows by expert, per-expert counts and offsets."""
+    """examples/moe_matmul_ogs.py:84-121: stable sort of rows by expert, per-expert counts and offsets.
+    On the GPU the three tables come from one routing kernel; the host synchronisation the reference has
+    (``.item()`` for the size of the dummy tensor, :113) is kept because the signature needs that size."""
     E = W.size(0)
     device = A.device
+    if A.is_cuda and E <= 512 and top1_expert_per_token.dtype in (torch.int32, torch.int64):
+        counts, offsets, idx, max_count = moe_routing_op(top1_expert_per_token, E)
+        return (A, W, counts, offsets, idx, torch.empty(int(max_count.item()), device=device))
     sorted_to_orig_token_idx = torch.argsort(top1_expert_per_token, stable=True).to(torch.int32)
     expert_token_counts = torch.bincount(top1_expert_per_token, minlength=E).to(torch.int32)
     expert_token_offsets = torch.empty(E + 1, dtype=torch.int32, device=device)
@@ -28,6 +33,20 @@ def moe_matmul_ogs_helion_kernel_args_gen(A: torch.Tensor, W: torch.Tensor, top1
     max_T_per_expert = int(expert_token_counts.max().item())
     return (A, W, expert_token_counts, expert_token_offsets, sorted_to_orig_token_idx,
             torch.empty(max_T_per_expert, device=device))
+
+
+def moe_matmul_topk(A: torch.Tensor, W: torch.Tensor, expert_ids: torch.Tensor, top_k: int = 1) -> torch.Tensor:
+    """Top-k form without the replicated activations and without any host synchronisation: ``A`` is [T_tok, K],
+    ``expert_ids`` holds T_tok*top_k ids (token-major, i.e. ``topk_indices.reshape(-1)``), the result is
+    [T_tok*top_k, N] with row r = A[r // top_k] @ W[expert_ids[r]].  Equals
+    ``moe_matmul_ogs(*moe_matmul_ogs_helion_kernel_args_gen(A.repeat_interleave(top_k, 0), W, expert_ids))``."""
+    return moe_matmul_topk_op(A, W, expert_ids, int(top_k))
+
+
+def moe_routing(expert_ids: torch.Tensor, num_experts: int):
+    """(counts, offsets, sorted_to_orig_idx, max_count) as int32 device tensors from one kernel; the tensor form
+    of examples/moe_matmul_ogs.py:98-113 with ``max_count`` left on the device."""
+    return moe_routing_op(expert_ids, int(num_experts))
 
 
 def moe_matmul_ogs_reference(A: torch.Tensor, W: torch.Tensor, top1_expert_per_token: torch.Tensor) -> torch.Tensor:

@@ -137,3 +137,71 @@ def moe_matmul_ogs_op(A: torch.Tensor, W: torch.Tensor, expert_token_counts: tor
 @moe_matmul_ogs_op.register_fake
 def _(A, W, expert_token_counts, expert_token_offsets, sorted_to_orig_token_idx, max_T_per_expert):
     return A.new_empty((A.shape[0], W.shape[2]), dtype=torch.promote_types(A.dtype, W.dtype))
+
+
+# ------------------------------------------------------------------------------ moe routing tables
+@torch.library.custom_op("helion_amd::moe_routing", mutates_args=())
+def moe_routing_op(expert_ids: torch.Tensor, num_experts: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(counts [E], offsets [E+1], idx [T], max_count [1]), all int32 on the device, no host synchronisation."""
+    _require_cuda(expert_ids)
+    if expert_ids.dim() != 1 or expert_ids.dtype not in (torch.int32, torch.int64):
+        raise ValueError("moe_routing expects a 1-D int32 or int64 tensor of expert ids")
+    ids = expert_ids.contiguous()
+    T, E = ids.numel(), int(num_experts)
+    dev = ids.device
+    counts = torch.empty(E, dtype=torch.int32, device=dev)
+    offsets = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    idx = torch.empty(T, dtype=torch.int32, device=dev)
+    max_count = torch.empty(1, dtype=torch.int32, device=dev)
+    lib = _lib.load()
+    ws_bytes = lib.hx_moe_routing_workspace_bytes(T, E)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+    rc = lib.hx_moe_routing(ids.data_ptr(), int(ids.dtype == torch.int64), T, E, counts.data_ptr(), offsets.data_ptr(),
+                            idx.data_ptr(), max_count.data_ptr(), ws.data_ptr() if ws is not None else None, ws_bytes,
+                            _stream_ptr(dev))
+    _lib.check(rc, "hx_moe_routing")
+    return counts, offsets, idx, max_count
+
+
+@moe_routing_op.register_fake
+def _(expert_ids, num_experts):
+    i32 = dict(dtype=torch.int32)
+    return (expert_ids.new_empty(num_experts, **i32), expert_ids.new_empty(num_experts + 1, **i32),
+            expert_ids.new_empty(expert_ids.shape[0], **i32), expert_ids.new_empty(1, **i32))
+
+
+# ------------------------------------------------------------------------------ moe top-k matmul (routing fused in)
+@torch.library.custom_op("helion_amd::moe_matmul_topk", mutates_args=())
+def moe_matmul_topk_op(A: torch.Tensor, W: torch.Tensor, expert_ids: torch.Tensor, top_k: int) -> torch.Tensor:
+    _require_cuda(A, W, expert_ids)
+    if A.dim() != 2 or W.dim() != 3:
+        raise ValueError("moe_matmul_topk expects A [T_tok,K] and W [E,K,N]")
+    T_tok, K = A.shape
+    E, K2, N = W.shape
+    if K != K2:
+        raise ValueError(f"size mismatch K={K} vs W.size(1)={K2}")
+    if top_k < 1 or expert_ids.numel() != T_tok * top_k:
+        raise ValueError("expert_ids must hold T_tok * top_k ids (token-major)")
+    if expert_ids.dtype not in (torch.int32, torch.int64):
+        raise ValueError("expert_ids must be int32 or int64")
+    dtype = torch.promote_types(A.dtype, W.dtype)
+    if dtype not in (torch.bfloat16, torch.float16):
+        raise TypeError(f"moe_matmul_topk supports float16/bfloat16, got {A.dtype} x {W.dtype}")
+    A = A.to(dtype).contiguous()
+    W = W.to(dtype).contiguous()
+    ids = expert_ids.reshape(-1).contiguous()
+    C = torch.empty((T_tok * top_k, N), dtype=dtype, device=A.device)
+    if C.numel() == 0:
+        return C
+    lib = _lib.load()
+    ws_bytes = lib.hx_moe_topk_workspace_bytes(T_tok, top_k, E)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=A.device)
+    rc = lib.hx_moe_topk_matmul(A.data_ptr(), W.data_ptr(), C.data_ptr(), ids.data_ptr(), int(ids.dtype == torch.int64),
+                                T_tok, top_k, K, N, E, _DT[dtype], ws.data_ptr(), ws_bytes, _stream_ptr(A.device))
+    _lib.check(rc, "hx_moe_topk_matmul")
+    return C
+
+
+@moe_matmul_topk_op.register_fake
+def _(A, W, expert_ids, top_k):
+    return A.new_empty((A.shape[0] * top_k, W.shape[2]), dtype=torch.promote_types(A.dtype, W.dtype))

@@ -92,6 +92,31 @@ int hx_moe_grouped_gemm(const void* A, const void* W, void* C, const int32_t* co
                         void* stream);
 size_t hx_moe_workspace_bytes(int64_t T, int64_t E);
 
+/* Replaces the tensor ops of `moe_matmul_ogs_helion_kernel_args_gen(A, W, top1_expert_per_token)` (reference:
+ * examples/moe_matmul_ogs.py:84-121) with one kernel and no host synchronisation:
+ *   idx = argsort(expert_ids, stable=True); counts = bincount(expert_ids, minlength=E);
+ *   offsets = [0, cumsum(counts)]; *max_count = max(counts)   (the reference's `.item()` value, left on the device).
+ * expert_ids: [T] device array of int32 (ids_are_int64 == 0) or int64; counts [E], offsets [E+1], idx [T],
+ * max_count [1] are int32 device arrays.  Ids outside [0, E) are skipped: their rows appear in no expert's list,
+ * offsets[E] is then < T and idx[offsets[E]..T) is filled with -1.  Supported: E <= 512, T < 2^31 - 8192.
+ * workspace: hx_moe_routing_workspace_bytes(T, E) bytes of device scratch (0 up to 32768 rows, where one workgroup
+ * does the whole job in one launch); with less, larger inputs also run on that one workgroup, correct but slow. */
+int hx_moe_routing(const void* expert_ids, int ids_are_int64, int64_t T, int64_t E, int32_t* counts, int32_t* offsets,
+                   int32_t* idx, int32_t* max_count, void* workspace, size_t workspace_bytes, void* stream);
+size_t hx_moe_routing_workspace_bytes(int64_t T, int64_t E);
+
+/* Top-k form of the same path, without the reference caller's `A.repeat_interleave(top_k, 0)` copy and without
+ * its host synchronisation: routes on the device (hx_moe_routing) and runs the grouped GEMM with row r of C
+ * computed from row r / top_k of A_tok.
+ *   A_tok: [T_tok, K]; expert_ids: [T_tok*top_k] (row r = token r / top_k, slot r % top_k); W: [E,K,N];
+ *   C: [T_tok*top_k, N]; rows whose id is outside [0, E) are zero.
+ * With top_k == 1 this is moe_matmul_ogs(A, W, *args_gen(A, W, expert_ids)) (examples/moe_matmul_ogs.py:25-121).
+ * workspace: hx_moe_topk_workspace_bytes(T_tok, top_k, E) bytes, 16-byte aligned. */
+int hx_moe_topk_matmul(const void* A_tok, const void* W, void* C, const void* expert_ids, int ids_are_int64,
+                       int64_t T_tok, int64_t top_k, int64_t K, int64_t N, int64_t E, int dtype, void* workspace,
+                       size_t workspace_bytes, void* stream);
+size_t hx_moe_topk_workspace_bytes(int64_t T_tok, int64_t top_k, int64_t E);
+
 #ifdef __cplusplus
 }
 #endif

@@ -66,3 +66,10 @@ def test_attention_and_moe_argument_errors():
     assert lib.hx_moe_grouped_gemm(16, 16, 16, 16, 16, 16, 8, 8, 8, 2, 8, 2, None, 0, None) == -1  # f32 tag
     assert lib.hx_moe_grouped_gemm(16, 16, 16, 16, 16, 16, 8, 8, 8, 2, 8, 1, None, 0, None) == -3  # no workspace
     assert b"workspace" in lib.hx_last_error()
+    assert lib.hx_moe_routing(16, 1, 100, 513, 16, 16, 16, 16, None, 0, None) == -2  # more experts than the kernel's table holds
+    assert lib.hx_moe_routing(None, 1, 100, 8, 16, 16, 16, 16, None, 0, None) == -1
+    assert lib.hx_moe_routing(16, 1, -1, 8, 16, 16, 16, 16, None, 0, None) == -1
+    assert lib.hx_moe_routing_workspace_bytes(32768, 8) == 0 and lib.hx_moe_routing_workspace_bytes(1 << 20, 8) == 64 * 8 * 4
+    assert lib.hx_moe_topk_workspace_bytes(1000, 2, 30) >= lib.hx_moe_workspace_bytes(2000, 30) + 2000 * 4
+    assert lib.hx_moe_topk_matmul(16, 16, 16, 16, 1, 8, 0, 8, 8, 2, 1, None, 0, None) == -1  # top_k < 1
+    assert lib.hx_moe_topk_matmul(16, 16, 16, 16, 1, 8, 2, 8, 8, 2, 1, None, 0, None) == -3  # no workspace
