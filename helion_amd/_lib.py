@@ -29,8 +29,8 @@ _SIGNATURES = {
     ),
     "hx_fp8_attention": (
         _c.c_int,
-        [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int,
-         _c.c_int, _c.c_void_p],
+        [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64,
+         _c.c_int64, _c.c_int, _c.c_int, _c.c_void_p],
     ),
     "hx_moe_grouped_gemm": (
         _c.c_int,

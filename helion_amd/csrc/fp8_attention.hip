@@ -14,6 +14,12 @@
 // 16..31 = the same keys of block 1; the V^T operand reads the matching two 16-byte chunks.
 // Row max / row sum need no cross-lane traffic inside the key loop: each lane reduces its own
 // values and the two lanes of a query are combined once (exact_max) or once per tile (online).
+//
+// V comes in either of two physical layouts per head: [D][S] (VSD = false; "pre-transposed" and contiguous) or
+// [S][D] (VSD = true; what examples/fp8_attention.py:110-133 really hands over: `v.permute(0,1,3,2).to(e4m3)`
+// keeps the memory order of the [B,H,S,D] source and only the strides say [D,S]).  In the second case a V tile
+// sits in LDS like a K tile, rows = keys, and the V^T operand is formed by transposing LDS reads
+// (ds_read_b64_tr_b8: 8 keys x 16 columns per 16 lanes), so neither layout needs a copy.
 #include "hx_common.h"
 
 #define ATT_BN 64      // keys per tile
@@ -28,6 +34,14 @@ template <int RB>
 __device__ __forceinline__ int att_swz(int row) {
   return RB == 128 ? ((row >> 1) & 7) : ((row >> 2) & 3);
 }
+// V tile in the [keys][D bytes] layout: one transposing read has 32 lanes fetch 8 consecutive key rows x two
+// adjacent 16-byte chunks; the swizzle has to spread those over all banks and must leave bit 0 (which chunk of
+// the pair) alone.  RB = 128: rows r, r+1 share a 256-byte bank window -> (r>>1)&3 into bits 2:1;  RB = 64: rows
+// r, r+4 share a 64-byte quarter of it -> (r>>2)&1 into bit 1.
+template <int RB>
+__device__ __forceinline__ int att_vswz(int row) {
+  return RB == 128 ? (((row >> 1) & 3) << 1) : (((row >> 2) & 1) << 1);
+}
 
 // wait until at most `newer` tiles' worth of this wave's DMA instructions (IPT per tile) are outstanding
 template <int IPT>
@@ -37,7 +51,7 @@ __device__ __forceinline__ void att_wait_tiles(int newer) {
   else __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(0));
 }
 
-template <int D, int OUT, bool EXACT>
+template <int D, int OUT, bool EXACT, bool VSD>
 __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t* __restrict__ Q, const uint8_t* __restrict__ Kt,
                                                                   const uint8_t* __restrict__ Vt, void* __restrict__ Out, int S,
                                                                   int BH, int qtiles) {
@@ -45,7 +59,7 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
   constexpr int DB = D / 32;      // 32-row blocks of O^T
   constexpr int KROWS_PER_DMA = 1024 / D;
   constexpr int KPW = (ATT_BN / KROWS_PER_DMA) / ATT_WAVES;  // K DMA instructions per wave per tile
-  constexpr int VPW = (D / 16) / ATT_WAVES;                  // V DMA instructions per wave per tile (16 rows x 64 B each)
+  constexpr int VPW = VSD ? KPW : (D / 16) / ATT_WAVES;      // V DMA instructions per wave per tile ([D][S]: 16 rows x 64 B each)
   constexpr int TILE = ATT_BN * D;                           // bytes of a K tile == bytes of a V tile
   __shared__ __attribute__((aligned(1024))) uint8_t smem[ATT_NS][2][TILE];
 
@@ -67,7 +81,7 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
 
   const uint8_t* Qh = Q + (long)bh * S * D;
   const uint8_t* Kh = Kt + (long)bh * S * D;
-  const uint8_t* Vh = Vt + (long)bh * D * S;
+  const uint8_t* Vh = Vt + (long)bh * D * S;  // either layout: D*S bytes per head
 
   // ---- Q fragments (B operand of S^T): lane (q, G): Q[q][64t + 32G .. +31]
   v8i qf[KSTEPS];
@@ -88,7 +102,8 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
   const int k_lrow = lane / KCPR, k_lpos = lane % KCPR;
   const uint32_t k_vo = (uint32_t)(k_lrow * D + ((k_lpos ^ att_swz<D>(w * KROWS_PER_DMA + k_lrow)) * 16));
   const int v_lrow = lane >> 2, v_lpos = lane & 3;
-  const uint32_t v_vo = (uint32_t)(v_lrow * S + ((v_lpos ^ att_swz<64>(v_lrow)) * 16));
+  const uint32_t v_vo = VSD ? (uint32_t)(k_lrow * D + ((k_lpos ^ att_vswz<D>(w * KROWS_PER_DMA + k_lrow)) * 16))
+                            : (uint32_t)(v_lrow * S + ((v_lpos ^ att_swz<64>(v_lrow)) * 16));
   const uint32_t lds0 = hx_lds_addr(&smem[0][0][0]);
   auto issue_k = [&](int tile, int stage) {
 #pragma unroll
@@ -101,7 +116,8 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
 #pragma unroll
     for (int jj = 0; jj < VPW; ++jj) {
       const int j = w + ATT_WAVES * jj;
-      hx_g2l16_s(Vh + (long)(j * 16) * S + (long)tile * ATT_BN, v_vo, lds0 + (uint32_t)stage * 2 * TILE + TILE + j * 1024);
+      if (VSD) hx_g2l16_s(Vh + ((long)tile * ATT_BN + j * KROWS_PER_DMA) * D, v_vo, lds0 + (uint32_t)stage * 2 * TILE + TILE + j * 1024);
+      else hx_g2l16_s(Vh + (long)(j * 16) * S + (long)tile * ATT_BN, v_vo, lds0 + (uint32_t)stage * 2 * TILE + TILE + j * 1024);
     }
   };
 
@@ -118,9 +134,34 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
         const int row = kb * 32 + krow;
         k_off[kb][t][h] = row * D + (((4 * t + 2 * G + h) ^ att_swz<D>(row)) * 16);
       }
-  int v_off[2];  // [block] byte offsets in the V tile for d-row lane%32 (add db*32*64)
+  int v_off[2];  // [D][S] layout: [block] byte offsets in the V tile for d-row lane%32 (add db*32*64)
 #pragma unroll
   for (int kb = 0; kb < 2; ++kb) v_off[kb] = q31 * 64 + (((2 * kb + G) ^ att_swz<64>(q31)) * 16);
+  // [S][D] layout: transposing read j (0..3) of a 32-row block of V^T fetches keys kr0..kr0+7,
+  // kr0 = 32*(j>>1) + 16*G + 8*(j&1); this lane supplies 8 bytes of key row kr0 + (lane%16)/2, columns
+  // 16*((lane>>4)&1) + 8*(lane&1) .. +7 of the block, and receives column lane%32, keys kr0..kr0+7.
+  // Block db adds 2*db to the chunk index in bits the swizzle's xor commutes with: offset ^ (db*32).
+  int vt_off[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int row = 32 * (j >> 1) + 16 * G + 8 * (j & 1) + ((lane & 15) >> 1);
+    vt_off[j] = row * D + (((((lane >> 4) & 1)) ^ att_vswz<D>(row)) * 16) + (lane & 1) * 8;
+  }
+  auto load_vfrag = [&](const uint8_t* sv, int d) -> v8i {
+    if (VSD) {
+      v8i f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v2i part = __builtin_amdgcn_ds_read_tr8_b64_v2i32((v2i __attribute__((address_space(3)))*)(sv + (vt_off[j] ^ (d * 32))));
+        f[2 * j] = part[0];
+        f[2 * j + 1] = part[1];
+      }
+      return f;
+    }
+    v4i lo = *(const v4i*)(sv + d * 32 * 64 + v_off[0]);
+    v4i hi = *(const v4i*)(sv + d * 32 * 64 + v_off[1]);
+    return (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+  };
 
   const float c = (float)((1.0 / __builtin_sqrt((double)D)) * 1.44269504);
   const int ntiles = S / ATT_BN;
@@ -234,12 +275,7 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
       }
     }
 #pragma unroll
-    for (int d = 0; d < DB; ++d) {
-      v4i lo = *(const v4i*)(sv + d * 32 * 64 + v_off[0]);
-      v4i hi = *(const v4i*)(sv + d * 32 * 64 + v_off[1]);
-      v8i vf = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-      o[d] = hx_mfma_32x32x64_e4m3(vf, pf, o[d]);
-    }
+    for (int d = 0; d < DB; ++d) o[d] = hx_mfma_32x32x64_e4m3(load_vfrag(sv, d), pf, o[d]);
   };
 
   for (int t = 0; t < ATT_LEAD && t < ntiles; ++t) {
@@ -302,17 +338,24 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
   }
 }
 
-template <int D, int OUT>
-static int launch_att(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t S, int exact, hipStream_t s) {
+template <int D, int OUT, bool EXACT, bool VSD>
+static void launch_att_kernel(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t S, hipStream_t s) {
   const int qtiles = (int)((S + ATT_BM - 1) / ATT_BM);
   const int hpx = (int)((BH + 7) / 8);
   const int grid = 8 * hpx * qtiles;
-  if (exact)
-    hipLaunchKernelGGL((hx_fp8_attention_kernel<D, OUT, true>), dim3(grid), dim3(256), 0, s, (const uint8_t*)q, (const uint8_t*)k,
-                       (const uint8_t*)v, out, (int)S, (int)BH, qtiles);
-  else
-    hipLaunchKernelGGL((hx_fp8_attention_kernel<D, OUT, false>), dim3(grid), dim3(256), 0, s, (const uint8_t*)q, (const uint8_t*)k,
-                       (const uint8_t*)v, out, (int)S, (int)BH, qtiles);
+  hipLaunchKernelGGL((hx_fp8_attention_kernel<D, OUT, EXACT, VSD>), dim3(grid), dim3(256), 0, s, (const uint8_t*)q, (const uint8_t*)k,
+                     (const uint8_t*)v, out, (int)S, (int)BH, qtiles);
+}
+
+template <int D, int OUT>
+static int launch_att(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t S, int exact, bool vsd, hipStream_t s) {
+  if (exact) {
+    if (vsd) launch_att_kernel<D, OUT, true, true>(q, k, v, out, BH, S, s);
+    else launch_att_kernel<D, OUT, true, false>(q, k, v, out, BH, S, s);
+  } else {
+    if (vsd) launch_att_kernel<D, OUT, false, true>(q, k, v, out, BH, S, s);
+    else launch_att_kernel<D, OUT, false, false>(q, k, v, out, BH, S, s);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     hx_set_error("hx_fp8_attention: launch failed: %s", hipGetErrorString(e));
@@ -322,7 +365,7 @@ static int launch_att(const void* q, const void* k, const void* v, void* out, in
 }
 
 extern "C" int hx_fp8_attention(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t S, int64_t D,
-                                int out_dtype, int exact_max, void* stream) {
+                                int64_t v_stride_d, int64_t v_stride_s, int out_dtype, int exact_max, void* stream) {
   if (BH < 0 || S < 0 || D < 0) {
     hx_set_error("hx_fp8_attention: negative size");
     return HX_ERR_BAD_ARG;
@@ -341,6 +384,14 @@ extern "C" int hx_fp8_attention(const void* q, const void* k, const void* v, voi
                  (long long)D);
     return HX_ERR_UNSUPPORTED;
   }
+  bool vsd;
+  if (v_stride_s == 1 && (v_stride_d == S || D == 1)) vsd = false;       // [D][S] per head
+  else if (v_stride_d == 1 && (v_stride_s == D || S == 1)) vsd = true;   // [S][D] per head
+  else {
+    hx_set_error("hx_fp8_attention: v strides (d: %lld, s: %lld) are neither [D][S] (S, 1) nor [S][D] (1, D) per head",
+                 (long long)v_stride_d, (long long)v_stride_s);
+    return HX_ERR_UNSUPPORTED;
+  }
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) {
     hx_set_error("hx_fp8_attention: pointers must be 16-byte aligned");
     return HX_ERR_UNSUPPORTED;
@@ -351,9 +402,9 @@ extern "C" int hx_fp8_attention(const void* q, const void* k, const void* v, voi
   }
   hipStream_t s = (hipStream_t)stream;
   if (D == 128) {
-    if (out_dtype == HX_F32) return launch_att<128, HX_F32>(q, k, v, out, BH, S, exact_max, s);
-    return launch_att<128, HX_E4M3>(q, k, v, out, BH, S, exact_max, s);
+    if (out_dtype == HX_F32) return launch_att<128, HX_F32>(q, k, v, out, BH, S, exact_max, vsd, s);
+    return launch_att<128, HX_E4M3>(q, k, v, out, BH, S, exact_max, vsd, s);
   }
-  if (out_dtype == HX_F32) return launch_att<64, HX_F32>(q, k, v, out, BH, S, exact_max, s);
-  return launch_att<64, HX_E4M3>(q, k, v, out, BH, S, exact_max, s);
+  if (out_dtype == HX_F32) return launch_att<64, HX_F32>(q, k, v, out, BH, S, exact_max, vsd, s);
+  return launch_att<64, HX_E4M3>(q, k, v, out, BH, S, exact_max, vsd, s);
 }

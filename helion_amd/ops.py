@@ -83,13 +83,17 @@ def fp8_attention_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batch: i
         raise ValueError(f"shape mismatch: q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)} (v must be [BH, D, S])")
     if out_dtype not in (torch.float8_e4m3fn, torch.float32):
         raise TypeError(f"unsupported out_dtype {out_dtype}")
-    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    q, k = q.contiguous(), k.contiguous()
+    # v is logically [BH, D, S].  The reference's preprocessing hands it over as a permuted view of [BH, S, D]
+    # memory (strides (S*D, 1, D)); the kernel reads that layout directly, so only other stridings are copied.
+    if bh > 1 and v.stride(0) != s * d or v.stride()[1:] not in ((s, 1), (1, d)):
+        v = v.contiguous()
     out = torch.empty((batch, heads, s, d), dtype=out_dtype, device=q.device)
     if bh == 0 or s == 0:
         return out
     lib = _lib.load()
-    rc = lib.hx_fp8_attention(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), bh, s, d, _DT[out_dtype],
-                              1 if exact_max else 0, _stream_ptr(q.device))
+    rc = lib.hx_fp8_attention(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), bh, s, d, v.stride(1), v.stride(2),
+                              _DT[out_dtype], 1 if exact_max else 0, _stream_ptr(q.device))
     _lib.check(rc, "hx_fp8_attention")
     return out
 

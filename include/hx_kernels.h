@@ -67,14 +67,19 @@ int hx_fp8_gemm_path(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k
 
 /* Replaces the device side of `fp8_attention_kernel(q, k, v, batch, heads)` (reference:
  * examples/fp8_attention.py:22-106; generated kernel test/test_examples.expected:718-766).
- * q,k: [BH,S,D] e4m3fn contiguous; v: [BH,D,S] e4m3fn contiguous (pre-transposed);
+ * q,k: [BH,S,D] e4m3fn contiguous; v: logically [BH,D,S] e4m3fn, element (bh,d,s) at
+ *   v[bh*S*D + d*v_stride_d + s*v_stride_s], in one of two physical layouts per head:
+ *   (v_stride_d, v_stride_s) = (S, 1): [D][S] contiguous ("pre-transposed");
+ *   (v_stride_d, v_stride_s) = (1, D): [S][D], which is what the reference's own preprocessing produces
+ *   (examples/fp8_attention.py:119-121: `v.permute(0,1,3,2).to(e4m3)` keeps the memory order of [B,H,S,D]);
+ *   neither needs a copy: the second is read with transposing LDS loads.
  * out: [BH,S,D] contiguous (== [batch,heads,S,D]) of out_dtype HX_E4M3 (reference) or HX_F32.
  * exact_max != 0: two passes, P is quantised to e4m3 against the exact row max (bit-faithful to
  *   the reference's ref-eager execution); exact_max == 0: one pass, online softmax, P quantised
  *   against the running max (what the reference's compiled kernel does).
  * Supported: D == 128 or 64, S % 64 == 0. */
 int hx_fp8_attention(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t S,
-                     int64_t D, int out_dtype, int exact_max, void* stream);
+                     int64_t D, int64_t v_stride_d, int64_t v_stride_s, int out_dtype, int exact_max, void* stream);
 
 /* Replaces the device side of `moe_matmul_ogs(A, W, expert_token_counts, expert_token_offsets,
  * sorted_to_orig_token_idx, max_T_per_expert_tensor)` (reference: examples/moe_matmul_ogs.py:25-80;

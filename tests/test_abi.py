@@ -57,11 +57,13 @@ def test_gemm_path_selection():
 
 def test_attention_and_moe_argument_errors():
     lib = _lib.load()
-    assert lib.hx_fp8_attention(1, 1, 1, 1, -1, 64, 64, 3, 1, None) == -1
-    assert lib.hx_fp8_attention(16, 16, 16, 16, 2, 100, 64, 3, 1, None) == -2  # S % 64
-    assert lib.hx_fp8_attention(16, 16, 16, 16, 2, 128, 96, 3, 1, None) == -2  # D
-    assert lib.hx_fp8_attention(16, 16, 16, 16, 2, 128, 64, 1, 1, None) == -1  # bf16 output not offered
-    assert lib.hx_fp8_attention(None, None, None, None, 0, 128, 64, 3, 1, None) == 0
+    assert lib.hx_fp8_attention(1, 1, 1, 1, -1, 64, 64, 64, 1, 3, 1, None) == -1
+    assert lib.hx_fp8_attention(16, 16, 16, 16, 2, 100, 64, 100, 1, 3, 1, None) == -2  # S % 64
+    assert lib.hx_fp8_attention(16, 16, 16, 16, 2, 128, 96, 128, 1, 3, 1, None) == -2  # D
+    assert lib.hx_fp8_attention(16, 16, 16, 16, 2, 128, 64, 128, 1, 1, 1, None) == -1  # bf16 output not offered
+    assert lib.hx_fp8_attention(16, 16, 16, 16, 2, 128, 64, 256, 2, 3, 1, None) == -2  # v neither [D][S] nor [S][D]
+    assert b"strides" in lib.hx_last_error()
+    assert lib.hx_fp8_attention(None, None, None, None, 0, 128, 64, 128, 1, 3, 1, None) == 0
     assert lib.hx_moe_workspace_bytes(1000, 30) >= 1000
     assert lib.hx_moe_grouped_gemm(16, 16, 16, 16, 16, 16, 8, 8, 8, 2, 8, 2, None, 0, None) == -1  # f32 tag
     assert lib.hx_moe_grouped_gemm(16, 16, 16, 16, 16, 16, 8, 8, 8, 2, 8, 1, None, 0, None) == -3  # no workspace

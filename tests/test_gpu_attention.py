@@ -104,3 +104,32 @@ def test_c4_sampled_heads_and_key_permutation():
     out_p = hx.fp8_attention_kernel(qd, kd[:, perm].contiguous(), vd[:, :, perm].contiguous(), b, h, out_dtype=torch.float32)
     # same exact row max, same quantisation grid; only MFMA summation order differs
     assert rel_err(out_p, out) <= 5e-3
+
+
+@pytest.mark.parametrize("b,h,s,d", [(1, 2, 128, 64), (2, 3, 256, 64), (1, 3, 192, 128), (2, 4, 512, 128)])
+@pytest.mark.parametrize("exact", [True, False])
+def test_v_as_permuted_view_of_seq_major_memory(b, h, s, d, exact):
+    """examples/fp8_attention.py:110-133 hands v over as a [BH, D, S] *view* of [BH, S, D] memory (permute, cast,
+    reshape: strides (S*D, 1, D)).  The kernel reads that layout in place; operands and summation order are the
+    same as for the contiguous [BH, D, S] tensor, so the results must be identical bit for bit."""
+    g = torch.Generator().manual_seed(s + d)
+    q32, k32, v32 = (torch.randn(b, h, s, d, generator=g) for _ in range(3))
+    q8, k8, v8 = hx.preprocess_fp8_attention_inputs(q32.to(DEV), k32.to(DEV), v32.to(DEV))
+    assert v8.shape == (b * h, d, s) and v8.stride() == (s * d, 1, d)       # what the reference's own code produces
+    out_view = hx.fp8_attention_kernel(q8, k8, v8, b, h, out_dtype=torch.float32, exact_max=exact)
+    out_contig = hx.fp8_attention_kernel(q8, k8, v8.contiguous(), b, h, out_dtype=torch.float32, exact_max=exact)
+    assert torch.equal(out_view, out_contig)
+    if exact:
+        ref = orc.fp8_attention(q8.cpu(), k8.cpu(), v8.cpu(), b, h, torch.float32)
+        assert rel_err(out_view, ref) <= TOL
+        out8 = hx.fp8_attention_kernel(q8, k8, v8, b, h)
+        assert torch.equal(out8.view(torch.uint8), hx.fp8_attention_kernel(q8, k8, v8.contiguous(), b, h).view(torch.uint8))
+
+
+def test_tritonbench_wrapper_runs_on_the_reference_layout():
+    g = torch.Generator().manual_seed(11)
+    q32, k32, v32 = (torch.randn(1, 2, 256, 128, generator=g).to(DEV) for _ in range(3))
+    out = hx.fp8_attention_tritonbench(q32, k32, v32)()
+    q8, k8, v8 = hx.preprocess_fp8_attention_inputs(q32.cpu(), k32.cpu(), v32.cpu())
+    ref = orc.fp8_attention(q8, k8, v8, 1, 2)
+    assert out.dtype == E4M3 and rel_err(out, ref) <= 0.08
