@@ -155,35 +155,56 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
     kstep(fa0, fb0, fa1, fb1, stage, 1, true, false, 0, 0);
     kstep(fa1, fb1, fa0, fb0, 0, 0, false, false, 0, 0);
   }
-  HX_WAIT_VM0();  // the trailing re-fetch must have landed before the workgroup's LDS is released
+  HX_WAIT_VM0();    // the trailing re-fetch has landed ...
+  __syncthreads();  // ... and every wave is past its last fragment read: the LDS can be reused
 
-  // ---- epilogue: acc[bj][bi][4a+b] is C[m0 + wm*128 + bi*32 + lane%32][n0 + wn*128 + bj*32 + 8a + 4g + b]
+  // ---- epilogue: acc[bj][bi][4a+b] is C[m0 + wm*128 + bi*32 + lane%32][n0 + wn*128 + bj*32 + 8a + 4g + b].
+  // A lane holds only 4 consecutive columns of a row, so direct stores would hit every 128-byte line of C with
+  // eight separate 16-byte writes.  Each wave instead passes its 32 x 128 block of a row group through its own
+  // quarter of the LDS and writes whole rows: 16 bytes per lane, consecutive lanes on consecutive bytes.
   float alpha = 1.f;
   if (scale_a) alpha = *scale_a;
   if (scale_b) alpha = alpha * *scale_b;
+  constexpr int ESZ = (int)sizeof(out_t);
+  constexpr int ROWB = 128 * ESZ;                   // bytes of one output row of this wave
+  constexpr int RSTR = ROWB + (ESZ == 2 ? 8 : 16);  // padded row stride: conflict-free 8/16-byte writes down a column
+  constexpr int LPR = ROWB / 16;                    // lanes per row when reading back 16 bytes per lane
+  constexpr int RPI = 64 / LPR;                     // rows per store instruction
+  uint8_t* st = &smem[0][0][0] + w * T256_TILE_BYTES;  // this wave's 32 KB
+  typedef out_t ov4 __attribute__((ext_vector_type(4)));
+  const int rb_row = lane / LPR, rb_ch = lane % LPR;
 #pragma unroll
   for (int bi = 0; bi < 4; ++bi) {
-    const long m = m0 + wm * 128 + bi * 32 + r31;
-    out_t* crow = C + m * ldc + n0 + wn * 128 + 4 * g;
-    if (EDGE && m >= M) continue;
 #pragma unroll
     for (int bj = 0; bj < 4; ++bj)
 #pragma unroll
       for (int a = 0; a < 4; ++a) {
-        typedef out_t ov4 __attribute__((ext_vector_type(4)));
         ov4 o;
 #pragma unroll
         for (int b = 0; b < 4; ++b) o[b] = (out_t)(acc[bj][bi][4 * a + b] * alpha);
-        if (!EDGE) {
-          *(ov4*)(crow + bj * 32 + 8 * a) = o;
+        *(ov4*)(st + r31 * RSTR + (bj * 32 + 8 * a + 4 * g) * ESZ) = o;
+      }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // LDS operations of one wave execute in order
+#pragma unroll
+    for (int p = 0; p < 32 / RPI; ++p) {
+      const int row = p * RPI + rb_row;
+      const v4i v = *(const v4i*)(st + row * RSTR + rb_ch * 16);
+      const long m = m0 + wm * 128 + bi * 32 + row;
+      out_t* dst = C + m * ldc + n0 + wn * 128 + rb_ch * (16 / ESZ);
+      if (!EDGE) {
+        *(v4i*)dst = v;
+      } else if (m < M) {
+        const long n = n0 + wn * 128 + rb_ch * (16 / ESZ);
+        if (n + 16 / ESZ <= N && ((uintptr_t)dst & 15) == 0) {
+          *(v4i*)dst = v;
         } else {
-          const long n = n0 + wn * 128 + 4 * g + bj * 32 + 8 * a;
-          if (n + 4 <= N && ((uintptr_t)(crow + bj * 32 + 8 * a) & (sizeof(ov4) - 1)) == 0) *(ov4*)(crow + bj * 32 + 8 * a) = o;
-          else
-            for (int b = 0; b < 4; ++b)
-              if (n + b < N) crow[bj * 32 + 8 * a + b] = o[b];
+          const out_t* e = (const out_t*)&v;
+          for (int b = 0; b < 16 / ESZ; ++b)
+            if (n + b < N) dst[b] = e[b];
         }
       }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
 }
 
@@ -486,7 +507,7 @@ static int gemm_path_kmajor(int64_t M, int64_t N, int64_t K, int64_t lda, int64_
   if (!ok) return 0;
   if (M <= 16 && lda >= K && ldb >= K) return 2;
   if (lda >= (1LL << 27) || ldb >= (1LL << 27)) return 0;
-  if ((M % 256 == 0) && (N % 256 == 0) && (ldc % 4 == 0) && aligned(c, 16)) return 1;
+  if ((M % 256 == 0) && (N % 256 == 0) && (ldc % 8 == 0) && aligned(c, 16)) return 1;  // 16-byte row-aligned stores
   if (M * lda < (1LL << 32) && N * ldb < (1LL << 32)) return 3;
   return 0;
 }
