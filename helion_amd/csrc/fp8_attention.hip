@@ -309,32 +309,50 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
   }
   const float l_lane = (l4[0] + l4[1]) + (l4[2] + l4[3]);
 
+  __syncthreads();  // every wave is past its last K/V fragment read: the LDS ring can be reused
   if (!active) return;
   // ---------------- epilogue: o[db][4a+b] is O[q0 + lane%32][32 db + 8a + 4G + b]
+  // A lane holds 4 consecutive columns of its row, so direct stores would write every output line in 16- or
+  // 32-byte pieces.  Each wave instead passes its 32 rows through its own part of the LDS, PASS_COLS columns at a
+  // time, and writes 16 bytes per lane with consecutive lanes on consecutive bytes of a row.
   const float l = l_lane + __shfl_xor(l_lane, 32);
-  const int qrow = q0 + q31;
-  if (qrow >= S) return;
-  if (OUT == HX_F32) {
-    float* orow = (float*)Out + ((long)bh * S + qrow) * D + 4 * G;
+  constexpr int ESZ = OUT == HX_F32 ? 4 : 1;
+  constexpr int PASS_COLS = OUT == HX_F32 ? D / 2 : D;  // 256 or 128 bytes of a row per pass (128 or 64 for D = 64)
+  constexpr int PASS_BYTES = PASS_COLS * ESZ;
+  constexpr int RSTR = PASS_BYTES + 16;                 // padded row stride
+  constexpr int LPR = PASS_BYTES / 16;                  // lanes per row on the way out
+  constexpr int RPI = 64 / LPR;                         // rows per store instruction
+  constexpr int NDB = PASS_COLS / 32;                   // 32-column accumulator blocks per pass
+  static_assert(ATT_WAVES * 32 * RSTR <= ATT_NS * 2 * TILE, "output staging fits the K/V ring");
+  uint8_t* st = &smem[0][0][0] + w * (32 * RSTR);
+  uint8_t* out_rows = (uint8_t*)Out + ((long)bh * S + q0) * D * ESZ;
+  const int rb_row = lane / LPR, rb_ch = lane % LPR;
 #pragma unroll
-    for (int d = 0; d < DB; ++d)
+  for (int h = 0; h < D / PASS_COLS; ++h) {
 #pragma unroll
-      for (int a = 0; a < 4; ++a) {
-        v4f v;
-#pragma unroll
-        for (int b = 0; b < 4; ++b) v[b] = o[d][4 * a + b] / l;
-        *(v4f*)(orow + d * 32 + 8 * a) = v;
-      }
-  } else {
-    uint8_t* orow = (uint8_t*)Out + ((long)bh * S + qrow) * D + 4 * G;
-#pragma unroll
-    for (int d = 0; d < DB; ++d)
+    for (int dd = 0; dd < NDB; ++dd)
 #pragma unroll
       for (int a = 0; a < 4; ++a) {
-        int dw = HX_CVT_PK_E4M3(o[d][4 * a] / l, o[d][4 * a + 1] / l, 0, false);
-        dw = HX_CVT_PK_E4M3(o[d][4 * a + 2] / l, o[d][4 * a + 3] / l, dw, true);
-        *(int*)(orow + d * 32 + 8 * a) = dw;
+        const int d = h * NDB + dd;
+        if (OUT == HX_F32) {
+          v4f v;
+#pragma unroll
+          for (int b = 0; b < 4; ++b) v[b] = o[d][4 * a + b] / l;
+          *(v4f*)(st + q31 * RSTR + (dd * 32 + 8 * a + 4 * G) * 4) = v;
+        } else {
+          int dw = HX_CVT_PK_E4M3(o[d][4 * a] / l, o[d][4 * a + 1] / l, 0, false);
+          dw = HX_CVT_PK_E4M3(o[d][4 * a + 2] / l, o[d][4 * a + 3] / l, dw, true);
+          *(int*)(st + q31 * RSTR + dd * 32 + 8 * a + 4 * G) = dw;
+        }
       }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // LDS operations of one wave execute in order
+#pragma unroll
+    for (int p = 0; p < 32 / RPI; ++p) {
+      const int row = p * RPI + rb_row;
+      const v4i v = *(const v4i*)(st + row * RSTR + rb_ch * 16);
+      *(v4i*)(out_rows + ((long)row * D + h * PASS_COLS) * ESZ + rb_ch * 16) = v;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
 }
 
