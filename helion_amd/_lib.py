@@ -50,6 +50,16 @@ _SIGNATURES = {
          _c.c_int64, _c.c_int, _c.c_void_p, _c.c_size_t, _c.c_void_p],
     ),
     "hx_moe_topk_workspace_bytes": (_c.c_size_t, [_c.c_int64, _c.c_int64, _c.c_int64]),
+    "hx_cast_e4m3": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int, _c.c_void_p, _c.c_void_p]),
+    "hx_fp8_attention_preprocess": (
+        _c.c_int,
+        [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int, _c.c_void_p],
+    ),
+    "hx_fp8_quantize": (
+        _c.c_int,
+        [_c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_size_t, _c.c_void_p],
+    ),
+    "hx_fp8_quantize_workspace_bytes": (_c.c_size_t, [_c.c_int64]),
 }
 
 

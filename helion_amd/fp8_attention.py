@@ -5,7 +5,7 @@ from typing import Callable
 
 import torch
 
-from .ops import fp8_attention_op
+from .ops import cast_e4m3_x3_op, fp8_attention_op
 
 
 def fp8_attention_kernel(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batch: int, heads: int, *,
@@ -19,7 +19,15 @@ def fp8_attention_kernel(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batc
 
 
 def preprocess_fp8_attention_inputs(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
-    """examples/fp8_attention.py:110-133: cast to e4m3 (v permuted to [B,H,D,S] first), flatten batch*heads."""
+    """examples/fp8_attention.py:110-133: cast to e4m3 (v permuted to [B,H,D,S] first), flatten batch*heads.
+    The permute-then-cast of the reference keeps v's memory in [B,H,S,D] order (only the strides change), so on the
+    GPU all three tensors go through one cast kernel and v comes back as the same strided view."""
+    batch, heads, seq_len, head_dim = q.shape
+    if (q.is_cuda and q.dtype == k.dtype == v.dtype and q.dtype in (torch.float16, torch.bfloat16, torch.float32)
+            and q.shape == k.shape == v.shape and q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
+        q_fp8, k_fp8, v_fp8 = cast_e4m3_x3_op(q, k, v)
+        return (q_fp8.reshape(batch * heads, seq_len, head_dim), k_fp8.reshape(batch * heads, seq_len, head_dim),
+                v_fp8.permute(0, 1, 3, 2).reshape(batch * heads, head_dim, seq_len))
     q_fp8 = q.to(torch.float8_e4m3fn)
     k_fp8 = k.to(torch.float8_e4m3fn)
     v = v.permute(0, 1, 3, 2)

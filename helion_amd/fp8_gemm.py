@@ -4,7 +4,7 @@ from __future__ import annotations
 
 import torch
 
-from .ops import fp8_gemm_op
+from .ops import fp8_gemm_op, fp8_quantize_op
 
 
 def fp8_gemm(x: torch.Tensor, y: torch.Tensor, *, scale_a: torch.Tensor | None = None,
@@ -20,6 +20,14 @@ def fp8_gemm_scaled(x: torch.Tensor, y: torch.Tensor, scale_a: torch.Tensor, sca
                     out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """``cast((x @ y) * scale_a * scale_b)`` — the per-tensor-scaled form torch._scaled_mm computes."""
     return fp8_gemm_op(x, y, scale_a, scale_b, out_dtype)
+
+
+def fp8_quantize_per_tensor(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """Per-tensor e4m3 quantisation for ``fp8_gemm_scaled``: returns ``(q, scale)`` with ``scale = max|x| / 448``
+    (1 for an all-zero tensor) and ``q = (x * (448 / max|x|)).to(float8_e4m3fn)``, so ``q.float() * scale ~ x``.
+    Three launches, no host synchronisation.  (The reference's example only ever passes unit scales,
+    examples/fp8_gemm.py:74-78; this is the producer of real ones.)"""
+    return fp8_quantize_op(x)
 
 
 def reference_fp8_gemm_pytorch(x_fp8: torch.Tensor, y_fp8: torch.Tensor) -> torch.Tensor:

@@ -209,3 +209,50 @@ def moe_matmul_topk_op(A: torch.Tensor, W: torch.Tensor, expert_ids: torch.Tenso
 @moe_matmul_topk_op.register_fake
 def _(A, W, expert_ids, top_k):
     return A.new_empty((A.shape[0] * top_k, W.shape[2]), dtype=torch.promote_types(A.dtype, W.dtype))
+
+
+# ------------------------------------------------------------------------------ casts / quantisation in front of the fp8 kernels
+@torch.library.custom_op("helion_amd::cast_e4m3_x3", mutates_args=())
+def cast_e4m3_x3_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Three equally sized contiguous fp16/bf16/fp32 tensors -> e4m3 (same shapes), one launch."""
+    _require_cuda(q, k, v)
+    if not (q.dtype == k.dtype == v.dtype) or q.dtype not in _DT or q.dtype == torch.float8_e4m3fn:
+        raise TypeError(f"cast_e4m3_x3 expects three float16/bfloat16/float32 tensors of one dtype, got {q.dtype}, {k.dtype}, {v.dtype}")
+    if not (q.numel() == k.numel() == v.numel()):
+        raise ValueError("cast_e4m3_x3 expects equally sized tensors")
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    outs = [torch.empty(t.shape, dtype=torch.float8_e4m3fn, device=t.device) for t in (q, k, v)]
+    lib = _lib.load()
+    rc = lib.hx_fp8_attention_preprocess(q.data_ptr(), k.data_ptr(), v.data_ptr(), outs[0].data_ptr(), outs[1].data_ptr(),
+                                         outs[2].data_ptr(), q.numel(), _DT[q.dtype], _stream_ptr(q.device))
+    _lib.check(rc, "hx_fp8_attention_preprocess")
+    return outs[0], outs[1], outs[2]
+
+
+@cast_e4m3_x3_op.register_fake
+def _(q, k, v):
+    f8 = torch.float8_e4m3fn
+    return q.new_empty(q.shape, dtype=f8), k.new_empty(k.shape, dtype=f8), v.new_empty(v.shape, dtype=f8)
+
+
+@torch.library.custom_op("helion_amd::fp8_quantize", mutates_args=())
+def fp8_quantize_op(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """(e4m3 tensor of x's shape, 0-d fp32 scale) with x ~ q * scale; scale = max|x| / 448."""
+    _require_cuda(x)
+    if x.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+        raise TypeError(f"fp8_quantize expects float16/bfloat16/float32, got {x.dtype}")
+    x = x.contiguous()
+    q = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=x.device)
+    scale = torch.empty((), dtype=torch.float32, device=x.device)
+    lib = _lib.load()
+    ws_bytes = lib.hx_fp8_quantize_workspace_bytes(x.numel())
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+    rc = lib.hx_fp8_quantize(x.data_ptr(), q.data_ptr(), x.numel(), _DT[x.dtype], scale.data_ptr(), ws.data_ptr(), ws_bytes,
+                             _stream_ptr(x.device))
+    _lib.check(rc, "hx_fp8_quantize")
+    return q, scale
+
+
+@fp8_quantize_op.register_fake
+def _(x):
+    return x.new_empty(x.shape, dtype=torch.float8_e4m3fn), x.new_empty((), dtype=torch.float32)

@@ -122,6 +122,29 @@ int hx_moe_topk_matmul(const void* A_tok, const void* W, void* C, const void* ex
                        size_t workspace_bytes, void* stream);
 size_t hx_moe_topk_workspace_bytes(int64_t T_tok, int64_t top_k, int64_t E);
 
+/* `x.to(torch.float8_e4m3fn)` on the device for fp16 / bf16 / fp32 sources, optionally times *multiplier (a device
+ * fp32, NULL = 1): dst[i] = e4m3(src[i] * m), round to nearest even, |v| <= 464 gives at most 448, larger or NaN
+ * gives NaN (what torch's cast does).  The cast of examples/fp8_attention.py:113-121.  src_dtype: HX_F16, HX_BF16,
+ * HX_F32; src and dst 16-byte aligned; any n. */
+int hx_cast_e4m3(const void* src, void* dst, int64_t n, int src_dtype, const float* multiplier, void* stream);
+
+/* The three casts of `preprocess_fp8_attention_inputs(q, k, v)` (reference: examples/fp8_attention.py:110-133) in one
+ * launch: q8, k8, v8 = e4m3(q), e4m3(k), e4m3(v), n elements each, element order unchanged.  The reference permutes v
+ * to [B,H,D,S] before its cast, which changes strides but not memory order; the caller takes the same view of v8
+ * (strides (S*D, 1, D)) and hx_fp8_attention reads it in place. */
+int hx_fp8_attention_preprocess(const void* q, const void* k, const void* v, void* q8, void* k8, void* v8, int64_t n,
+                                int src_dtype, void* stream);
+
+/* Per-tensor quantisation for the scaled GEMM (the reference's baseline call passes unit scales,
+ * examples/fp8_gemm.py:74-78; this produces real ones; no counterpart function in the reference):
+ *   amax = max|src|;  *scale_out = amax / 448 (1 if amax == 0);  dst[i] = e4m3(src[i] * (448 / amax))
+ * so that dst * scale_out ~ src and hx_fp8_gemm(..., scale_a = scale_out, ...) undoes the scaling.  A NaN in src
+ * makes the scale NaN.  scale_out: one device fp32.  workspace: hx_fp8_quantize_workspace_bytes(n) bytes, 16-byte
+ * aligned.  Three launches (partial maxima, final reduction, cast), no host synchronisation. */
+int hx_fp8_quantize(const void* src, void* dst, int64_t n, int src_dtype, float* scale_out, void* workspace,
+                    size_t workspace_bytes, void* stream);
+size_t hx_fp8_quantize_workspace_bytes(int64_t n);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,6 +23,11 @@ Pinning status (see tests/test_oracle_*.py):
 * fp8_attention             : float64 brute force (S<=32), closed-form special cases (S=1,
   uniform scores), permutation invariance, row-max-of-p == 1, a statement-by-statement walk of the
   reference kernel body with a single tile.
+* fp8_quantize_per_tensor   : the reference has no such function (it only ever passes unit scales,
+  ``examples/fp8_gemm.py:74-78``), so there is nothing of the reference's to pin it against: it is the
+  build's own definition (amax / 448 scaling), pinned by its algebraic properties (exact powers of two,
+  the amax element lands on +-448, dequantisation error within half an e4m3 step) and by the numpy
+  e4m3 encoder above.
 * moe_matmul_ogs            : the reference's own unit test skips the accuracy check
   (``test/test_examples.py:434-458``), so the *reference's tests* pin nothing here; the oracle is
   pinned by the semantic definition ``moe_matmul_ogs_reference`` (per-expert dense matmul),
@@ -219,6 +224,20 @@ def preprocess_fp8_attention_inputs(q, k, v):
 # --------------------------------------------------------------------------------------
 # moe_matmul_ogs
 # --------------------------------------------------------------------------------------
+
+
+def fp8_quantize_per_tensor(x: torch.Tensor):
+    """Definition of the per-tensor quantiser in front of the scaled GEMM (no counterpart in the reference):
+    ``amax = max|x|`` in fp32; ``scale = amax / 448`` (1 if amax == 0); ``q = e4m3(x * (448 / amax))`` with both
+    divisions and the product rounded once in fp32.  Returns ``(q, scale)`` with ``scale`` a 0-d fp32 tensor."""
+    xf = x.to(torch.float32)
+    amax = xf.abs().max() if xf.numel() else torch.zeros((), dtype=torch.float32)
+    if float(amax) == 0.0:
+        return to_e4m3(xf), torch.ones((), dtype=torch.float32)
+    c448 = torch.tensor(448.0, dtype=torch.float32)
+    scale = amax / c448
+    inv = c448 / amax
+    return to_e4m3(xf * inv), scale
 
 
 def moe_args_gen(A: torch.Tensor, W: torch.Tensor, expert_per_row: torch.Tensor):

@@ -75,3 +75,16 @@ def test_attention_and_moe_argument_errors():
     assert lib.hx_moe_topk_workspace_bytes(1000, 2, 30) >= lib.hx_moe_workspace_bytes(2000, 30) + 2000 * 4
     assert lib.hx_moe_topk_matmul(16, 16, 16, 16, 1, 8, 0, 8, 8, 2, 1, None, 0, None) == -1  # top_k < 1
     assert lib.hx_moe_topk_matmul(16, 16, 16, 16, 1, 8, 2, 8, 8, 2, 1, None, 0, None) == -3  # no workspace
+
+
+def test_cast_and_quantize_argument_errors():
+    lib = _lib.load()
+    assert lib.hx_cast_e4m3(16, 16, -1, 0, None, None) == -1
+    assert lib.hx_cast_e4m3(16, 16, 8, 3, None, None) == -1      # e4m3 is not a source type
+    assert lib.hx_cast_e4m3(None, 16, 8, 0, None, None) == -1
+    assert lib.hx_cast_e4m3(24, 16, 8, 0, None, None) == -2      # misaligned
+    assert lib.hx_cast_e4m3(None, None, 0, 0, None, None) == 0
+    assert lib.hx_fp8_attention_preprocess(16, 16, None, 16, 16, 16, 8, 1, None) == -1
+    assert lib.hx_fp8_quantize_workspace_bytes(1 << 20) >= 16 + 4
+    assert lib.hx_fp8_quantize(16, 16, 8, 0, None, 16, 1 << 20, None) == -1   # no scale_out
+    assert lib.hx_fp8_quantize(16, 16, 8, 0, 16, None, 0, None) == -3
