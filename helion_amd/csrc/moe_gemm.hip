@@ -160,8 +160,11 @@ __global__ __launch_bounds__(256) void hx_moe_tile256(const uint8_t* __restrict_
   const uint8_t* We = W + (long)mt.expert * K * N * 2 + n0 * 2 + (long)(w * 16) * N * 2;  // wave-uniform
   const int wk_l = lane >> 5, wpos = lane & 31;
   uint32_t w_vo[4];
+  // The last column tile may be ragged (N % 256 != 0, N % 8 == 0): chunks past the end re-read the last valid chunk of
+  // the row; the columns they feed are never stored.
+  const int cmax = (int)((min((long)N - n0, (long)MOE_BN) >> 3) - 1);
 #pragma unroll
-  for (int j = 0; j < 4; ++j) w_vo[j] = (uint32_t)(wk_l * N * 2 + ((wpos ^ (moe_wswz(2 * j + wk_l) << 1)) * 16));
+  for (int j = 0; j < 4; ++j) w_vo[j] = (uint32_t)(wk_l * N * 2 + min(wpos ^ (moe_wswz(2 * j + wk_l) << 1), cmax) * 16);
   const uint32_t lds0 = hx_lds_addr(&smem[0][0][0]);
 
   // DMA instruction i (0..15) of a k-tile: i < 8 -> gathered A rows 64w + 8i .., else W k-rows 16w + 2(i-8), +1
@@ -280,7 +283,8 @@ __global__ __launch_bounds__(256) void hx_moe_tile256(const uint8_t* __restrict_
             ov4 o;
 #pragma unroll
             for (int b = 0; b < 4; ++b) o[b] = (out_t)acc[bj][bi][4 * a + b];
-            *(ov4*)(crow + bj * 32 + 8 * a) = o;
+            // N % 8 == 0 and the piece starts at a multiple of 4: it is either wholly inside the row or wholly outside
+            if (n0 + wn * 128 + 4 * g + bj * 32 + 8 * a < N) *(ov4*)(crow + bj * 32 + 8 * a) = o;
           }
       }
     }
@@ -359,7 +363,7 @@ template <bool BF>
 static int launch_moe(const void* A, const void* W, void* C, const int32_t* counts, const int32_t* offsets, const int32_t* idx,
                       int64_t T, int64_t K, int64_t N, int64_t E, int64_t a_div, void* ws, hipStream_t s) {
   typedef typename Mfma16<BF>::T T16;
-  const bool fast = (K % MOE_BK == 0) && (N % MOE_BN == 0) && K >= MOE_BK && (((T + a_div - 1) / a_div) * K * 2 < (1LL << 32)) && (N * 4 < (1LL << 31)) && (((uintptr_t)A | (uintptr_t)W | (uintptr_t)C) & 15) == 0;
+  const bool fast = (K % MOE_BK == 0) && (N % 8 == 0) && K >= MOE_BK && (((T + a_div - 1) / a_div) * K * 2 < (1LL << 32)) && (N * 4 < (1LL << 31)) && (((uintptr_t)A | (uintptr_t)W | (uintptr_t)C) & 15) == 0;
   const int bm = fast ? MOE_BM : 64;
   const int max_tiles = (int)moe_max_tiles(T, E, bm);
   int* num_tiles = (int*)ws;
@@ -374,7 +378,7 @@ static int launch_moe(const void* A, const void* W, void* C, const int32_t* coun
   hipLaunchKernelGGL(hx_moe_mark, dim3(max_tiles < 1024 ? max_tiles : 1024), dim3(256), 0, s, (const int*)num_tiles,
                      (const MoeTile*)table, idx, (int)T, flags);
   if (fast) {
-    const int tiles_n = (int)(N / MOE_BN);
+    const int tiles_n = (int)((N + MOE_BN - 1) / MOE_BN);
     hipLaunchKernelGGL(hx_moe_tile256<BF>, dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W, (T16*)C,
                        (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, max_tiles, tiles_n, (int)a_div);
   } else {

@@ -28,6 +28,10 @@ def _run(A, W, ex):
     (2048, 512, 768, 8, 2, torch.bfloat16),    # top-2 expanded rows
     (300, 64, 256, 16, 1, torch.bfloat16),     # most tiles nearly empty
     (37, 100, 19, 3, 1, torch.bfloat16),
+    (512, 128, 384, 4, 1, torch.bfloat16),     # tile256 kernel, ragged last column tile (N % 256 = 128)
+    (600, 64, 1408, 8, 2, torch.float16),      # N = 5.5 tiles
+    (256, 64, 8, 2, 1, torch.bfloat16),        # a single column tile with one valid 16-byte chunk
+    (300, 192, 200, 5, 1, torch.bfloat16),     # N % 8 == 0, nothing else aligned
 ])
 def test_shapes_vs_oracle(T, K, N, E, topk, dtype):
     A, W, ex = inputs.moe_inputs(T // topk, K, N, E, topk, seed=T + K, dtype=dtype)
