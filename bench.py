@@ -1,13 +1,14 @@
 #!/usr/bin/env python3
 """Benchmark of the hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only c2,c3,c4,c5] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only c2,c3,c4,c5,next] [--no-cpu-baseline]
 
 The defaults (40 warm-up + 100 timed launches) are long enough for the GPU's clocks to settle under load; a
 handful of launches reads ~15 % low.  A "step" is one launch of the FP8 GEMM at the headline configuration (M=N=K=8192, e4m3 operands,
 B column-major, per-tensor fp32 scales, bf16 output) with inputs resident in HBM.  The JSON line also
 carries the other three configurations (decode-shape GEMM, FP8 attention, MoE grouped GEMM) under
-"other_workloads", each with its own roofline object, and the ref-eager CPU path (ATen's CPU
+"other_workloads" together with the kernels either side of them (casts, quantisation, routing), each with its own roofline
+object, and the ref-eager CPU path (ATen's CPU
 torch._scaled_mm on the 1024^3 configuration) under "cpu_baseline".
 """
 from __future__ import annotations
@@ -147,6 +148,46 @@ def bench_c5(steps, warmup):
     }
 
 
+def bench_next_rows(steps, warmup):
+    """The kernels either side of the three hot kernels (routing tables, top-k entry, casts, quantisation), each against the
+    HBM roofline of its algorithmic bytes.  Launch-latency-sized kernels are reported in microseconds as well."""
+    import torch
+    import helion_amd as hx
+    from helion_amd import inputs
+
+    out = {}
+    n_it, n_w = min(steps, 50), min(warmup, 20)
+
+    def hbm(nbytes, ms, kernel, workload):
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        return {"workload": workload, "ms_per_launch": ms, "value": gbs, "unit": "GB/s",
+                "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
+                             "traffic": None, "kernel": kernel, "avg_launch_ms": ms, "algorithmic_bytes_per_launch": float(nbytes)}}
+
+    # preprocessing casts at the C4 shape: 3 x (fp16 in + e4m3 out)
+    q, k, v = (torch.randn(4, 32, 4096, 128, device="cuda").to(torch.float16) for _ in range(3))
+    ms, _ = _time_launches(lambda: hx.preprocess_fp8_attention_inputs(q, k, v), n_it, n_w)
+    out["attention_preprocess_cast"] = hbm(3 * q.numel() * 3, ms, "hx_cast_e4m3_kernel<f16> x3 in one launch",
+                                           "preprocess_fp8_attention_inputs at C4 shape, fp16 -> e4m3, 3 x 67M elements")
+    del q, k, v
+    # per-tensor quantisation of a bf16 8192^2 operand: read for amax, read again + write e4m3
+    x = torch.randn(8192, 8192, device="cuda", dtype=torch.bfloat16)
+    ms, _ = _time_launches(lambda: hx.fp8_quantize_per_tensor(x), n_it, n_w)
+    out["fp8_quantize_per_tensor"] = hbm(x.numel() * 5, ms, "hx_amax_partial + hx_amax_final + hx_cast_e4m3_kernel<bf16>",
+                                         "amax -> scale -> e4m3 of a bf16 8192x8192 operand (bytes: 2 reads + 1 write)")
+    del x
+    # routing tables at the C5 row count and at 1M rows
+    _, _, ex = inputs.moe_c5("cuda")
+    ms, _ = _time_launches(lambda: hx.moe_routing(ex, 8), n_it, n_w)
+    out["moe_routing_c5"] = hbm(ex.numel() * (8 + 8 + 4), ms, "hx_moe_routing_kernel<int64, one workgroup>",
+                                "stable sort/count/scan of 32768 int64 expert ids, E=8 (launch-latency sized: see ms_per_launch)")
+    big = ex.repeat(32)
+    ms, _ = _time_launches(lambda: hx.moe_routing(big, 8), n_it, n_w)
+    out["moe_routing_1m"] = hbm(big.numel() * (8 + 8 + 4), ms, "hx_moe_routing_kernel count + scan + scatter",
+                                "the same for 1048576 rows (three launches)")
+    return out
+
+
 def cpu_baseline():
     """The reference's ref-eager CPU path for fp8_gemm (ATen CPU torch._scaled_mm, unit scales, fp32
     accumulate, bf16 result) on the 1024^3 configuration, repeated for about 10 s of CPU time."""
@@ -175,7 +216,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=40)
-    ap.add_argument("--only", default="c2,c3,c4,c5")
+    ap.add_argument("--only", default="c2,c3,c4,c5,next")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run three plain 1 GiB device copies (a known-traffic kernel to scale rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE by)")
@@ -208,6 +249,9 @@ def main():
         torch.cuda.empty_cache()
     if "c5" in only:
         others["c5_moe_grouped_gemm"] = bench_c5(args.steps, args.warmup)
+        torch.cuda.empty_cache()
+    if "next" in only:
+        others.update(bench_next_rows(args.steps, args.warmup))
         torch.cuda.empty_cache()
     line = {
         "metric": "FP8 GEMM/attention TFLOP/s + % of MI355X FP8 MFMA peak (or % HBM BW), 1 GPU",
