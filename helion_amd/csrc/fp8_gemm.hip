@@ -28,7 +28,12 @@
 
 // EDGE: M and/or N are not multiples of 256.  Rows past the end are clamped to the last row on load (their
 // products land in accumulators that are never stored) and the stores are guarded.
-template <int OUT, bool EDGE>
+// BROW: B is row-major ([K][N], N contiguous; `Bt`/`ldb` are then B itself and its row stride).  The B tile sits in
+// LDS as [128 k][256 B of n], chunk stored at pos = chunk ^ ((k&7)<<1), and the MFMA operand (32 consecutive k of one
+// column per lane) is formed by four transposing reads (ds_read_b64_tr_b8: 8 k x 16 n per 16 lanes) instead of two
+// 16-byte reads; one DMA instruction moves 4 k-rows x 256 B.  N must be a multiple of 16; with EDGE, chunks past
+// the end re-read the row's last valid chunk.
+template <int OUT, bool EDGE, bool BROW>
 __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __restrict__ A, const uint8_t* __restrict__ Bt,
                                                           typename OutT<OUT>::T* __restrict__ C, int M, int N, int K, long lda,
                                                           long ldb, long ldc, const float* __restrict__ scale_a,
@@ -64,17 +69,27 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
   const int lrow = lane >> 3, lpos = lane & 7;
   const uint32_t a_vo0 = (uint32_t)(lrow * lda + (lpos ^ ((lrow >> 1) & 7)) * 16);        // j even
   const uint32_t a_vo1 = (uint32_t)(lrow * lda + (lpos ^ ((4 + (lrow >> 1)) & 7)) * 16);  // j odd
-  const uint32_t b_vo0 = (uint32_t)(lrow * ldb + (lpos ^ ((lrow >> 1) & 7)) * 16);
-  const uint32_t b_vo1 = (uint32_t)(lrow * ldb + (lpos ^ ((4 + (lrow >> 1)) & 7)) * 16);
-  const uint8_t* gA = A + (m0 + w * 64) * lda;   // wave-uniform
-  const uint8_t* gB = Bt + (n0 + w * 64) * ldb;  // wave-uniform
+  // row-major B: wave w owns k rows [32w, 32w+32) of the k-tile; instruction j covers rows 32w+4j .. +3, 16 chunks each
+  const int brow = lane >> 4, bpos = lane & 15;
+  const int bcmax = BROW ? (int)((min((long)N - n0, (long)T256_BN) >> 4) - 1) : 0;  // last valid chunk of this tile's rows
+  auto brow_vo = [&](int kodd) {  // kodd: (row within the 8-row swizzle period) >= 4, i.e. j odd
+    int chunk = bpos ^ (((4 * kodd + brow) & 7) << 1);
+    if (EDGE) chunk = min(chunk, bcmax);
+    return (uint32_t)(brow * ldb + chunk * 16);
+  };
+  const uint32_t b_vo0 = BROW ? brow_vo(0) : (uint32_t)(lrow * ldb + (lpos ^ ((lrow >> 1) & 7)) * 16);
+  const uint32_t b_vo1 = BROW ? brow_vo(1) : (uint32_t)(lrow * ldb + (lpos ^ ((4 + (lrow >> 1)) & 7)) * 16);
+  const uint8_t* gA = A + (m0 + w * 64) * lda;                                  // wave-uniform
+  const uint8_t* gB = BROW ? Bt + (long)(w * 32) * ldb + n0 : Bt + (n0 + w * 64) * ldb;  // wave-uniform
   const uint32_t lds0 = hx_lds_addr(&smem[0][0][0]) + (uint32_t)w * 64 * 128;
 
   // DMA instruction i (0..15) of a k-tile: i < 8 -> A rows 64w + 8i .., else B rows 64w + 8(i-8) ..
   auto issue_one = [&](int kt, int stage, int i) {
     const long kb = (long)kt * T256_BK;
     const uint32_t la = lds0 + (uint32_t)stage * 2 * T256_TILE_BYTES, lb = la + T256_TILE_BYTES;
-    if (!EDGE) {
+    if (BROW && i >= 8) {  // 4 k-rows x 256 B; column clamping (EDGE) is already in the per-lane offsets
+      hx_g2l16_s(gB + (kb + (long)(i - 8) * 4) * ldb, (i & 1) ? b_vo1 : b_vo0, lb + (i - 8) * 1024);
+    } else if (!EDGE) {
       if (i < 8) hx_g2l16_s(gA + (long)i * 8 * lda + kb, (i & 1) ? a_vo1 : a_vo0, la + i * 1024);
       else hx_g2l16_s(gB + (long)(i - 8) * 8 * ldb + kb, (i & 1) ? b_vo1 : b_vo0, lb + (i - 8) * 1024);
     } else {  // per-lane clamped row; the whole matrix is below 4 GB (checked by the host), so the offset fits 32 bits
@@ -98,6 +113,10 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
   const int x = ((g * 2) ^ ((r31 >> 1) & 7)) * 16;
   const int a_base = (wm * 128 + r31) * 128;
   const int b_base = (wn * 128 + r31) * 128;
+  // row-major B: transposing read j (0..3) of column block bj, k-step t fetches k = 64t + 32g + 8j .. +7; this lane
+  // supplies 8 bytes of row (that k) + (lane%16)/2, columns 16*((lane>>4)&1) + 8*(lane&1) .. +7 of the block and
+  // receives column lane%32.  Block bj / wave column wn add to chunk bits the swizzle's xor commutes with.
+  const int bt_off = (32 * g + ((lane & 15) >> 1)) * 256 + (((((lane >> 4) & 1)) ^ (((lane & 15) >> 1) << 1)) * 16) + (lane & 1) * 8;
 
   v16f acc[4][4];  // [bj][bi]: rows = n (B side), cols = m (A side)
 #pragma unroll
@@ -109,6 +128,18 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
 
   // fragment f (0..7) of the 64-byte k-step t of a stage: f < 4 -> A rows 32f.. of this wave, else B rows 32(f-4)..
   auto load_frag = [&](v8i(&af)[4], v8i(&bf)[4], int stage, int t, int f) {
+    if (BROW && f >= 4) {
+      const uint8_t* sb = &smem[stage][1][0] + (bt_off ^ ((wn * 8 + (f - 4) * 2) * 16)) + t * 16384;
+      v8i v;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const v2i part = __builtin_amdgcn_ds_read_tr8_b64_v2i32((v2i __attribute__((address_space(3)))*)(sb + j * 2048));
+        v[2 * j] = part[0];
+        v[2 * j + 1] = part[1];
+      }
+      bf[f - 4] = v;
+      return;
+    }
     const uint8_t* base = (f < 4) ? &smem[stage][0][0] + a_base + f * 4096 : &smem[stage][1][0] + b_base + (f - 4) * 4096;
     v4i lo = *(const v4i*)(base + (x ^ (t * 64)));
     v4i hi = *(const v4i*)(base + (x ^ (t * 64 + 16)));
@@ -512,9 +543,16 @@ static int gemm_path_kmajor(int64_t M, int64_t N, int64_t K, int64_t lda, int64_
   return 0;
 }
 
+// row-major B (N contiguous) on the tile kernel's transposing-read mode
+static bool gemm_path_rowmajor_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, const void* a, const void* b) {
+  return M > 16 && (lda % 16 == 0) && (ldb_k % 16 == 0) && (K % 128 == 0) && K >= 128 && (N % 16 == 0) && ldb_k >= N && aligned(a, 16) &&
+         aligned(b, 16) && lda < (1LL << 27) && ldb_k < (1LL << 27) && M * lda < (1LL << 32);
+}
+
 extern "C" int hx_fp8_gemm_path(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
                                 const void* a, const void* b, const void* c) {
   if (ldb_k == 1) return gemm_path_kmajor(M, N, K, lda, ldb_n, ldc, a, b, c);
+  if (ldb_n == 1 && gemm_path_rowmajor_ok(M, N, K, lda, ldb_k, a, b)) return 4;
   return 0;
 }
 
@@ -522,14 +560,25 @@ template <int OUT>
 static void launch_kmajor(int path, const void* a, const void* bt, void* c, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                           int64_t ldc, const float* sa, const float* sb, hipStream_t stream) {
   typedef typename OutT<OUT>::T out_t;
-  if (path == 1 || path == 3) {
+  if (path == 4) {  // row-major B; ldb is its row stride
     const int tiles_m = (int)((M + 255) / 256), tiles_n = (int)((N + 255) / 256);
-    if (path == 1)
-      hipLaunchKernelGGL((hx_fp8_gemm_tile256<OUT, false>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
+    const bool edge = (M % 256 != 0) || (N % 256 != 0) || (ldc % 8 != 0) || !aligned(c, 16);
+    if (!edge)
+      hipLaunchKernelGGL((hx_fp8_gemm_tile256<OUT, false, true>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
                          (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m,
                          tiles_n);
     else
-      hipLaunchKernelGGL((hx_fp8_gemm_tile256<OUT, true>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
+      hipLaunchKernelGGL((hx_fp8_gemm_tile256<OUT, true, true>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
+                         (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m,
+                         tiles_n);
+  } else if (path == 1 || path == 3) {
+    const int tiles_m = (int)((M + 255) / 256), tiles_n = (int)((N + 255) / 256);
+    if (path == 1)
+      hipLaunchKernelGGL((hx_fp8_gemm_tile256<OUT, false, false>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
+                         (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m,
+                         tiles_n);
+    else
+      hipLaunchKernelGGL((hx_fp8_gemm_tile256<OUT, true, false>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
                          (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m,
                          tiles_n);
   } else {  // path == 2
@@ -557,7 +606,7 @@ static int launch_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int
   typedef typename OutT<OUT>::T out_t;
   int path = hx_fp8_gemm_path(M, N, K, lda, ldb_k, ldb_n, ldc, a, b, c);
   if (path != 0) {
-    launch_kmajor<OUT>(path, a, b, c, M, N, K, lda, ldb_n, ldc, sa, sb, stream);
+    launch_kmajor<OUT>(path, a, b, c, M, N, K, lda, path == 4 ? ldb_k : ldb_n, ldc, sa, sb, stream);
   } else {
     // row-major B with a workspace: transpose it once into K-contiguous form, then take a fast path
     int tpath = 0;
@@ -582,8 +631,11 @@ static int launch_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int
 }
 
 extern "C" size_t hx_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t ldb_k, int64_t ldb_n) {
-  // only a row-major B (N contiguous) that could take a fast path after a transpose needs scratch: N*K bytes
+  // Only a row-major B (N contiguous) that the tile kernel cannot read in place (M <= 16: the skinny kernel wants K
+  // contiguous; N or the row stride not a multiple of 16) but that could take a fast path after a transpose needs
+  // scratch: N*K bytes.
   if (M <= 0 || N <= 0 || K <= 0 || ldb_k == 1 || ldb_n != 1 || K % 128 != 0) return 0;
+  if (M > 16 && N % 16 == 0 && ldb_k % 16 == 0) return 0;
   return (size_t)(N * K);
 }
 

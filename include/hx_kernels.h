@@ -49,18 +49,21 @@ const char* hx_last_error(void);
  * c: [M,N] of out_dtype (HX_F16 = reference default, HX_BF16, HX_F32), element (m,n) at c[m*ldc+n].
  * scale_a/scale_b: device pointers to one fp32 each, or NULL for 1.0 (the reference hard-codes
  *    1.0, helion/language/matmul_ops.py:232-233).
- * Chooses between the 256x256 MFMA tile kernel (with guarded edge tiles when M or N is ragged), the skinny
- * (M<=16) wave-split-K kernel and a bounds-checked general kernel from the shape, strides and alignment.
+ * Chooses between the 256x256 MFMA tile kernel (with guarded edge tiles when M or N is ragged; it reads a
+ * column-major B directly and a row-major B through transposing LDS loads), the skinny (M<=16) wave-split-K kernel
+ * and a bounds-checked general kernel from the shape, strides and alignment.
  * workspace: optional device scratch of hx_fp8_gemm_workspace_bytes(...) bytes, 16-byte aligned. */
 int hx_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int64_t lda,
                 int64_t ldb_k, int64_t ldb_n, int64_t ldc, const float* scale_a, const float* scale_b,
                 int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
-/* Scratch hx_fp8_gemm can use for these arguments (0 unless B is row-major: then N*K bytes for a one-off
- * transpose into the K-contiguous layout; without it a row-major B runs on the slow general kernel). */
+/* Scratch hx_fp8_gemm can use for these arguments: 0 unless B is row-major AND the tile kernel cannot read it in
+ * place (M <= 16, or N / the row stride not a multiple of 16); then N*K bytes for a one-off transpose into the
+ * K-contiguous layout, without which such a B runs on the slow general kernel. */
 size_t hx_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t ldb_k, int64_t ldb_n);
 
-/* Which kernel hx_fp8_gemm would launch for these arguments: 0 general, 1 tile256, 2 skinny, 3 tile256 with
- * guarded edge tiles (M or N not a multiple of 256).
+/* Which kernel hx_fp8_gemm would launch for these arguments: 0 general (or, given a workspace, transpose + fast
+ * path), 1 tile256, 2 skinny, 3 tile256 with guarded edge tiles (M or N not a multiple of 256), 4 tile256 reading a
+ * row-major B in place (edges included).
  * (Diagnostic; lets tests assert that the fast paths are the ones exercised.) */
 int hx_fp8_gemm_path(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n,
                      int64_t ldc, const void* a, const void* b, const void* c);

@@ -47,10 +47,13 @@ def test_gemm_path_selection():
     assert lib.hx_fp8_gemm_path(8192, 8192, 8192, 8192, 1, 8192, 8192, A, A, A) == 1
     assert lib.hx_fp8_gemm_path(16, 28672, 8192, 8192, 1, 8192, 28672, A, A, A) == 2
     assert lib.hx_fp8_gemm_path(1, 512, 256, 256, 1, 256, 512, A, A, A) == 2
-    assert lib.hx_fp8_gemm_path(256, 256, 256, 256, 256, 1, 256, A, A, A) == 0  # row-major B
+    assert lib.hx_fp8_gemm_path(256, 256, 256, 256, 256, 1, 256, A, A, A) == 4  # row-major B, read in place
+    assert lib.hx_fp8_gemm_path(16, 256, 256, 256, 256, 1, 256, A, A, A) == 0   # row-major B for the skinny shape: via workspace
+    assert lib.hx_fp8_gemm_path(100, 72, 128, 128, 72, 1, 72, A, A, A) == 0     # row-major B, N % 16 != 0
     assert lib.hx_fp8_gemm_path(100, 70, 50, 50, 1, 50, 70, A, A, A) == 0  # ragged K
     assert lib.hx_fp8_gemm_path(1000, 1000, 1024, 1024, 1, 1024, 1000, A, A, A) == 3  # ragged M/N: guarded edge tiles
-    assert lib.hx_fp8_gemm_workspace_bytes(256, 512, 384, 512, 1) == 512 * 384  # row-major B: transpose scratch
+    assert lib.hx_fp8_gemm_workspace_bytes(256, 512, 384, 512, 1) == 0          # row-major B the tile kernel reads in place
+    assert lib.hx_fp8_gemm_workspace_bytes(8, 512, 384, 512, 1) == 512 * 384    # skinny shape: transpose scratch
     assert lib.hx_fp8_gemm_workspace_bytes(256, 512, 384, 1, 384) == 0
     assert lib.hx_fp8_gemm_path(256, 256, 256, 256, 1, 256, 256, A + 1, A, A) == 0  # misaligned
 

@@ -38,19 +38,41 @@ def test_shapes_vs_oracle(m, n, k, path, out_dtype):
     assert rel_err(out, ref) <= (1e-2 if out_dtype != torch.float32 else 1e-4)
 
 
-@pytest.mark.parametrize("m,k,n", [(256, 384, 512), (300, 256, 200), (16, 1024, 512), (64, 100, 48)])
-def test_row_major_b_goes_through_the_transpose_workspace(m, k, n):
+@pytest.mark.parametrize("m,k,n,path,ws", [
+    (256, 384, 512, 4, 0),            # tile kernel reads the row-major B in place (transposing LDS loads)
+    (512, 1024, 768, 4, 0),
+    (300, 256, 208, 4, 0),            # ragged M and N (N % 16 == 0): clamped chunks, guarded stores
+    (1000, 512, 1008, 4, 0),
+    (17, 128, 16, 4, 0),              # one valid 16-byte chunk per row
+    (300, 256, 200, 0, 200 * 256),    # N % 16 != 0: transposed into the workspace, then the edge-tile kernel
+    (16, 1024, 512, 0, 512 * 1024),   # skinny shape: transposed, then the skinny kernel
+    (64, 100, 48, 0, 0),              # K % 128 != 0: general kernel
+])
+def test_row_major_b(m, k, n, path, ws):
     g = torch.Generator().manual_seed(m + n)
     x = torch.randn(m, k, generator=g).to(E4M3); y = torch.randn(k, n, generator=g).to(E4M3)  # y row-major
     lib = _lib.load()
-    want = n * k if k % 128 == 0 else 0
-    assert lib.hx_fp8_gemm_workspace_bytes(m, n, k, n, 1) == want
-    out = hx.fp8_gemm(x.to(DEV), y.to(DEV), out_dtype=torch.float32)
-    assert rel_err(out, orc.fp8_gemm(x, y, out_dtype=torch.float32)) <= 1e-4
+    xd, yd = x.to(DEV), y.to(DEV)
+    assert lib.hx_fp8_gemm_path(m, n, k, k, n, 1, n, xd.data_ptr(), yd.data_ptr(), xd.data_ptr()) == path
+    assert lib.hx_fp8_gemm_workspace_bytes(m, n, k, n, 1) == ws
+    for od, tol in ((torch.float32, 1e-4), (torch.bfloat16, 1e-2)):
+        out = hx.fp8_gemm(xd, yd, out_dtype=od)
+        assert rel_err(out, orc.fp8_gemm(x, y, out_dtype=od)) <= tol
+    # the same arithmetic as the column-major path: identical bits
+    assert torch.equal(hx.fp8_gemm(xd, yd, out_dtype=torch.float32), hx.fp8_gemm(xd, yd.T.contiguous().T, out_dtype=torch.float32))
     # a strided (non-compact) row-major view works too
     ybig = torch.randn(k, n + 16, generator=g).to(E4M3)
-    out2 = hx.fp8_gemm(x.to(DEV), ybig.to(DEV)[:, :n], out_dtype=torch.float32)
+    out2 = hx.fp8_gemm(xd, ybig.to(DEV)[:, :n], out_dtype=torch.float32)
     assert rel_err(out2, orc.fp8_gemm(x, ybig[:, :n].contiguous(), out_dtype=torch.float32)) <= 1e-4
+
+
+def test_row_major_b_at_benchmark_size_matches_column_major():
+    a, b, sa, sb = inputs.gemm_c2(DEV)
+    b_row = b.contiguous()                       # [K, N] row-major copy of the column-major operand
+    assert b_row.stride() == (8192, 1) and b.stride() == (1, 8192)
+    out_col = hx.fp8_gemm(a, b, scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16)
+    out_row = hx.fp8_gemm(a, b_row, scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16)
+    assert torch.equal(out_col, out_row)
 
 
 def test_reference_call_form_and_defaults():
