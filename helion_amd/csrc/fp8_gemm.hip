@@ -4,7 +4,7 @@
 // Three kernels:
 //   hx_fp8_gemm_tile256 : 256x256x128 workgroup tile, 4 waves (2x2) of 128x128, 32x32x64 fp8 MFMA,
 //                         A/B k-tiles DMA'd global->LDS (double buffered, XOR-swizzled 16B chunks).
-//   hx_fp8_gemm_skinny_direct : M <= 16, K <= 8192; HBM-bound streaming of B^T through registers into
+//   hx_fp8_gemm_skinny_direct : M <= 32, K <= 8192; HBM-bound streaming of B^T through registers into
 //                         16x16x128 MFMA, K split across the 8 waves of a workgroup, partials summed in LDS.
 //   hx_fp8_gemm_skinny  : M <= 16, larger K; same split, A panel staged through LDS in 8 KB chunks of K.
 //   hx_fp8_gemm_general : bounds-checked, arbitrary strides (fallback for ragged/unaligned inputs).
@@ -387,13 +387,15 @@ __global__ __launch_bounds__(512) void hx_fp8_gemm_skinny(const uint8_t* __restr
 // also across the barrier that sums the eight wave partials.
 // ------------------------------------------------------------------------------------------
 #define SKD_MAXS 8
-template <int OUT, bool FULL>  // FULL: K == 8192, every wave owns exactly 8 k-steps (no per-step predicates)
+// FULL: K == 8192, every wave owns exactly 8 k-steps (no per-step predicates).  MB: 16-row blocks of A (M <= 16*MB);
+// every block reuses the B fragment a wave has just assembled, so rows beyond 16 cost MFMAs but no extra traffic.
+template <int OUT, bool FULL, int MB>
 __global__ __launch_bounds__(512) void hx_fp8_gemm_skinny_direct(const uint8_t* __restrict__ A, const uint8_t* __restrict__ Bt,
                                                                 typename OutT<OUT>::T* __restrict__ C, int M, int N, int K,
                                                                 long lda, long ldb, long ldc, const float* __restrict__ scale_a,
                                                                 const float* __restrict__ scale_b) {
   typedef typename OutT<OUT>::T out_t;
-  __shared__ __attribute__((aligned(16))) float red[2][SK_WAVES][4][64];  // [parity][wave][r][lane]
+  __shared__ __attribute__((aligned(16))) float red[2][SK_WAVES][MB * 4][64];  // [parity][wave][4*mb + r][lane]
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -425,16 +427,17 @@ __global__ __launch_bounds__(512) void hx_fp8_gemm_skinny_direct(const uint8_t* 
       if (FULL || s < nmine) load_step(s);
   }
 
-  // ---- A fragments: lane (m = j, g) holds A[m][128*(w + 8s) + 32g .. +31]
-  v8i af[SKD_MAXS];
-  {
-    const uint8_t* ap = A + (long)min(j, M - 1) * lda + g * 32 + (long)w * 128;
+  // ---- A fragments: lane (m = 16*mb + j, g) holds A[m][128*(w + 8s) + 32g .. +31]
+  v8i af[MB][SKD_MAXS];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const uint8_t* ap = A + (long)min(mb * 16 + j, M - 1) * lda + g * 32 + (long)w * 128;
 #pragma unroll
     for (int s = 0; s < SKD_MAXS; ++s)
       if (FULL || s < nmine) {
         const v4i* p = (const v4i*)(ap + (long)s * SK_WAVES * 128);
         v4i lo = p[0], hi = p[1];
-        af[s] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        af[mb][s] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
       }
   }
   float alpha = 1.f;
@@ -445,7 +448,9 @@ __global__ __launch_bounds__(512) void hx_fp8_gemm_skinny_direct(const uint8_t* 
   for (int gi = 0; gi < my_groups; ++gi) {
     const bool more = gi + 1 < my_groups;
     if (more) point_at(gi + 1);
-    v4f acc = {0.f, 0.f, 0.f, 0.f};
+    v4f acc[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb] = (v4f){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < SKD_MAXS; ++s)
       if (FULL || s < nmine) {
@@ -458,20 +463,23 @@ __global__ __launch_bounds__(512) void hx_fp8_gemm_skinny_direct(const uint8_t* 
           bf[4 + d] = __builtin_amdgcn_mov_dpp(send, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]: lane ^ 1
         }
         if (more) load_step(s);  // the registers just consumed take this k-step of the next column group
-        acc = hx_mfma_16x16x128_e4m3(af[s], bf, acc);
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[mb] = hx_mfma_16x16x128_e4m3(af[mb][s], bf, acc[mb]);
       }
-    // ---- sum the 8 wave partials: acc[r] is C[4g + r][column of lane j = cg*16 + (j>>1) + 8*(j&1)]
+    // ---- sum the 8 wave partials: acc[mb][r] is C[16mb + 4g + r][column of lane j = cg*16 + (j>>1) + 8*(j&1)]
     const int cg = blockIdx.x + gi * gridDim.x;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) red[parity][w][r][lane] = acc[r];
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[parity][w][4 * mb + r][lane] = acc[mb][r];
     __syncthreads();
-    if (tid < 256) {
-      const int l2 = tid & 63, r = tid >> 6;
+    if (tid < 256 * MB) {  // MB <= 2: 512 threads cover 16*MB rows x 16 columns
+      const int l2 = tid & 63, rr = tid >> 6;  // rr = 4*mb + r
       float sum = 0.f;
 #pragma unroll
-      for (int ww = 0; ww < SK_WAVES; ++ww) sum += red[parity][ww][r][l2];
+      for (int ww = 0; ww < SK_WAVES; ++ww) sum += red[parity][ww][rr][l2];
       const int j2 = l2 & 15;
-      const int m = 4 * (l2 >> 4) + r, n = cg * 16 + (j2 >> 1) + 8 * (j2 & 1);
+      const int m = 16 * (rr >> 2) + 4 * (l2 >> 4) + (rr & 3), n = cg * 16 + (j2 >> 1) + 8 * (j2 & 1);
       if (m < M && n < N) C[(long)m * ldc + n] = (out_t)(sum * alpha);
     }
     parity ^= 1;  // the next group writes the other buffer, so one barrier per group is enough
@@ -536,7 +544,7 @@ static int gemm_path_kmajor(int64_t M, int64_t N, int64_t K, int64_t lda, int64_
                             const void* c) {
   const bool ok = (lda % 16 == 0) && (ldb % 16 == 0) && (K % 128 == 0) && aligned(a, 16) && aligned(b, 16) && K >= 128;
   if (!ok) return 0;
-  if (M <= 16 && lda >= K && ldb >= K) return 2;
+  if ((M <= 16 || (M <= 32 && K <= 8192)) && lda >= K && ldb >= K) return 2;
   if (lda >= (1LL << 27) || ldb >= (1LL << 27)) return 0;
   if ((M % 256 == 0) && (N % 256 == 0) && (ldc % 8 == 0) && aligned(c, 16)) return 1;  // 16-byte row-aligned stores
   if (M * lda < (1LL << 32) && N * ldb < (1LL << 32)) return 3;
@@ -587,11 +595,17 @@ static void launch_kmajor(int path, const void* a, const void* bt, void* c, int6
     (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     const int ncg = (int)((N + 15) / 16);
     const int grid = ncg < cus ? ncg : cus;
-    if (K == 8192)
-      hipLaunchKernelGGL((hx_fp8_gemm_skinny_direct<OUT, true>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
+    if (K == 8192 && M <= 16)
+      hipLaunchKernelGGL((hx_fp8_gemm_skinny_direct<OUT, true, 1>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
+                         (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb);
+    else if (K == 8192)
+      hipLaunchKernelGGL((hx_fp8_gemm_skinny_direct<OUT, true, 2>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
+                         (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb);
+    else if (K < 8192 && M <= 16)
+      hipLaunchKernelGGL((hx_fp8_gemm_skinny_direct<OUT, false, 1>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
                          (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb);
     else if (K < 8192)
-      hipLaunchKernelGGL((hx_fp8_gemm_skinny_direct<OUT, false>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
+      hipLaunchKernelGGL((hx_fp8_gemm_skinny_direct<OUT, false, 2>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
                          (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb);
     else
       hipLaunchKernelGGL(hx_fp8_gemm_skinny<OUT>, dim3(grid), dim3(512), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,

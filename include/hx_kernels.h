@@ -50,7 +50,7 @@ const char* hx_last_error(void);
  * scale_a/scale_b: device pointers to one fp32 each, or NULL for 1.0 (the reference hard-codes
  *    1.0, helion/language/matmul_ops.py:232-233).
  * Chooses between the 256x256 MFMA tile kernel (with guarded edge tiles when M or N is ragged; it reads a
- * column-major B directly and a row-major B through transposing LDS loads), the skinny (M<=16) wave-split-K kernel
+ * column-major B directly and a row-major B through transposing LDS loads), the skinny (M<=16, or M<=32 with K<=8192) wave-split-K kernel
  * and a bounds-checked general kernel from the shape, strides and alignment.
  * workspace: optional device scratch of hx_fp8_gemm_workspace_bytes(...) bytes, 16-byte aligned. */
 int hx_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int64_t lda,

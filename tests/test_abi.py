@@ -47,6 +47,8 @@ def test_gemm_path_selection():
     assert lib.hx_fp8_gemm_path(8192, 8192, 8192, 8192, 1, 8192, 8192, A, A, A) == 1
     assert lib.hx_fp8_gemm_path(16, 28672, 8192, 8192, 1, 8192, 28672, A, A, A) == 2
     assert lib.hx_fp8_gemm_path(1, 512, 256, 256, 1, 256, 512, A, A, A) == 2
+    assert lib.hx_fp8_gemm_path(32, 28672, 8192, 8192, 1, 8192, 28672, A, A, A) == 2   # up to 32 rows when K <= 8192
+    assert lib.hx_fp8_gemm_path(33, 28672, 8192, 8192, 1, 8192, 28672, A, A, A) == 3
     assert lib.hx_fp8_gemm_path(256, 256, 256, 256, 256, 1, 256, A, A, A) == 4  # row-major B, read in place
     assert lib.hx_fp8_gemm_path(16, 256, 256, 256, 256, 1, 256, A, A, A) == 0   # row-major B for the skinny shape: via workspace
     assert lib.hx_fp8_gemm_path(100, 72, 128, 128, 72, 1, 72, A, A, A) == 0     # row-major B, N % 16 != 0

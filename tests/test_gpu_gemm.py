@@ -25,7 +25,8 @@ def _path(m, n, k):
 @pytest.mark.parametrize("m,n,k,path", [
     (256, 256, 256, 1), (512, 512, 512, 1), (1024, 1024, 1024, 1), (256, 768, 128, 1), (768, 256, 1152, 1),
     (16, 512, 1024, 2), (1, 16, 128, 2), (5, 48, 256, 2), (16, 1000, 384, 2), (9, 33, 8192 + 128, 2), (16, 64, 16384, 2),
-    (1000, 1000, 1024, 3), (300, 200, 256, 3), (257, 255, 128, 3), (17, 256, 256, 3), (255, 1, 128, 3),
+    (17, 256, 256, 2), (32, 512, 8192, 2), (24, 100, 1152, 2), (31, 33, 384, 2),        # two 16-row blocks on the skinny kernel
+    (1000, 1000, 1024, 3), (300, 200, 256, 3), (257, 255, 128, 3), (33, 256, 256, 3), (32, 64, 8192 + 128, 3), (255, 1, 128, 3),
     (100, 70, 50, 0), (256, 256, 200, 0), (3, 5, 7, 0), (64, 64, 0, 0),
 ])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16, torch.float32])
