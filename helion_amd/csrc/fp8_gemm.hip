@@ -201,11 +201,12 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
   constexpr int RSTR = ROWB + (ESZ == 2 ? 8 : 16);  // padded row stride: conflict-free 8/16-byte writes down a column
   constexpr int LPR = ROWB / 16;                    // lanes per row when reading back 16 bytes per lane
   constexpr int RPI = 64 / LPR;                     // rows per store instruction
-  uint8_t* st = &smem[0][0][0] + w * T256_TILE_BYTES;  // this wave's 32 KB
+  constexpr int NBUF = (2 * 32 * RSTR <= T256_TILE_BYTES) ? 2 : 1;  // 16-bit outputs: two staging blocks per wave
+  uint8_t* st = &smem[0][0][0] + w * T256_TILE_BYTES;               // this wave's 32 KB
   typedef out_t ov4 __attribute__((ext_vector_type(4)));
   const int rb_row = lane / LPR, rb_ch = lane % LPR;
-#pragma unroll
-  for (int bi = 0; bi < 4; ++bi) {
+  auto stage = [&](int bi) {  // accumulators of row group bi -> staging block bi % NBUF
+    uint8_t* sb = st + (bi % NBUF) * (32 * RSTR);
 #pragma unroll
     for (int bj = 0; bj < 4; ++bj)
 #pragma unroll
@@ -213,13 +214,15 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
         ov4 o;
 #pragma unroll
         for (int b = 0; b < 4; ++b) o[b] = (out_t)(acc[bj][bi][4 * a + b] * alpha);
-        *(ov4*)(st + r31 * RSTR + (bj * 32 + 8 * a + 4 * g) * ESZ) = o;
+        *(ov4*)(sb + r31 * RSTR + (bj * 32 + 8 * a + 4 * g) * ESZ) = o;
       }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // LDS operations of one wave execute in order
+  };
+  auto drain = [&](int bi) {  // staging block -> C, whole row pieces
+    const uint8_t* sb = st + (bi % NBUF) * (32 * RSTR);
 #pragma unroll
     for (int p = 0; p < 32 / RPI; ++p) {
       const int row = p * RPI + rb_row;
-      const v4i v = *(const v4i*)(st + row * RSTR + rb_ch * 16);
+      const v4i v = *(const v4i*)(sb + row * RSTR + rb_ch * 16);
       const long m = m0 + wm * 128 + bi * 32 + row;
       out_t* dst = C + m * ldc + n0 + wn * 128 + rb_ch * (16 / ESZ);
       if (!EDGE) {
@@ -235,6 +238,15 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
         }
       }
     }
+  };
+  // The LDS executes one wave's operations in order, so a block may be refilled as soon as the reads that drain it
+  // have been issued; the fences only pin that program order.  With two blocks the conversion of the next row group
+  // runs under the LDS and store latency of the previous one.
+#pragma unroll
+  for (int bi = 0; bi < 4 + NBUF - 1; ++bi) {
+    if (bi < 4) stage(bi);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    if (bi >= NBUF - 1) drain(bi - (NBUF - 1));
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
 }
