@@ -169,3 +169,28 @@ def test_c2_8192_cube_sampled_rows_and_checksum():
     got = out.double().sum(1).cpu()
     scale = (orc.dq(a).double().abs() @ orc.dq(b.T.contiguous()).double().abs().sum(0)) * alpha
     assert float(((got - expect).abs() / scale).max()) < 1e-4
+
+
+def test_random_shapes_layouts_and_dtypes_vs_oracle():
+    """A seeded sweep over shapes that land on every kernel (tile, edge tile, row-major B in place, skinny with one or
+    two row blocks, transpose-through-workspace, general) and over both B layouts and all output types."""
+    rng = np.random.default_rng(1234)
+    lib = _lib.load()
+    seen = set()
+    for case in range(48):
+        m = int(rng.choice([1, 7, 16, 17, 32, 33, 100, 256, 300, 513]))
+        n = int(rng.choice([16, 48, 100, 256, 272, 400, 512, 1000]))
+        k = int(rng.choice([128, 256, 384, 1024, 200]))
+        row_major = bool(rng.integers(0, 2))
+        od = [torch.float16, torch.bfloat16, torch.float32][int(rng.integers(0, 3))]
+        g = torch.Generator().manual_seed(case)
+        x = (torch.randn(m, k, generator=g) * 0.7).to(E4M3)
+        y = (torch.randn(k, n, generator=g) * 0.7).to(E4M3)            # row-major [K, N]
+        yd = y.to(DEV) if row_major else y.to(DEV).T.contiguous().T      # or column-major with the same values
+        sa = torch.rand((), generator=g) * 1.5 + 0.5; sb = torch.rand((), generator=g) * 1.5 + 0.5
+        xd = x.to(DEV)
+        seen.add(lib.hx_fp8_gemm_path(m, n, k, k, yd.stride(0), yd.stride(1), n, xd.data_ptr(), yd.data_ptr(), xd.data_ptr()))
+        out = hx.fp8_gemm(xd, yd, scale_a=sa.to(DEV), scale_b=sb.to(DEV), out_dtype=od)
+        ref = orc.fp8_gemm(x, y, sa, sb, od)
+        assert rel_err(out, ref) <= (1e-2 if od != torch.float32 else 1e-4), (case, m, n, k, row_major, od)
+    assert seen >= {0, 2, 3, 4}   # the aligned tile path (1) has its own cases above
