@@ -133,3 +133,24 @@ def test_tritonbench_wrapper_runs_on_the_reference_layout():
     q8, k8, v8 = hx.preprocess_fp8_attention_inputs(q32.cpu(), k32.cpu(), v32.cpu())
     ref = orc.fp8_attention(q8, k8, v8, 1, 2)
     assert out.dtype == E4M3 and rel_err(out, ref) <= 0.08
+
+
+def test_random_shapes_layouts_vs_oracle():
+    """A seeded sweep over head counts, sequence lengths (every multiple of 64 class: 64, odd multiples, multiples of
+    128), both head dims, both V memory orders and both output types."""
+    rng = np.random.default_rng(99)
+    for case in range(20):
+        b = int(rng.integers(1, 3)); h = int(rng.integers(1, 6))
+        s = int(rng.choice([64, 128, 192, 320, 448, 512, 704]))
+        d = int(rng.choice([64, 128]))
+        v_seq_major = bool(rng.integers(0, 2))
+        q, k, v = inputs.attention_inputs(b, h, s, d, seed=1000 + case)
+        vd = v.to(DEV)
+        if v_seq_major:
+            vd = vd.transpose(1, 2).contiguous().transpose(1, 2)        # [BH, D, S] view of [BH, S, D] memory
+            assert vd.stride() == (s * d, 1, d)
+        ref = orc.fp8_attention(q, k, v, b, h, torch.float32)
+        out = hx.fp8_attention_kernel(q.to(DEV), k.to(DEV), vd, b, h, out_dtype=torch.float32)
+        assert rel_err(out, ref) <= TOL, (case, b, h, s, d, v_seq_major)
+        out8 = hx.fp8_attention_kernel(q.to(DEV), k.to(DEV), vd, b, h)
+        assert rel_err(out8, orc.fp8_attention(q, k, v, b, h)) <= 0.08, (case, b, h, s, d, v_seq_major)

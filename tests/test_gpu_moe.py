@@ -82,3 +82,22 @@ def test_c5_sampled_rows():
         assert rel_err(out[pick.to(DEV)], ref) <= 1e-2
     # top-2: the two rows of a token hold the same activations but different experts
     assert not torch.equal(out[0], out[1])
+
+
+def test_random_shapes_vs_oracle():
+    """A seeded sweep over row counts, K/N that land on the MFMA kernel (K % 64 == 0, N % 8 == 0, ragged last column
+    tile included) and on the general kernel, expert counts, top-k and both 16-bit types; replicated and top-k entry."""
+    rng = np.random.default_rng(7)
+    for case in range(16):
+        tokens = int(rng.choice([1, 50, 256, 700, 1500]))
+        K = int(rng.choice([64, 128, 320, 100]))
+        N = int(rng.choice([8, 256, 264, 384, 1000, 50]))
+        E = int(rng.choice([1, 3, 8, 40]))
+        topk = int(rng.choice([1, 2])) if E >= 2 else 1
+        dtype = [torch.bfloat16, torch.float16][int(rng.integers(0, 2))]
+        A, W, ex = inputs.moe_inputs(tokens, K, N, E, topk, seed=500 + case, dtype=dtype)
+        ref = orc.moe_matmul_ogs_reference(A, W, ex)
+        out = _run(A, W, ex)
+        assert rel_err(out, ref) <= 1e-2, (case, tokens, K, N, E, topk, dtype)
+        out2 = hx.moe_matmul_topk(A[::topk].contiguous().to(DEV), W.to(DEV), ex.to(DEV), topk)
+        assert torch.equal(out, out2), (case, tokens, K, N, E, topk, dtype)
