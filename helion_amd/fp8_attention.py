@@ -1,6 +1,7 @@
 """Drop-in for the reference's examples/fp8_attention.py."""
 from __future__ import annotations
 
+import math
 from typing import Callable
 
 import torch
@@ -42,3 +43,50 @@ def fp8_attention_tritonbench(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor)
     batch, heads, seq_len, head_dim = q.shape
     q_fp8, k_fp8, v_fp8 = preprocess_fp8_attention_inputs(q, k, v)
     return lambda: fp8_attention_kernel(q_fp8, k_fp8, v_fp8, batch, heads)
+
+
+def _fp8_attention_pytorch_impl(q_fp8: torch.Tensor, k_fp8: torch.Tensor, v_fp8: torch.Tensor, batch: int, heads: int,
+                                seq_len: int, head_dim: int) -> torch.Tensor:
+    """The reference's torch baseline (examples/fp8_attention.py:158-238), head by head with torch._scaled_mm.  Its
+    numerics differ from the kernel's on purpose: it normalises p by its row sum *before* the e4m3 cast."""
+    log2e = 1.44269504
+    sm_scale = 1.0 / math.sqrt(float(head_dim))
+    one = torch.tensor(1.0, device=q_fp8.device)
+    heads_out = []
+    for i in range(batch * heads):
+        k_t = k_fp8[i].contiguous().t()                       # [dim, seq], column-major as _scaled_mm wants
+        qk = torch._scaled_mm(q_fp8[i], k_t, one, one, use_fast_accum=False, out_dtype=torch.float32)
+        qk_max = torch.amax(qk, dim=-1, keepdim=True)
+        p = torch.exp2((qk * sm_scale - qk_max * sm_scale) * log2e)
+        p8 = (p / p.sum(dim=-1, keepdim=True)).to(torch.float8_e4m3fn)
+        v_t = v_fp8[i].contiguous().t()                       # [seq, dim], column-major
+        o = torch._scaled_mm(p8, v_t, one, one, use_fast_accum=False, out_dtype=torch.float32)
+        heads_out.append(o.to(torch.float8_e4m3fn))
+    return torch.stack(heads_out, dim=0).reshape(batch, heads, seq_len, head_dim)
+
+
+def fp8_attention_pytorch(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> Callable[[], torch.Tensor]:
+    """examples/fp8_attention.py:242-256: the baseline as a thunk, preprocessing hoisted out of it."""
+    batch, heads, seq_len, head_dim = q.shape
+    q_fp8, k_fp8, v_fp8 = preprocess_fp8_attention_inputs(q, k, v)
+    return lambda: _fp8_attention_pytorch_impl(q_fp8, k_fp8, v_fp8, batch, heads, seq_len, head_dim)
+
+
+def check(batch: int, heads: int, seq_len: int, head_dim: int) -> None:
+    """examples/fp8_attention.py:260-283: kernel against the torch baseline, atol = rtol = 0.1, then a timing table."""
+    from .testing import run_example
+
+    torch.manual_seed(42)
+    q, k, v = (torch.randn(batch, heads, seq_len, head_dim, dtype=torch.float16, device="cuda") for _ in range(3))
+    run_example(fp8_attention_tritonbench(q, k, v), fp8_attention_pytorch(q, k, v), (), atol=0.1, rtol=0.1)
+
+
+def main() -> None:
+    """examples/fp8_attention.py:287-295."""
+    check(1, 2, 128, 64)
+    check(2, 4, 256, 64)
+    check(4, 8, 512, 128)
+
+
+if __name__ == "__main__":
+    main()

@@ -41,3 +41,23 @@ def reference_fp8_gemm_pytorch(x_fp8: torch.Tensor, y_fp8: torch.Tensor) -> torc
 def fp8_gemm_tritonbench(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     """examples/fp8_gemm.py:82-91."""
     return fp8_gemm(a, b)
+
+
+def check(m: int, k: int, n: int) -> None:
+    """examples/fp8_gemm.py:95-109: randn -> e4m3 operands (row-major y), kernel against torch._scaled_mm."""
+    from .testing import run_example
+
+    x = torch.randn([m, k], device="cuda", dtype=torch.float32).to(torch.float8_e4m3fn)
+    y = torch.randn([k, n], device="cuda", dtype=torch.float32).to(torch.float8_e4m3fn)
+    run_example(fp8_gemm, reference_fp8_gemm_pytorch, (x, y))
+
+
+def main() -> None:
+    """examples/fp8_gemm.py:113-119."""
+    check(256, 256, 256)
+    check(512, 512, 512)
+    check(1024, 1024, 1024)
+
+
+if __name__ == "__main__":
+    main()

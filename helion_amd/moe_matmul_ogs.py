@@ -61,3 +61,25 @@ def moe_matmul_ogs_reference(A: torch.Tensor, W: torch.Tensor, top1_expert_per_t
             continue
         C[token_idx] = A[token_idx] @ W[e]
     return C
+
+
+def check(T: int, K: int, N: int, n_experts: int) -> None:
+    """examples/moe_matmul_ogs.py:152-179: fp16 operands, random top-1 routing, kernel against the per-expert
+    definition (rtol 1e-2, atol 1e-1 as in helion/_testing.py:341-349)."""
+    from .testing import run_example
+
+    dtype, device = torch.float16, "cuda"
+    A = torch.randn(T, K, device=device, dtype=dtype)
+    W = torch.randn(n_experts, K, N, device=device, dtype=dtype)
+    top1_expert_per_token = torch.randint(n_experts, (T,), device=device)
+    args = moe_matmul_ogs_helion_kernel_args_gen(A, W, top1_expert_per_token)
+    run_example(lambda: moe_matmul_ogs(*args), lambda: moe_matmul_ogs_reference(A, W, top1_expert_per_token), ())
+
+
+def main() -> None:
+    """examples/moe_matmul_ogs.py:182-186."""
+    check(1000, 500, 200, 30)
+
+
+if __name__ == "__main__":
+    main()
