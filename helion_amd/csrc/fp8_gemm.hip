@@ -10,6 +10,8 @@
 //   hx_fp8_gemm_general : bounds-checked, arbitrary strides (fallback for ragged/unaligned inputs).
 #include "hx_common.h"
 
+#include <type_traits>
+
 // ------------------------------------------------------------------------------------------
 // tile256
 // ------------------------------------------------------------------------------------------
@@ -18,8 +20,9 @@
 //   the chunk stored at (row, pos) is global chunk  pos ^ swz(row),  swz(row) = (row >> 1) & 7.
 // One DMA instruction of a wave moves 8 rows x 128 B (lane = row_in_8 * 8 + pos), so global reads
 // are whole 128-byte lines and LDS writes are 1024 contiguous bytes.
-// MFMA operand fetch: lane (r = lane%32, g = lane/32) of k-step t reads chunks 4t+2g and 4t+2g+1 of
-// row r: two ds_read_b128.  A and B use the same lane->k mapping, which is all the contraction needs.
+// MFMA operand fetch (16x16x128, one instruction spans the whole 128-byte k-tile): lane (r = lane%16, g = lane/16)
+// reads chunks 2g and 2g+1 of row r: two ds_read_b128.  A and B use the same lane->k mapping, which is all the
+// contraction needs.  (Against the 32x32x64 shape this halves the accumulator traffic per flop: +3 % measured.)
 
 #define T256_BM 256
 #define T256_BN 256
@@ -29,9 +32,9 @@
 // EDGE: M and/or N are not multiples of 256.  Rows past the end are clamped to the last row on load (their
 // products land in accumulators that are never stored) and the stores are guarded.
 // BROW: B is row-major ([K][N], N contiguous; `Bt`/`ldb` are then B itself and its row stride).  The B tile sits in
-// LDS as [128 k][256 B of n], chunk stored at pos = chunk ^ ((k&7)<<1), and the MFMA operand (32 consecutive k of one
-// column per lane) is formed by four transposing reads (ds_read_b64_tr_b8: 8 k x 16 n per 16 lanes) instead of two
-// 16-byte reads; one DMA instruction moves 4 k-rows x 256 B.  N must be a multiple of 16; with EDGE, chunks past
+// LDS as [128 k][256 B of n], chunk stored at pos = chunk ^ (((k&7)<<1) | ((k>>5)&1)), and the MFMA operand (32
+// consecutive k of one column per lane) is formed by four transposing reads (ds_read_b64_tr_b8: 8 k x 16 n per 16
+// lanes) instead of two 16-byte reads; one DMA instruction moves 4 k-rows x 256 B.  N must be a multiple of 16; with EDGE, chunks past
 // the end re-read the row's last valid chunk.
 template <int OUT, bool EDGE, bool BROW>
 __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __restrict__ A, const uint8_t* __restrict__ Bt,
@@ -73,7 +76,7 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
   const int brow = lane >> 4, bpos = lane & 15;
   const int bcmax = BROW ? (int)((min((long)N - n0, (long)T256_BN) >> 4) - 1) : 0;  // last valid chunk of this tile's rows
   auto brow_vo = [&](int kodd) {  // kodd: (row within the 8-row swizzle period) >= 4, i.e. j odd
-    int chunk = bpos ^ (((4 * kodd + brow) & 7) << 1);
+    int chunk = bpos ^ ((((4 * kodd + brow) & 7) << 1) | (w & 1));  // k = 32w + 4j + brow: (k>>5)&1 = w&1
     if (EDGE) chunk = min(chunk, bcmax);
     return (uint32_t)(brow * ldb + chunk * 16);
   };
@@ -108,122 +111,128 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
     for (int i = 0; i < 16; ++i) issue_one(kt, stage, i);
   };
 
-  // ---- MFMA operand addressing
-  const int r31 = lane & 31, g = lane >> 5;
-  const int x = ((g * 2) ^ ((r31 >> 1) & 7)) * 16;
-  const int a_base = (wm * 128 + r31) * 128;
-  const int b_base = (wn * 128 + r31) * 128;
-  // row-major B: transposing read j (0..3) of column block bj, k-step t fetches k = 64t + 32g + 8j .. +7; this lane
-  // supplies 8 bytes of row (that k) + (lane%16)/2, columns 16*((lane>>4)&1) + 8*(lane&1) .. +7 of the block and
-  // receives column lane%32.  Block bj / wave column wn add to chunk bits the swizzle's xor commutes with.
-  const int bt_off = (32 * g + ((lane & 15) >> 1)) * 256 + (((((lane >> 4) & 1)) ^ (((lane & 15) >> 1) << 1)) * 16) + (lane & 1) * 8;
+  // ---- MFMA operand addressing (16x16x128: lane = row/column lane%16, k = 32*(lane/16) .. +31 of the 128-byte k-tile)
+  const int r16 = lane & 15, gq = lane >> 4;
+  const int x16 = ((2 * gq) ^ ((r16 >> 1) & 7)) * 16;  // chunk 2gq of the row, swizzled; chunk 2gq+1 is at x16 ^ 16
+  const int a_base = (wm * 128 + r16) * 128;
+  const int b_base = (wn * 128 + r16) * 128;
+  // row-major B: transposing read j (0..3) of column block bj fetches k = 32gq + 8j .. +7; this lane supplies 8 bytes of
+  // row (that k) + (lane%16)/2, columns 8*(lane&1) .. +7 of the block's 16-byte chunk, and receives column lane%16.
+  // The chunk index wn*8 + bj enters by xor, which commutes with the swizzle's xor.
+  const int bt_off = (32 * gq + (r16 >> 1)) * 256 + ((((r16 >> 1) << 1) | (gq & 1)) * 16) + (lane & 1) * 8;
 
-  v16f acc[4][4];  // [bj][bi]: rows = n (B side), cols = m (A side)
+  // acc[bj][bi][r] is C[m0 + wm*128 + 16 bi + lane%16][n0 + wn*128 + 16 bj + 4*(lane/16) + r]
+  v4f acc[8][8];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    for (int j = 0; j < 8; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
 
-  // fragment f (0..7) of the 64-byte k-step t of a stage: f < 4 -> A rows 32f.. of this wave, else B rows 32(f-4)..
-  auto load_frag = [&](v8i(&af)[4], v8i(&bf)[4], int stage, int t, int f) {
-    if (BROW && f >= 4) {
-      const uint8_t* sb = &smem[stage][1][0] + (bt_off ^ ((wn * 8 + (f - 4) * 2) * 16)) + t * 16384;
-      v8i v;
+  auto load_a = [&](v8i& f, int stage, int bi) {
+    const uint8_t* base = &smem[stage][0][0] + a_base + bi * 2048;
+    v4i lo = *(const v4i*)(base + x16);
+    v4i hi = *(const v4i*)(base + (x16 ^ 16));
+    f = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+  };
+  auto load_b = [&](v8i& f, int stage, int bj) {
+    if (BROW) {
+      const uint8_t* sb = &smem[stage][1][0] + (bt_off ^ ((wn * 8 + bj) * 16));
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const v2i part = __builtin_amdgcn_ds_read_tr8_b64_v2i32((v2i __attribute__((address_space(3)))*)(sb + j * 2048));
-        v[2 * j] = part[0];
-        v[2 * j + 1] = part[1];
+        f[2 * j] = part[0];
+        f[2 * j + 1] = part[1];
       }
-      bf[f - 4] = v;
-      return;
+    } else {
+      const uint8_t* base = &smem[stage][1][0] + b_base + bj * 2048;
+      v4i lo = *(const v4i*)(base + x16);
+      v4i hi = *(const v4i*)(base + (x16 ^ 16));
+      f = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
     }
-    const uint8_t* base = (f < 4) ? &smem[stage][0][0] + a_base + f * 4096 : &smem[stage][1][0] + b_base + (f - 4) * 4096;
-    v4i lo = *(const v4i*)(base + (x ^ (t * 64)));
-    v4i hi = *(const v4i*)(base + (x ^ (t * 64 + 16)));
-    v8i v = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-    if (f < 4) af[f] = v; else bf[f - 4] = v;
   };
-  // One k-step: 16 MFMAs on the current fragments.  Slotted between them, in program order pinned by scheduling
-  // barriers: the 8 fragment loads of the next k-step (under the first 8 MFMAs) and, when DMA is set, the 16 DMA
-  // instructions of a later k-tile, one per MFMA.  Spreading the DMA keeps the wave's in-order instruction stream
-  // from stalling behind a burst of 64 address-coalescing requests (4 waves x 16) right after the barrier.
-  auto kstep = [&](v8i(&ca)[4], v8i(&cb)[4], v8i(&na)[4], v8i(&nb)[4], int nstage, int nt, bool load_next, bool dma, int dkt,
-                   int dstage) {
+  // One k-tile = 64 MFMAs in two halves, row-block-major: half h multiplies the 8 A fragments with B fragments
+  // 4h .. 4h+3.  Other work is slotted between the MFMAs in an order pinned by scheduling barriers:
+  //   first half : the B fragments 4..7 of this k-tile (from its own stage);
+  //   barrier    : "tile kt+1 has landed in every wave's view and nobody reads stage kt&1 any more";
+  //   second half: A fragment bi of the NEXT k-tile goes into the registers of A fragment bi as soon as its last MFMA of
+  //                this tile has been issued (28 MFMAs before its first use), B fragments 0..3 of the next tile replace
+  //                the dead ones, and one DMA instruction of tile kt+2 goes out every other MFMA into the stage just
+  //                freed.  Spreading the DMA keeps the wave's in-order instruction stream from stalling behind a burst
+  //                of address-coalescing requests right after the barrier.
+  // No register set is double-buffered, so every k-tile runs the same code.  The last one reads "next" fragments that
+  // nobody uses (from a stage that holds an older tile, or nothing yet when there is a single k-tile): cheaper than a
+  // peeled copy of the tile, which costs the accumulators their fixed registers.
+  const int nk = K / T256_BK;
+  v8i fa[8], fb[8];
+  auto ktile = [&](int kt, auto with_dma) {
+    constexpr bool dma = decltype(with_dma)::value;
+    const int stage = kt & 1;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      if (load_next && i < 8) load_frag(na, nb, nstage, nt, i);
-      acc[i >> 2][i & 3] = hx_mfma_32x32x64_e4m3(cb[i >> 2], ca[i & 3], acc[i >> 2][i & 3]);
-      if (dma) issue_one(dkt, dstage, i);
+    for (int i = 0; i < 32; ++i) {
+      const int bi = i >> 2, bj = i & 3;
+      if ((i & 7) == 0) load_b(fb[4 + (i >> 3)], stage, 4 + (i >> 3));
+      acc[bj][bi] = hx_mfma_16x16x128_e4m3(fb[bj], fa[bi], acc[bj][bi]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    HX_WAIT_VM0();
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+      const int bi = i >> 2, bj = 4 + (i & 3);
+      acc[bj][bi] = hx_mfma_16x16x128_e4m3(fb[bj], fa[bi], acc[bj][bi]);
+      if ((i & 3) == 3) load_a(fa[bi], stage ^ 1, bi);
+      if ((i & 7) == 1) load_b(fb[i >> 3], stage ^ 1, i >> 3);
+      if ((i & 1) && dma) issue_one(kt + 2, stage, i >> 1);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-
-  // Software pipeline.  k-tile kt lives in stage kt&1.  While the MFMAs of (kt, t=0) run, the fragments of
-  // (kt, t=1) are fetched; then one barrier says "tile kt+1 has landed in every wave's view and nobody reads
-  // stage kt&1 any more"; under the MFMAs of (kt, t=1) the fragments of (kt+1, t=0) are fetched and the DMA of
-  // tile kt+2 goes out into the stage just freed.  (Past the end the DMA re-fetches the last tile into the free
-  // stage: harmless, and it keeps the loop free of branches around the accumulators.)
-  const int nk = K / T256_BK;
-  v8i fa0[4], fb0[4], fa1[4], fb1[4];
   issue(0, 0);
   if (nk > 1) issue(1, 1);
   if (nk > 1) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(16)); else HX_WAIT_VM0();
   __syncthreads();
 #pragma unroll
-  for (int f = 0; f < 8; ++f) load_frag(fa0, fb0, 0, 0, f);
-  for (int kt = 0; kt < nk - 1; ++kt) {
-    const int stage = kt & 1;
-    kstep(fa0, fb0, fa1, fb1, stage, 1, true, false, 0, 0);
-    HX_WAIT_VM0();
-    __syncthreads();
-    kstep(fa1, fb1, fa0, fb0, stage ^ 1, 0, true, true, min(kt + 2, nk - 1), stage);
-  }
-  {
-    const int stage = (nk - 1) & 1;
-    kstep(fa0, fb0, fa1, fb1, stage, 1, true, false, 0, 0);
-    kstep(fa1, fb1, fa0, fb0, 0, 0, false, false, 0, 0);
-  }
-  HX_WAIT_VM0();    // the trailing re-fetch has landed ...
-  __syncthreads();  // ... and every wave is past its last fragment read: the LDS can be reused
+  for (int f = 0; f < 8; ++f) load_a(fa[f], 0, f);
+#pragma unroll
+  for (int f = 0; f < 4; ++f) load_b(fb[f], 0, f);
+  int kt = 0;
+  for (; kt + 2 < nk; ++kt) ktile(kt, std::true_type{});
+  for (; kt < nk; ++kt) ktile(kt, std::false_type{});  // the last two k-tiles have nothing left to fetch
+  __syncthreads();  // every wave is past its last fragment read: the LDS can be reused
 
-  // ---- epilogue: acc[bj][bi][4a+b] is C[m0 + wm*128 + bi*32 + lane%32][n0 + wn*128 + bj*32 + 8a + 4g + b].
-  // A lane holds only 4 consecutive columns of a row, so direct stores would hit every 128-byte line of C with
-  // eight separate 16-byte writes.  Each wave instead passes its 32 x 128 block of a row group through its own
+  // ---- epilogue.  A lane holds only 4 consecutive columns of a row, so direct stores would hit every 128-byte line
+  // of C with eight separate 16-byte writes.  Each wave instead passes 32 rows x 128 columns at a time through its own
   // quarter of the LDS and writes whole rows: 16 bytes per lane, consecutive lanes on consecutive bytes.
   float alpha = 1.f;
   if (scale_a) alpha = *scale_a;
   if (scale_b) alpha = alpha * *scale_b;
   constexpr int ESZ = (int)sizeof(out_t);
-  constexpr int ROWB = 128 * ESZ;                   // bytes of one output row of this wave
-  constexpr int RSTR = ROWB + (ESZ == 2 ? 8 : 16);  // padded row stride: conflict-free 8/16-byte writes down a column
-  constexpr int LPR = ROWB / 16;                    // lanes per row when reading back 16 bytes per lane
-  constexpr int RPI = 64 / LPR;                     // rows per store instruction
+  constexpr int ROWB = 128 * ESZ;                    // bytes of one output row of this wave
+  constexpr int RSTR = ROWB + 16;                    // padded row stride: conflict-free 8/16-byte writes down a column
+  constexpr int LPR = ROWB / 16;                     // lanes per row when reading back 16 bytes per lane
+  constexpr int RPI = 64 / LPR;                      // rows per store instruction
   constexpr int NBUF = (2 * 32 * RSTR <= T256_TILE_BYTES) ? 2 : 1;  // 16-bit outputs: two staging blocks per wave
   uint8_t* st = &smem[0][0][0] + w * T256_TILE_BYTES;               // this wave's 32 KB
   typedef out_t ov4 __attribute__((ext_vector_type(4)));
   const int rb_row = lane / LPR, rb_ch = lane % LPR;
-  auto stage = [&](int bi) {  // accumulators of row group bi -> staging block bi % NBUF
-    uint8_t* sb = st + (bi % NBUF) * (32 * RSTR);
+  auto stage_rows = [&](int b32) {  // accumulators of rows 32 b32 .. +31 -> staging block b32 % NBUF
+    uint8_t* sb = st + (b32 % NBUF) * (32 * RSTR);
 #pragma unroll
-    for (int bj = 0; bj < 4; ++bj)
+    for (int h = 0; h < 2; ++h)
 #pragma unroll
-      for (int a = 0; a < 4; ++a) {
+      for (int bj = 0; bj < 8; ++bj) {
         ov4 o;
 #pragma unroll
-        for (int b = 0; b < 4; ++b) o[b] = (out_t)(acc[bj][bi][4 * a + b] * alpha);
-        *(ov4*)(sb + r31 * RSTR + (bj * 32 + 8 * a + 4 * g) * ESZ) = o;
+        for (int b = 0; b < 4; ++b) o[b] = (out_t)(acc[bj][2 * b32 + h][b] * alpha);
+        *(ov4*)(sb + (h * 16 + r16) * RSTR + (bj * 16 + 4 * gq) * ESZ) = o;
       }
   };
-  auto drain = [&](int bi) {  // staging block -> C, whole row pieces
-    const uint8_t* sb = st + (bi % NBUF) * (32 * RSTR);
+  auto drain = [&](int b32) {  // staging block -> C, whole row pieces
+    const uint8_t* sb = st + (b32 % NBUF) * (32 * RSTR);
 #pragma unroll
     for (int p = 0; p < 32 / RPI; ++p) {
       const int row = p * RPI + rb_row;
       const v4i v = *(const v4i*)(sb + row * RSTR + rb_ch * 16);
-      const long m = m0 + wm * 128 + bi * 32 + row;
+      const long m = m0 + wm * 128 + b32 * 32 + row;
       out_t* dst = C + m * ldc + n0 + wn * 128 + rb_ch * (16 / ESZ);
       if (!EDGE) {
         *(v4i*)dst = v;
@@ -243,10 +252,10 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
   // have been issued; the fences only pin that program order.  With two blocks the conversion of the next row group
   // runs under the LDS and store latency of the previous one.
 #pragma unroll
-  for (int bi = 0; bi < 4 + NBUF - 1; ++bi) {
-    if (bi < 4) stage(bi);
+  for (int b32 = 0; b32 < 4 + NBUF - 1; ++b32) {
+    if (b32 < 4) stage_rows(b32);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    if (bi >= NBUF - 1) drain(bi - (NBUF - 1));
+    if (b32 >= NBUF - 1) drain(b32 - (NBUF - 1));
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
 }
