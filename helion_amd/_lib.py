@@ -60,6 +60,14 @@ _SIGNATURES = {
         [_c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_size_t, _c.c_void_p],
     ),
     "hx_fp8_quantize_workspace_bytes": (_c.c_size_t, [_c.c_int64]),
+    "hx_matmul": (
+        _c.c_int,
+        [_c.c_void_p, _c.c_void_p, _c.c_void_p] + [_c.c_int64] * 7 + [_c.c_void_p, _c.c_int, _c.c_int, _c.c_int, _c.c_int, _c.c_int,
+                                                                      _c.c_void_p, _c.c_size_t, _c.c_void_p],
+    ),
+    "hx_matmul_workspace_bytes": (_c.c_size_t, [_c.c_int64] * 7 + [_c.c_int, _c.c_int, _c.c_int, _c.c_int]),
+    "hx_matmul_splits": (_c.c_int, [_c.c_int64] * 7 + [_c.c_int, _c.c_int]),
+    "hx_matmul_path": (_c.c_int, [_c.c_int64] * 7 + [_c.c_int, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p]),
 }
 
 

@@ -11,14 +11,7 @@
 //   3. hx_moe_tile256 / hx_moe_general : the grouped GEMM over (row tile, column tile) pairs;
 //   4. hx_moe_zero_rows  : zero-fills rows whose flag is still clear.
 // Padded rows of a tile are never stored, so there is no read-modify-write and no write race.
-#include "hx_common.h"
-
-struct MoeTile {
-  int expert;
-  int row_start;  // position in the sorted order (index into idx)
-  int rows;       // valid rows in this tile (1..BM)
-  int pad;
-};
+#include "gemm16_tile256.h"
 
 // workspace layout: [0] int num_tiles | [16 ..) MoeTile table[max_tiles] | flags[T] bytes
 static inline size_t moe_table_bytes(int64_t max_tiles) { return 16 + (size_t)max_tiles * sizeof(MoeTile); }
@@ -72,223 +65,6 @@ __global__ void hx_moe_zero_rows(T16* __restrict__ C, long ldc, int T, int N, co
   if (row >= T || flags[row]) return;
   T16* c = C + (long)row * ldc;
   for (int n = threadIdx.x; n < N; n += blockDim.x) c[n] = (T16)0.f;
-}
-
-// ------------------------------------------------------------------------------------------
-// tile256: 256 gathered rows x 256 columns x 64 k per step; 4 waves (2x2) of 128x128; 32x32x16 MFMA.
-//   A tile  [256 rows][128 B]  : same chunk-swizzled layout as the fp8 GEMM; the DMA gathers rows
-//                                through idx, so the gather costs nothing extra.
-//   W tile  [64 k][512 B]      : row = k, 32 chunks of 8 columns; chunk stored at pos = chunk ^ (moe_wswz(k)<<1).
-//                                The MFMA wants 8 consecutive k per lane for one column, W has the
-//                                columns contiguous: ds_read_b64_tr_b16 transposes 4(k) x 16(n) blocks
-//                                on the way out of LDS (two reads per operand).
-// ------------------------------------------------------------------------------------------
-// Swizzle of a W-tile row, in units of 32 bytes (a pair of chunks).  One transposing read has the 32 lanes
-// that the LDS serves together fetch 4 consecutive k rows x two adjacent 32-byte column groups; rows are 512 B
-// apart (the same banks), so the 8 (row, group) combinations must land in 8 different 32-byte bank groups:
-// k&3 goes to bits 2:1 and bit 2 of k to bit 0, which the column-group bit then flips.
-__device__ __forceinline__ int moe_wswz(int k) { return ((k & 3) << 1) | ((k >> 2) & 1); }
-
-template <bool BF>
-struct Mfma16;
-template <>
-struct Mfma16<true> {
-  typedef __bf16 T;
-  typedef v8bf V8;
-  static __device__ __forceinline__ v16f run(v8bf a, v8bf b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
-};
-template <>
-struct Mfma16<false> {
-  typedef _Float16 T;
-  typedef v8h V8;
-  static __device__ __forceinline__ v16f run(v8h a, v8h b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
-};
-
-#define MOE_BM 256
-#define MOE_BN 256
-#define MOE_BK 64
-#define MOE_TILE_BYTES (256 * 128)
-
-template <bool BF>
-__global__ __launch_bounds__(256) void hx_moe_tile256(const uint8_t* __restrict__ A, const uint8_t* __restrict__ W,
-                                                     typename Mfma16<BF>::T* __restrict__ C, const int* __restrict__ num_tiles,
-                                                     const MoeTile* __restrict__ table, const int32_t* __restrict__ idx, int T, int K,
-                                                     int N, int max_tiles, int tiles_n, int a_div) {
-  typedef typename Mfma16<BF>::T out_t;
-  typedef typename Mfma16<BF>::V8 V8;
-  // [stage][A|W][32 KB]
-  __shared__ __attribute__((aligned(1024))) uint8_t smem[2][2][MOE_TILE_BYTES];
-
-  // XCD-contiguous grouped raster over (row tile, column tile), as in the fp8 GEMM
-  int tile;
-  {
-    const int nwg = gridDim.x, wg = blockIdx.x;
-    const int per = nwg >> 3, rem = nwg & 7, xcd = wg & 7, loc = wg >> 3;
-    tile = (xcd < rem) ? xcd * (per + 1) + loc : rem * (per + 1) + (xcd - rem) * per + loc;
-  }
-  const int GM = 8;
-  const int group_size = GM * tiles_n;
-  const int gid = tile / group_size;
-  const int first_m = gid * GM;
-  const int gm = min(max_tiles - first_m, GM);
-  const int tm = first_m + (tile % group_size) % gm;
-  const int tn = (tile % group_size) / gm;
-  if (tm >= *num_tiles) return;
-  const MoeTile mt = table[tm];
-  const long n0 = (long)tn * MOE_BN;
-
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = w >> 1, wn = w & 1;
-
-  // ---- A DMA: wave w owns tile rows [64w, 64w+64), 8 instructions of 8 rows; rows are gathered, so the
-  // per-lane byte offset carries the row (A is below 4 GB, checked by the host).
-  const int lrow = lane >> 3, lpos = lane & 7;
-  uint32_t a_vo[8];
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    int lr = w * 64 + j * 8 + lrow;
-    lr = lr < mt.rows ? lr : 0;  // padded rows re-read row 0 of the tile; never stored
-    int r = idx[mt.row_start + lr];
-    r = (r >= 0 && r < T) ? r : 0;
-    const int swz = ((j & 1) ? 4 + (lrow >> 1) : (lrow >> 1)) & 7;
-    // a_div > 1: C row r is the product of A row r / a_div (top-k routing without a replicated A)
-    a_vo[j] = (uint32_t)(r / a_div) * (uint32_t)(K * 2) + (uint32_t)((lpos ^ swz) * 16);
-  }
-  // ---- W DMA: wave w owns k rows [16w, 16w+16), 8 instructions of 2 rows x 512 B.
-  // row k = 16w + 2j + (lane>>5); chunk = (lane&31) ^ (moe_wswz(k)<<1); k&7 = (2j + (lane>>5)) & 7
-  const uint8_t* We = W + (long)mt.expert * K * N * 2 + n0 * 2 + (long)(w * 16) * N * 2;  // wave-uniform
-  const int wk_l = lane >> 5, wpos = lane & 31;
-  uint32_t w_vo[4];
-  // The last column tile may be ragged (N % 256 != 0, N % 8 == 0): chunks past the end re-read the last valid chunk of
-  // the row; the columns they feed are never stored.
-  const int cmax = (int)((min((long)N - n0, (long)MOE_BN) >> 3) - 1);
-#pragma unroll
-  for (int j = 0; j < 4; ++j) w_vo[j] = (uint32_t)(wk_l * N * 2 + min(wpos ^ (moe_wswz(2 * j + wk_l) << 1), cmax) * 16);
-  const uint32_t lds0 = hx_lds_addr(&smem[0][0][0]);
-
-  // DMA instruction i (0..15) of a k-tile: i < 8 -> gathered A rows 64w + 8i .., else W k-rows 16w + 2(i-8), +1
-  auto issue_one = [&](int kt, int stage, int i) {
-    const uint32_t la = lds0 + (uint32_t)stage * 2 * MOE_TILE_BYTES + (uint32_t)w * 64 * 128;
-    const uint32_t lw = lds0 + (uint32_t)stage * 2 * MOE_TILE_BYTES + MOE_TILE_BYTES + (uint32_t)w * 16 * 512;
-    if (i < 8) hx_g2l16_s(A + (long)kt * 128, a_vo[i], la + i * 1024);
-    else hx_g2l16_s(We + (long)kt * MOE_BK * N * 2 + (long)(2 * (i - 8)) * N * 2, w_vo[(i - 8) & 3], lw + (i - 8) * 1024);
-  };
-  auto issue = [&](int kt, int stage) {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) issue_one(kt, stage, i);
-  };
-
-  // ---- operand addressing
-  const int r31 = lane & 31, g = lane >> 5;
-  const int ax = (g ^ ((r31 >> 1) & 7)) * 16;  // chunk (2*ks + g) ^ swz -> ax ^ (ks*32)
-  const int a_base = (wm * 128 + r31) * 128;
-  // transposing read: lane -> (block b = lane>>4, e = (lane>>2)&3, q = lane&3)
-  //   k = 16*ks + 8*(b>>1) + 4*half + e ; n = wn*128 + 32*bj + 16*(b&1) + 4q
-  const int tb = lane >> 4, te = (lane >> 2) & 3, tq = lane & 3;
-  const int tk = 8 * (tb >> 1) + te;                  // + 16*ks + 4*half
-  const int tn_ = wn * 128 + 16 * (tb & 1) + 4 * tq;  // + 32*bj
-  // byte offset of (k = tk + 4*half, n = tn_) in the W tile.  Column block bj adds 4 to the chunk index in bits
-  // the swizzle mask and tn_>>3 leave alone, so it is an xor with 64*bj; k-step ks adds 16 rows = 8192 bytes.
-  int w_off[2];
-#pragma unroll
-  for (int half = 0; half < 2; ++half) {
-    const int k = tk + 4 * half;
-    w_off[half] = k * 512 + (((tn_ >> 3) ^ (moe_wswz(k) << 1)) * 16) + (tn_ & 7) * 2;
-  }
-
-  v16f acc[4][4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-  // fragment f (0..7) of k-step ks (16 k) of a stage: f < 4 -> A rows 32f.. (one b128), else W columns 32(f-4)..
-  // (two transposing b64 reads)
-  auto load_frag = [&](V8(&af)[4], V8(&wf)[4], int stage, int ks, int f) {
-    if (f < 4) {
-      af[f] = *(const V8*)(&smem[stage][0][0] + a_base + f * 4096 + (ax ^ (ks * 32)));
-    } else {
-      const uint8_t* sw = &smem[stage][1][0];
-      v4s part[2];
-#pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        const int off = (w_off[half] ^ ((f - 4) * 64)) + ks * 8192;
-        part[half] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3)))*)(sw + off));
-      }
-      v8s both = (v8s){part[0][0], part[0][1], part[0][2], part[0][3], part[1][0], part[1][1], part[1][2], part[1][3]};
-      wf[f - 4] = __builtin_bit_cast(V8, both);
-    }
-  };
-  // One k-step: 16 MFMAs on the current fragments; pinned between them the 8 fragment loads of the next k-step and,
-  // when DMA is set, NDMA DMA instructions starting at number D0 (one per MFMA), as in the fp8 GEMM.
-  auto kstep = [&](V8(&ca)[4], V8(&cw)[4], V8(&na)[4], V8(&nw)[4], int nstage, int nks, bool load_next, bool dma, int dkt,
-                   int dstage, int d0) {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      if (load_next && i < 8) load_frag(na, nw, nstage, nks, i);
-      acc[i >> 2][i & 3] = Mfma16<BF>::run(cw[i >> 2], ca[i & 3], acc[i >> 2][i & 3]);
-      if (dma && (i & 1)) issue_one(dkt, dstage, d0 + (i >> 1));
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  };
-
-  // software pipeline, as in the fp8 GEMM: k-tile kt in stage kt&1, four k-steps per tile, fragments double
-  // buffered; the one barrier per tile sits before the last k-step's MFMAs; the 16 DMA instructions of tile kt+2 go
-  // out under the MFMAs of (kt, ks=3) and (kt+1, ks=0), one every other MFMA.
-  const int nk = K / MOE_BK;
-  V8 fa0[4], fw0[4], fa1[4], fw1[4];
-  issue(0, 0);
-  if (nk > 1) issue(1, 1);
-  if (nk > 1) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(16)); else HX_WAIT_VM0();
-  __syncthreads();
-#pragma unroll
-  for (int f = 0; f < 8; ++f) load_frag(fa0, fw0, 0, 0, f);
-  for (int kt = 0; kt < nk - 1; ++kt) {
-    const int stage = kt & 1;
-    // (kt, ks=0): second half of tile kt+1's DMA (its first half went out under (kt-1, ks=3)); stage^1 is free
-    // since the last barrier, and both halves are complete at this iteration's barrier
-    kstep(fa0, fw0, fa1, fw1, stage, 1, true, kt > 0, min(kt + 1, nk - 1), stage ^ 1, 8);
-    kstep(fa1, fw1, fa0, fw0, stage, 2, true, false, 0, 0, 0);
-    kstep(fa0, fw0, fa1, fw1, stage, 3, true, false, 0, 0, 0);
-    HX_WAIT_VM0();
-    __syncthreads();
-    // (kt, ks=3): first half of tile kt+2's DMA into the stage just freed
-    kstep(fa1, fw1, fa0, fw0, stage ^ 1, 0, true, true, min(kt + 2, nk - 1), stage, 0);
-  }
-  {
-    const int stage = (nk - 1) & 1;
-    kstep(fa0, fw0, fa1, fw1, stage, 1, true, nk > 1, nk - 1, stage ^ 1, 8);
-    kstep(fa1, fw1, fa0, fw0, stage, 2, true, false, 0, 0, 0);
-    kstep(fa0, fw0, fa1, fw1, stage, 3, true, false, 0, 0, 0);
-    kstep(fa1, fw1, fa0, fw0, 0, 0, false, false, 0, 0, 0);
-  }
-  HX_WAIT_VM0();  // trailing re-fetches must land before the workgroup's LDS is released
-
-  // ---- epilogue: acc[bj][bi][4a+b] is C[idx[row_start + wm*128 + bi*32 + lane%32]][n0 + wn*128 + bj*32 + 8a + 4g + b]
-#pragma unroll
-  for (int bi = 0; bi < 4; ++bi) {
-    const int lr = wm * 128 + bi * 32 + r31;
-    if (lr < mt.rows) {
-      const int r = idx[mt.row_start + lr];
-      if (r >= 0 && r < T) {
-        out_t* crow = C + (long)r * N + n0 + wn * 128 + 4 * g;
-#pragma unroll
-        for (int bj = 0; bj < 4; ++bj)
-#pragma unroll
-          for (int a = 0; a < 4; ++a) {
-            typedef out_t ov4 __attribute__((ext_vector_type(4)));
-            ov4 o;
-#pragma unroll
-            for (int b = 0; b < 4; ++b) o[b] = (out_t)acc[bj][bi][4 * a + b];
-            // N % 8 == 0 and the piece starts at a multiple of 4: it is either wholly inside the row or wholly outside
-            if (n0 + wn * 128 + 4 * g + bj * 32 + 8 * a < N) *(ov4*)(crow + bj * 32 + 8 * a) = o;
-          }
-      }
-    }
-  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -379,8 +155,10 @@ static int launch_moe(const void* A, const void* W, void* C, const int32_t* coun
                      (const MoeTile*)table, idx, (int)T, flags);
   if (fast) {
     const int tiles_n = (int)((N + MOE_BN - 1) / MOE_BN);
-    hipLaunchKernelGGL(hx_moe_tile256<BF>, dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W, (T16*)C,
-                       (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, max_tiles, tiles_n, (int)a_div);
+    G16Dense d = {};
+    d.lda = K; d.ldb = N; d.ldc = N;
+    hipLaunchKernelGGL((hx_gemm16_tile256<BF, 0>), dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W, (void*)C,
+                       (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, max_tiles, tiles_n, (int)a_div, d);
   } else {
     dim3 grid((unsigned)max_tiles, (unsigned)((N + 63) / 64));
     hipLaunchKernelGGL(hx_moe_general<T16>, grid, dim3(256), 0, s, (const T16*)A, (const T16*)W, (T16*)C, (const int*)num_tiles,

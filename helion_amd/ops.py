@@ -256,3 +256,52 @@ def fp8_quantize_op(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
 @fp8_quantize_op.register_fake
 def _(x):
     return x.new_empty(x.shape, dtype=torch.float8_e4m3fn), x.new_empty((), dtype=torch.float32)
+
+
+# ------------------------------------------------------------------------------ dense matmul (+ bias, relu, split-K)
+@torch.library.custom_op("helion_amd::matmul", mutates_args=())
+def matmul_op(x: torch.Tensor, y: torch.Tensor, bias: torch.Tensor | None, relu: bool, out_dtype: torch.dtype,
+              split_k: int) -> torch.Tensor:
+    _require_cuda(x, y, bias)
+    if x.dim() != 2 or y.dim() != 2:
+        raise ValueError("matmul expects 2-D operands")
+    m, k = x.shape
+    k2, n = y.shape
+    assert k == k2, f"size mismatch {k} != {k2}"
+    dt = torch.promote_types(x.dtype, y.dtype)
+    if dt not in (torch.float16, torch.bfloat16, torch.float32):
+        raise TypeError(f"matmul supports float16, bfloat16 and float32 operands, got {x.dtype} and {y.dtype}")
+    if out_dtype not in (dt, torch.float32):
+        raise TypeError(f"out_dtype must be {dt} or float32, got {out_dtype}")
+    x = x.to(dt)
+    y = y.to(dt)
+    if k > 1 and x.stride(1) != 1 or (m > 1 and x.stride(0) < k):
+        x = x.contiguous()
+    lda = x.stride(0) if m > 1 else max(k, 1)
+    if bias is not None:
+        if bias.numel() != n:
+            raise ValueError(f"bias must have {n} elements, got shape {tuple(bias.shape)}")
+        bias = bias.reshape(n)
+        if bias.dtype not in (dt, torch.float32):
+            bias = bias.to(torch.float32)
+        bias = bias.contiguous()
+    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    if m == 0 or n == 0:
+        return out
+    ldb_k = y.stride(0) if k > 1 else max(n, 1)
+    ldb_n = y.stride(1) if n > 1 else 1
+    lib = _lib.load()
+    has_ep = int(bias is not None or relu)
+    ws_bytes = lib.hx_matmul_workspace_bytes(m, n, k, lda, ldb_k, ldb_n, n, _DT[dt], _DT[out_dtype], has_ep, split_k)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
+    rc = lib.hx_matmul(x.data_ptr(), y.data_ptr(), out.data_ptr(), m, n, k, lda, ldb_k, ldb_n, n,
+                       bias.data_ptr() if bias is not None else None, _DT[bias.dtype] if bias is not None else 0,
+                       int(relu), _DT[dt], _DT[out_dtype], split_k, ws.data_ptr() if ws is not None else None, ws_bytes,
+                       _stream_ptr(x.device))
+    _lib.check(rc, "hx_matmul")
+    return out
+
+
+@matmul_op.register_fake
+def _(x, y, bias, relu, out_dtype, split_k):
+    return x.new_empty((x.shape[0], y.shape[1]), dtype=out_dtype)

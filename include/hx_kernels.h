@@ -148,6 +148,29 @@ int hx_fp8_quantize(const void* src, void* dst, int64_t n, int src_dtype, float*
                     size_t workspace_bytes, void* stream);
 size_t hx_fp8_quantize_workspace_bytes(int64_t n);
 
+/* Dense matmul with a fused epilogue — the reference's `matmul(x, y, epilogue)` (examples/matmul.py:25-56) and
+ * `matmul_split_k(x, y, epilogue)` (examples/matmul_split_k.py:30-68) for the epilogues its examples and tests use
+ * (identity, `acc + bias[tile[1]]`, `relu(acc + bias[tile[1]])`: examples/matmul.py:96-119, test/test_examples.py:143-200):
+ *   c[M,N] = cast( act( fp32(a[M,K]) @ fp32(b[K,N]) + bias[N] ) ),  fp32 accumulation, act = relu if `relu` else identity.
+ * in_dtype: HX_BF16 / HX_F16 (MFMA tile kernel when b is row-major (ldb_n == 1), K % 64 == 0, N % 8 == 0, lda % 8 == 0,
+ * ldb_k % 8 == 0, ldc % 4 == 0 and all pointers are 16-byte aligned) or HX_F32 (plain fp32 kernel, as is everything the
+ * tile kernel does not cover).  out_dtype: in_dtype, or HX_F32 for the raw accumulator an arbitrary epilogue can be
+ * applied to by the caller.  bias: null or [N] in in_dtype or HX_F32 (bias_dtype).
+ * split_k: 1 = every workgroup runs the whole K; n > 1 = K split n ways (fewer if K / 64 < n); 0 = the library picks
+ * (splits only while the output tiles alone do not fill the chip).  Splits go through fp32 partial sums in the
+ * workspace (hx_matmul_workspace_bytes(...) bytes, 16-byte aligned; 0 for one split) and are summed in a fixed order,
+ * with the epilogue applied to the whole sum: every split count gives the reference's one-split (eager) result up to
+ * fp32 summation order.  hx_matmul_splits tells the split count used; hx_matmul_path 1 = tile kernel, 0 = plain. */
+int hx_matmul(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k,
+              int64_t ldb_n, int64_t ldc, const void* bias, int bias_dtype, int relu, int in_dtype, int out_dtype,
+              int split_k, void* workspace, size_t workspace_bytes, void* stream);
+size_t hx_matmul_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
+                                 int in_dtype, int out_dtype, int has_epilogue, int split_k);
+int hx_matmul_splits(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc, int in_dtype,
+                     int split_k);
+int hx_matmul_path(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc, int in_dtype,
+                   const void* a, const void* b, const void* c, const void* bias);
+
 #ifdef __cplusplus
 }
 #endif

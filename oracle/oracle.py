@@ -11,6 +11,7 @@ What it restates (paths relative to the reference checkout):
   scales, ``out_dtype`` = accumulator dtype, then ``acc + result``)
 * ``examples/fp8_attention.py:22-106``     -> :func:`fp8_attention`
 * ``examples/moe_matmul_ogs.py:84-148``    -> :func:`moe_args_gen`, :func:`moe_matmul_ogs`
+* ``examples/matmul.py:25-56``, ``examples/matmul_split_k.py:30-68`` -> :func:`matmul`
 * ``helion/language/loops.py:491-533``     -> "one tile spans the whole dimension" in ref mode,
   which is why every tiled loop below has exactly one iteration.
 
@@ -28,6 +29,10 @@ Pinning status (see tests/test_oracle_*.py):
   build's own definition (amax / 448 scaling), pinned by its algebraic properties (exact powers of two,
   the amax element lands on +-448, dequantisation error within half an e4m3 step) and by the numpy
   e4m3 encoder above.
+* matmul (16-bit / fp32, bias and relu epilogues, also the split-K example, whose eager mode has
+  one split): float64 brute force on small shapes, identity-matrix and zero-operand special cases,
+  the relation the reference's tests assert (``x @ y``, ``relu(x @ y + bias)``:
+  ``test/test_examples.py:33-46,143-200,460-474``).
 * moe_matmul_ogs            : the reference's own unit test skips the accuracy check
   (``test/test_examples.py:434-458``), so the *reference's tests* pin nothing here; the oracle is
   pinned by the semantic definition ``moe_matmul_ogs_reference`` (per-expert dense matmul),
@@ -283,3 +288,23 @@ def moe_matmul_ogs_reference(A, W, expert_per_row) -> torch.Tensor:
             continue
         C[rows] = (A[rows].float() @ W[e].float()).to(dtype)
     return C
+
+
+# --------------------------------------------------------------------------------------------
+# dense matmul with an epilogue (examples/matmul.py:25-56; examples/matmul_split_k.py:30-68 in eager mode, where the
+# K dimension is one tile and therefore one split)
+# --------------------------------------------------------------------------------------------
+def matmul(x: torch.Tensor, y: torch.Tensor, bias: torch.Tensor | None = None, relu: bool = False,
+           out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """``acc = zeros(fp32); acc = addmm(acc, x, y)`` (examples/matmul.py:51-54; with an fp32 accumulator the eager mode
+    computes ``mm(x, y, out_dtype=fp32) + acc``, helion/runtime/ref_mode.py:186-211: exact products, fp32 sums),
+    ``out = epilogue(acc, tile)`` cast to ``promote_types(x.dtype, y.dtype)`` on the store (:55).  The epilogues
+    restated are the ones the reference's examples and tests pass: ``acc + bias[tile[1]]`` (bias promoted to fp32 by
+    the addition) and ``relu`` of it."""
+    dt = torch.promote_types(x.dtype, y.dtype)
+    acc = x.to(torch.float32) @ y.to(torch.float32)
+    if bias is not None:
+        acc = acc + bias.reshape(-1).to(torch.float32)
+    if relu:
+        acc = torch.relu(acc)
+    return acc.to(out_dtype if out_dtype is not None else dt)
