@@ -26,21 +26,6 @@ struct MoeTile {
 // k&3 goes to bits 2:1 and bit 2 of k to bit 0, which the column-group bit then flips.
 __device__ __forceinline__ int moe_wswz(int k) { return ((k & 3) << 1) | ((k >> 2) & 1); }
 
-template <bool BF>
-struct Mfma16;
-template <>
-struct Mfma16<true> {
-  typedef __bf16 T;
-  typedef v8bf V8;
-  static __device__ __forceinline__ v16f run(v8bf a, v8bf b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
-};
-template <>
-struct Mfma16<false> {
-  typedef _Float16 T;
-  typedef v8h V8;
-  static __device__ __forceinline__ v16f run(v8h a, v8h b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
-};
-
 #define MOE_BM 256
 #define MOE_BN 256
 #define MOE_BK 64

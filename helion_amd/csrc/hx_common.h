@@ -57,6 +57,23 @@ __device__ __forceinline__ v4f hx_mfma_16x16x128_e4m3(v8i a, v8i b, v4f c) {
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
 }
 
+// 16-bit MFMA (32x32x16, fp32 accumulate): lane l supplies 8 elements of row/col l%32, k = 8*(l/32) .. +7; the result
+// layout is that of the 32x32 fp8 MFMA above.
+template <bool BF>
+struct Mfma16;
+template <>
+struct Mfma16<true> {
+  typedef __bf16 T;
+  typedef v8bf V8;
+  static __device__ __forceinline__ v16f run(v8bf a, v8bf b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+};
+template <>
+struct Mfma16<false> {
+  typedef _Float16 T;
+  typedef v8h V8;
+  static __device__ __forceinline__ v16f run(v8h a, v8h b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+};
+
 template <int OUT>
 struct OutT;
 template <>

@@ -305,3 +305,38 @@ def matmul_op(x: torch.Tensor, y: torch.Tensor, bias: torch.Tensor | None, relu:
 @matmul_op.register_fake
 def _(x, y, bias, relu, out_dtype, split_k):
     return x.new_empty((x.shape[0], y.shape[1]), dtype=out_dtype)
+
+
+# ------------------------------------------------------------------------------ 16-bit attention
+@torch.library.custom_op("helion_amd::attention", mutates_args=())
+def attention_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+    _require_cuda(q, k, v)
+    if q.dtype not in (torch.float16, torch.bfloat16, torch.float32) or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise TypeError(f"attention expects q, k, v of one dtype out of float16, bfloat16, float32; got {q.dtype}, {k.dtype}, {v.dtype}")
+    if q.dim() < 2 or k.dim() != q.dim() or v.dim() != q.dim():
+        raise ValueError("attention expects q, k, v of shape [..., seq, head_dim] with the same number of dimensions")
+    m_dim, d = q.shape[-2], q.shape[-1]
+    n_dim = k.shape[-2]
+    assert n_dim == v.shape[-2]
+    assert d == k.shape[-1] == v.shape[-1]
+    if n_dim == 0 and q.numel():
+        raise ValueError("attention: no keys (softmax over an empty set)")
+    if q.numel() == 0:
+        return torch.empty_like(q, memory_format=torch.contiguous_format)
+    q3 = q.reshape(-1, m_dim, d).contiguous()
+    k3 = k.reshape(-1, n_dim, d).contiguous()
+    v3 = v.reshape(-1, n_dim, d).contiguous()
+    bh = q3.shape[0]
+    if k3.shape[0] != bh or v3.shape[0] != bh:
+        raise ValueError("attention: q, k, v disagree on the batch dimensions")
+    out = torch.empty_like(q3)
+    if out.numel():
+        rc = _lib.load().hx_attention(q3.data_ptr(), k3.data_ptr(), v3.data_ptr(), out.data_ptr(), bh, m_dim, n_dim, d,
+                                      _DT[q.dtype], _stream_ptr(q.device))
+        _lib.check(rc, "hx_attention")
+    return out.view(q.shape)
+
+
+@attention_op.register_fake
+def _(q, k, v):
+    return torch.empty_like(q, memory_format=torch.contiguous_format)

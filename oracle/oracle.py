@@ -12,6 +12,7 @@ What it restates (paths relative to the reference checkout):
 * ``examples/fp8_attention.py:22-106``     -> :func:`fp8_attention`
 * ``examples/moe_matmul_ogs.py:84-148``    -> :func:`moe_args_gen`, :func:`moe_matmul_ogs`
 * ``examples/matmul.py:25-56``, ``examples/matmul_split_k.py:30-68`` -> :func:`matmul`
+* ``examples/attention.py:33-84``          -> :func:`attention`
 * ``helion/language/loops.py:491-533``     -> "one tile spans the whole dimension" in ref mode,
   which is why every tiled loop below has exactly one iteration.
 
@@ -33,6 +34,9 @@ Pinning status (see tests/test_oracle_*.py):
   one split): float64 brute force on small shapes, identity-matrix and zero-operand special cases,
   the relation the reference's tests assert (``x @ y``, ``relu(x @ y + bias)``:
   ``test/test_examples.py:33-46,143-200,460-474``).
+* attention (16-bit / fp32): float64 brute force with explicit loops, closed-form special cases
+  (one key, uniform scores, a dominant key), key-permutation invariance, and the relation the
+  reference's tests assert (``scaled_dot_product_attention``: ``test/test_examples.py:342-390``).
 * moe_matmul_ogs            : the reference's own unit test skips the accuracy check
   (``test/test_examples.py:434-458``), so the *reference's tests* pin nothing here; the oracle is
   pinned by the semantic definition ``moe_matmul_ogs_reference`` (per-expert dense matmul),
@@ -308,3 +312,26 @@ def matmul(x: torch.Tensor, y: torch.Tensor, bias: torch.Tensor | None = None, r
     if relu:
         acc = torch.relu(acc)
     return acc.to(out_dtype if out_dtype is not None else dt)
+
+
+# --------------------------------------------------------------------------------------------
+# 16-bit / fp32 attention (examples/attention.py:33-84)
+# --------------------------------------------------------------------------------------------
+def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+    """One key tile (the eager mode's ``hl.tile`` spans the whole key dimension, helion/language/loops.py:506-510), so
+    the running max is the exact row max and the rescaling factor of the first and only step multiplies zeros:
+    ``qk = q @ k^T`` (:64), ``m = amax(qk) * qk_scale`` (:65), ``p = exp2(qk * qk_scale - m)`` (:66-67),
+    ``l = sum(p)`` (:68-70), ``acc = p.to(v.dtype) @ v`` in fp32 (:73-75), ``out = (acc / l).to(q.dtype)`` (:78-79).
+    The scores are kept in fp32 here, as the compiled kernel's dot product does; the eager mode's ``torch.bmm`` of
+    16-bit operands returns 16-bit scores, one more rounding that the tolerance of the parity tests covers."""
+    d = q.shape[-1]
+    qk_scale = (1.0 / math.sqrt(d)) * 1.44269504
+    q3 = q.reshape(-1, q.shape[-2], d).to(torch.float32)
+    k3 = k.reshape(-1, k.shape[-2], d).to(torch.float32)
+    v3 = v.reshape(-1, v.shape[-2], d)
+    qk = torch.bmm(q3, k3.transpose(1, 2))
+    m = torch.amax(qk, -1) * qk_scale
+    p = torch.exp2(qk * qk_scale - m[:, :, None])
+    l = p.sum(-1)
+    acc = torch.bmm(p.to(v.dtype).to(torch.float32), v3.to(torch.float32))
+    return (acc / l[:, :, None]).to(q.dtype).view(q.shape)
