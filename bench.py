@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only c2,c3,c4,c5,next] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only c2,c3,c4,c5,next,sib] [--no-cpu-baseline]
 
 The defaults (40 warm-up + 100 timed launches) are long enough for the GPU's clocks to settle under load; a
 handful of launches reads ~15 % low.  A "step" is one launch of the FP8 GEMM at the headline configuration (M=N=K=8192, e4m3 operands,
@@ -188,6 +188,46 @@ def bench_next_rows(steps, warmup):
     return out
 
 
+def bench_siblings(steps, warmup):
+    """The 16-bit siblings (dense matmul with epilogue, split-K matmul, flash attention) at the fp8 configurations'
+    shapes, against the bf16 MFMA roofline (split-K: launch-latency sized, reported in microseconds as well)."""
+    import torch
+    import helion_amd as hx
+    from helion_amd.matmul import bias_relu
+
+    out = {}
+    n_it, n_w = min(steps, 30), min(warmup, 10)
+
+    def mfma(flops, ms, kernel, workload):
+        tf = flops / (ms * 1e-3) / 1e12
+        return {"workload": workload, "ms_per_launch": ms, "value": tf, "unit": "TFLOP/s",
+                "roofline": {"bound": "mfma", "achieved": tf, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tf / PEAK_BF16_TFLOPS,
+                             "traffic": None, "kernel": kernel, "avg_launch_ms": ms, "algorithmic_flops_per_launch": float(flops)}}
+
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn(8192, 8192, device="cuda", generator=g).to(torch.bfloat16)
+    y = torch.randn(8192, 8192, device="cuda", generator=g).to(torch.bfloat16)
+    bias = torch.randn(8192, device="cuda", generator=g).to(torch.bfloat16)
+    ep = bias_relu(bias)
+    ms, _ = _time_launches(lambda: hx.matmul(x, y, ep), n_it, n_w)
+    out["matmul_bf16_bias_relu"] = mfma(2.0 * 8192**3, ms, "hx_gemm16_tile256<bf16, dense + epilogue>",
+                                        "matmul 8192^3 bf16, relu(acc + bias) fused, row-major operands")
+    del x, y, bias
+    x = torch.randn(64, 32768, device="cuda", generator=g).to(torch.float16)
+    y = torch.randn(32768, 64, device="cuda", generator=g).to(torch.float16)
+    ms, _ = _time_launches(lambda: hx.matmul_split_k(x, y), n_it, n_w)
+    out["matmul_split_k_fp16"] = mfma(2.0 * 64 * 64 * 32768, ms, "hx_gemm16_tile256<f16, split-K partials> + hx_matmul16_reduce",
+                                      "matmul_split_k 64 x 32768 x 64 fp16 (the example's shape; launch-latency sized)")
+    del x, y
+    for d in (128, 64):
+        q, k, v = (torch.randn(4, 32, 4096, d, device="cuda", generator=g).to(torch.bfloat16) for _ in range(3))
+        ms, _ = _time_launches(lambda: hx.attention(q, k, v), n_it, n_w)
+        out[f"attention_bf16_d{d}"] = mfma(4.0 * 4 * 32 * 4096 * 4096 * d, ms, f"hx_attention16_kernel<{d}, bf16>",
+                                           f"attention B4 H32 S4096 D{d} bf16 non-causal; flops counted as 4*B*H*S^2*D")
+        del q, k, v
+    return out
+
+
 def cpu_baseline():
     """The reference's ref-eager CPU path for fp8_gemm (ATen CPU torch._scaled_mm, unit scales, fp32
     accumulate, bf16 result) on the 1024^3 configuration, repeated for about 10 s of CPU time."""
@@ -216,7 +256,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=40)
-    ap.add_argument("--only", default="c2,c3,c4,c5,next")
+    ap.add_argument("--only", default="c2,c3,c4,c5,next,sib")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run three plain 1 GiB device copies (a known-traffic kernel to scale rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE by)")
@@ -252,6 +292,9 @@ def main():
         torch.cuda.empty_cache()
     if "next" in only:
         others.update(bench_next_rows(args.steps, args.warmup))
+        torch.cuda.empty_cache()
+    if "sib" in only:
+        others.update(bench_siblings(args.steps, args.warmup))
         torch.cuda.empty_cache()
     line = {
         "metric": "FP8 GEMM/attention TFLOP/s + % of MI355X FP8 MFMA peak (or % HBM BW), 1 GPU",

@@ -14,9 +14,12 @@
 // beyond one exchange between the two lanes of a query per tile.
 #include "hx_common.h"
 
+#include <type_traits>
+
 #define A16_BN 64
 #define A16_WAVES 4
 #define A16_BM (32 * A16_WAVES)
+#define A16_SLACK 8.f  // log2 of how far a row's running max may exceed its softmax reference point
 
 // K tile [64 keys][2D bytes], read as the A operand with 16-byte loads (16 lanes = 16 consecutive rows are served
 // together): the 16-byte chunk index is xor-ed so that those rows land in 16 different bank groups.
@@ -32,7 +35,7 @@ __device__ __forceinline__ int a16_vswz(int row) {
 }
 
 template <int D, bool BF>
-__global__ __launch_bounds__(256, 2) void hx_attention16_kernel(const uint8_t* __restrict__ Q, const uint8_t* __restrict__ Kp,
+__global__ __launch_bounds__(64 * A16_WAVES, 2) void hx_attention16_kernel(const uint8_t* __restrict__ Q, const uint8_t* __restrict__ Kp,
                                                                 const uint8_t* __restrict__ Vp, void* __restrict__ Out, int M, int N,
                                                                 int BH, int qtiles) {
   typedef typename Mfma16<BF>::T T16;
@@ -81,19 +84,21 @@ __global__ __launch_bounds__(256, 2) void hx_attention16_kernel(const uint8_t* _
   const uint32_t k_vo = (uint32_t)(lrow * RB + ((lpos ^ a16_kswz<D>(w * RPD + lrow)) * 16));
   const uint32_t v_vo = (uint32_t)(lrow * RB + ((lpos ^ a16_vswz<D>(w * RPD + lrow)) * 16));
   const uint32_t lds0 = hx_lds_addr(&smem[0][0][0]);
+  auto issue_k_one = [&](int tile, int jj) {
+    const int j = w + A16_WAVES * jj;
+    hx_g2l16_s(Kh + ((long)tile * A16_BN + j * RPD) * RB, k_vo, lds0 + (uint32_t)(tile % NS) * TILE + j * 1024);
+  };
+  auto issue_v_one = [&](int tile, int jj) {
+    const int j = w + A16_WAVES * jj;
+    hx_g2l16_s(Vh + ((long)tile * A16_BN + j * RPD) * RB, v_vo, lds0 + (uint32_t)(NS + tile % NS) * TILE + j * 1024);
+  };
   auto issue_k = [&](int tile) {
 #pragma unroll
-    for (int jj = 0; jj < IPW; ++jj) {
-      const int j = w + A16_WAVES * jj;
-      hx_g2l16_s(Kh + ((long)tile * A16_BN + j * RPD) * RB, k_vo, lds0 + (uint32_t)(tile % NS) * TILE + j * 1024);
-    }
+    for (int jj = 0; jj < IPW; ++jj) issue_k_one(tile, jj);
   };
   auto issue_v = [&](int tile) {
 #pragma unroll
-    for (int jj = 0; jj < IPW; ++jj) {
-      const int j = w + A16_WAVES * jj;
-      hx_g2l16_s(Vh + ((long)tile * A16_BN + j * RPD) * RB, v_vo, lds0 + (uint32_t)(NS + tile % NS) * TILE + j * 1024);
-    }
+    for (int jj = 0; jj < IPW; ++jj) issue_v_one(tile, jj);
   };
 
   // ---- MFMA operand addressing
@@ -127,17 +132,14 @@ __global__ __launch_bounds__(256, 2) void hx_attention16_kernel(const uint8_t* _
   const float c = (float)((1.0 / __builtin_sqrt((double)D)) * 1.44269504);
   const int ntiles = N / A16_BN;
 
-  auto scores = [&](const uint8_t* sk, v16f(&s)[2]) {
+  auto load_kfrag = [&](const uint8_t* sk, int mi) -> V8 {  // A operand of score MFMA mi = kb * KSTEPS + t
+    return *(const V8*)(sk + (k_off[mi / KSTEPS] ^ (32 * (mi % KSTEPS))));
+  };
+  const v16f zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  auto scores = [&](const uint8_t* sk, v16f(&s)[2]) {  // compiler-scheduled; used for the first tile only
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) s[kb][r] = 0.f;
-#pragma unroll
-      for (int t = 0; t < KSTEPS; ++t) {
-        const V8 kf = *(const V8*)(sk + (k_off[kb] ^ (32 * t)));
-        s[kb] = Mfma16<BF>::run(kf, qf[t], s[kb]);
-      }
-    }
+    for (int mi = 0; mi < 2 * KSTEPS; ++mi)
+      s[mi / KSTEPS] = Mfma16<BF>::run(load_kfrag(sk, mi), qf[mi % KSTEPS], mi % KSTEPS ? s[mi / KSTEPS] : zero16);
   };
 
   // The Q loads are the only memory operations the compiler tracks; retire them here so that it has no reason to put
@@ -152,74 +154,114 @@ __global__ __launch_bounds__(256, 2) void hx_attention16_kernel(const uint8_t* _
     for (int r = 0; r < 16; ++r) o[d][r] = 0.f;
   float l4[4] = {0.f, 0.f, 0.f, 0.f};  // four independent partial row sums per lane
 
-  auto softmax_pv = [&](v16f(&s)[2], const uint8_t* sv) {
-    float t0 = s[0][0], t1 = s[1][0];
-#pragma unroll
-    for (int r = 0; r < 16; r += 2) {
-      t0 = fmaxf(fmaxf(t0, s[0][r]), s[0][r + 1]);
-      t1 = fmaxf(fmaxf(t1, s[1][r]), s[1][r + 1]);
-    }
-    float tmax = fmaxf(t0, t1);
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-    const float neg_new = fminf(neg_m, -(tmax * c));
-    const float alpha = __builtin_amdgcn_exp2f(neg_new - neg_m);  // exp2(m_old - m_new); first tile: exp2(-inf) = 0
-    if (__builtin_amdgcn_ballot_w64(neg_new != neg_m)) {         // wave-uniform: most tiles leave every row max alone
-#pragma unroll
-      for (int i = 0; i < 4; ++i) l4[i] *= alpha;
-#pragma unroll
-      for (int d = 0; d < DB; ++d)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) o[d][r] *= alpha;
-    }
-    neg_m = neg_new;
-    V8 pf[4];
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][r], c, neg_m));
-        l4[r & 3] += p;
-        pf[2 * kb + (r >> 3)][r & 7] = (T16)p;
-      }
-#pragma unroll
-    for (int u = 0; u < 4; ++u)
-#pragma unroll
-      for (int d = 0; d < DB; ++d) o[d] = Mfma16<BF>::run(load_vfrag(sv, u, d), pf[u], o[d]);
+  // Pipeline.  K(t) and V(t) live in slot t % NS of their rings; step j reads K(j+1) and V(j); its barrier frees the
+  // slots of K(j) and V(j-1), which take K(j+NS) and V(j+NS-1) (past the end: the last tile again, so that every step
+  // issues the same number of DMA instructions and the counted waits stay exact).
+  //
+  // Inside a step the instruction order is pinned by scheduling barriers, one slot per MFMA, because left to itself
+  // the compiler emits the score MFMAs of the next tile, then the whole softmax, then the P.V MFMAs, and the matrix
+  // pipe idles through the middle part:
+  //   phase 0: row max of tile j's scores, new reference point, (rarely) rescaling of l and the accumulators;
+  //   phase A: one slot per score MFMA of tile j+1, each followed by exp2 / row sum / 16-bit cast of a few of tile j's
+  //            scores;
+  //   phase B: one slot per P.V MFMA of tile j.
+  // Fragments are read from LDS two slots ahead of the MFMA that consumes them; the step's DMA instructions go out one
+  // after every fourth MFMA (a burst of them would hold the in-order instruction stream up).
+  constexpr int NA = 2 * KSTEPS, NB = 4 * DB, EPS = 32 / NA;
+  auto issue_step0 = [&](int t) {  // what "step t - NS" would have issued
+    issue_k(min(t, ntiles - 1));
+    if (t >= 1) issue_v(min(t - 1, ntiles - 1));
   };
-
-  // Pipeline: at step j a wave issues the score MFMAs of tile j+1 and then does the softmax and P.V of tile j, so the
-  // matrix pipe runs under the softmax arithmetic.  K(t) and V(t) live in slot t % NS of their rings; step j reads
-  // K(j+1) and V(j); its barrier frees the slots of K(j) and V(j-1), which take K(j+NS) and V(j+NS-1).
-  auto wait_step = [&](int j) {  // K(j+1) and V(j) of this wave's DMA have landed
-    if (j - 1 + NS < ntiles) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 2) * 2 * IPW));
-    else HX_WAIT_VM0();
-  };
-  for (int t = 0; t < NS; ++t) {
-    if (t < ntiles) issue_k(t);
-    if (t >= 1 && t - 1 < ntiles) issue_v(t - 1);
-  }
-  wait_step(0);
+  for (int t = 0; t < NS; ++t) issue_step0(t);
+  __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 2) * 2 * IPW));
   __syncthreads();
   {
-    auto step = [&](v16f(&cur)[2], v16f(&next)[2], int j) {
-      wait_step(j);
+    auto step = [&](v16f(&cur)[2], v16f(&next)[2], int j, auto has_next_c) {
+      constexpr bool HAS_NEXT = decltype(has_next_c)::value;
+      __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 2) * 2 * IPW));  // this wave's part of K(j+1) and V(j) has landed
       __syncthreads();
-      if (j + NS < ntiles) issue_k(j + NS);
-      if (j + NS - 1 < ntiles) issue_v(j + NS - 1);
-      if (active) {
-        if (j + 1 < ntiles) scores(&smem[0][(j + 1) % NS][0], next);
-        softmax_pv(cur, &smem[1][j % NS][0]);
+      const int dk = min(j + NS, ntiles - 1), dv = min(j + NS - 1, ntiles - 1);
+      if (!active) {
+        issue_k(dk);
+        issue_v(dv);
+        return;
+      }
+      const uint8_t* sk = &smem[0][(j + 1) % NS][0];
+      const uint8_t* sv = &smem[1][j % NS][0];
+      V8 kf[3], vf[3];
+      if (HAS_NEXT) {
+        kf[0] = load_kfrag(sk, 0);
+        kf[1] = load_kfrag(sk, 1);
+      }
+      // ---- phase 0
+      float t0 = cur[0][0], t1 = cur[1][0];
+#pragma unroll
+      for (int r = 0; r < 16; r += 2) {
+        t0 = fmaxf(fmaxf(t0, cur[0][r]), cur[0][r + 1]);
+        t1 = fmaxf(fmaxf(t1, cur[1][r]), cur[1][r + 1]);
+      }
+      float tmax = fmaxf(t0, t1);
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+      // The reference point m of a row only moves when the tile's max exceeds it by more than 2^A16_SLACK: p, l and
+      // the accumulators then run up to that factor above their usual range (p <= 256: exact in either 16-bit format,
+      // and further from its underflow), the quotient acc / l is unchanged, and the rescaling pass below — 70
+      // multiplies per lane — runs on a few tiles per row block instead of on most of them.
+      const float cand = -(tmax * c);
+      const float neg_new = cand < neg_m - A16_SLACK ? cand : neg_m;
+      const float alpha = __builtin_amdgcn_exp2f(neg_new - neg_m);  // exp2(m_old - m_new); first tile: exp2(-inf) = 0
+      if (__builtin_amdgcn_ballot_w64(neg_new != neg_m)) {         // wave-uniform
+#pragma unroll
+        for (int i = 0; i < 4; ++i) l4[i] *= alpha;
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[d][r] *= alpha;
+      }
+      neg_m = neg_new;
+      __builtin_amdgcn_sched_barrier(0);
+      // ---- phase A
+      V8 pf[4];
+#pragma unroll
+      for (int mi = 0; mi < NA; ++mi) {
+        if (HAS_NEXT) {
+          if (mi + 2 < NA) kf[(mi + 2) % 3] = load_kfrag(sk, mi + 2);
+          next[mi / KSTEPS] = Mfma16<BF>::run(kf[mi % 3], qf[mi % KSTEPS], mi % KSTEPS ? next[mi / KSTEPS] : zero16);
+        }
+#pragma unroll
+        for (int e = mi * EPS; e < (mi + 1) * EPS; ++e) {
+          const int kb = e >> 4, r = e & 15;
+          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[kb][r], c, neg_m));
+          l4[r & 3] += p;
+          pf[2 * kb + (r >> 3)][r & 7] = (T16)p;
+        }
+        if ((mi & 3) == 1 && (mi >> 2) < IPW) issue_k_one(dk, mi >> 2);
+        if (mi >= NA - 2) vf[mi - (NA - 2)] = load_vfrag(sv, 0, mi - (NA - 2));
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // ---- phase B
+#pragma unroll
+      for (int mi = 0; mi < NB; ++mi) {
+        if (mi + 2 < NB) vf[(mi + 2) % 3] = load_vfrag(sv, (mi + 2) / DB, (mi + 2) % DB);
+        o[mi % DB] = Mfma16<BF>::run(vf[mi % 3], pf[mi / DB], o[mi % DB]);
+        if ((mi & 3) == 1 && (mi >> 2) < IPW) issue_v_one(dv, mi >> 2);
+        __builtin_amdgcn_sched_barrier(0);
       }
     };
     v16f sa[2], sb[2];
     if (active) scores(&smem[0][0][0], sa);
     int j = 0;
-    for (; j + 1 < ntiles; j += 2) {
-      step(sa, sb, j);
-      step(sb, sa, j + 1);
+    for (; j + 2 < ntiles; j += 2) {
+      step(sa, sb, j, std::true_type{});
+      step(sb, sa, j + 1, std::true_type{});
     }
-    if (j < ntiles) step(sa, sb, j);
+    if (j + 1 < ntiles) {
+      step(sa, sb, j, std::true_type{});
+      step(sb, sa, j + 1, std::false_type{});
+    } else {
+      step(sa, sb, j, std::false_type{});
+    }
   }
+  HX_WAIT_VM0();  // the trailing re-fetches have landed before the LDS is reused
   const float l_lane = (l4[0] + l4[1]) + (l4[2] + l4[3]);
 
   __syncthreads();  // every wave is past its last K/V fragment read: the LDS can be reused
@@ -332,7 +374,7 @@ template <int D, bool BF>
 static void launch_att16(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t M, int64_t N, hipStream_t s) {
   const int qtiles = (int)((M + A16_BM - 1) / A16_BM);
   const int hpx = (int)((BH + 7) / 8);
-  hipLaunchKernelGGL((hx_attention16_kernel<D, BF>), dim3(8 * hpx * qtiles), dim3(256), 0, s, (const uint8_t*)q, (const uint8_t*)k,
+  hipLaunchKernelGGL((hx_attention16_kernel<D, BF>), dim3(8 * hpx * qtiles), dim3(64 * A16_WAVES), 0, s, (const uint8_t*)q, (const uint8_t*)k,
                      (const uint8_t*)v, out, (int)M, (int)N, (int)BH, qtiles);
 }
 
