@@ -143,7 +143,7 @@ def bench_c5(steps, warmup):
         "workload": "C5 moe_matmul_ogs 16384 tokens x top-2 (Zipf 1.2), K4096 N14336 E8 bf16",
         "ms_per_launch": ms, "value": tf, "unit": "TFLOP/s",
         "roofline": {"bound": "mfma", "achieved": tf, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tf / PEAK_BF16_TFLOPS,
-                     "traffic": _traffic("moe_tile256_c5"), "kernel": "hx_moe_tile256 (+prep/mark/zero_rows)",
+                     "traffic": _traffic("moe_tile256_c5"), "kernel": "hx_gemm16_tile256<bf16, grouped> (+prep/mark/zero_rows)",
                      "avg_launch_ms": ms, "algorithmic_flops_per_launch": flops},
     }
 
