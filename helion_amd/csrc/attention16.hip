@@ -4,14 +4,15 @@
 //                      out = cast(acc / l).
 // q [BH, M, D], k [BH, N, D], v [BH, N, D], out [BH, M, D], all contiguous.
 //
-// MFMA kernel (D in {64, 128}, N % 64 == 0): workgroup = 4 waves = 128 queries of one head, wave = 32 queries.
+// MFMA kernel (D in {64, 128}): workgroup = 4 waves = 128 queries of one head, wave = 32 queries.
 // Per 64-key tile a wave computes S^T = K Q^T as two 32x32 blocks (32x32x16 MFMA, D/16 k-steps), so lane
 // (q = lane%32, G = lane/32) holds, per block, the scores of query q against keys 8*(r/4) + 4G + r%4, r = 0..15.
 // Registers 8u' .. 8u'+7 of a block, cast to 16 bits, are exactly the B operand of one k-step (16 keys) of
 // O^T[d][q] += V^T[d][key] P^T[key][q]; the matching V^T operand — for d = lane%32 the keys 16u + 8h + 4G + (0..3),
 // h = 0, 1 — is formed by two transposing LDS reads (ds_read_b64_tr_b16: 4 keys x 16 columns per 16 lanes) of the V
 // tile, which sits in LDS the way it sits in memory, rows = keys.  Row max and row sum need no cross-lane traffic
-// beyond one exchange between the two lanes of a query per tile.
+// beyond one exchange between the two lanes of a query per tile.  TAIL instantiations handle N % 64 != 0: the DMA of
+// the last tile re-reads row N-1 for the missing keys and their scores are set to -inf before the softmax.
 #include "hx_common.h"
 
 #include <type_traits>
@@ -34,7 +35,7 @@ __device__ __forceinline__ int a16_vswz(int row) {
   return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2);
 }
 
-template <int D, bool BF>
+template <int D, bool BF, bool TAIL>
 __global__ __launch_bounds__(64 * A16_WAVES, 2) void hx_attention16_kernel(const uint8_t* __restrict__ Q, const uint8_t* __restrict__ Kp,
                                                                 const uint8_t* __restrict__ Vp, void* __restrict__ Out, int M, int N,
                                                                 int BH, int qtiles) {
@@ -84,13 +85,22 @@ __global__ __launch_bounds__(64 * A16_WAVES, 2) void hx_attention16_kernel(const
   const uint32_t k_vo = (uint32_t)(lrow * RB + ((lpos ^ a16_kswz<D>(w * RPD + lrow)) * 16));
   const uint32_t v_vo = (uint32_t)(lrow * RB + ((lpos ^ a16_vswz<D>(w * RPD + lrow)) * 16));
   const uint32_t lds0 = hx_lds_addr(&smem[0][0][0]);
+  // TAIL: rows past the end of K / V are replaced by row N-1 (valid, finite data; the scores are masked)
+  auto tail_vo = [&](uint32_t vo, int tile, int j) {
+    const int rit = min(j * RPD + lrow, N - 1 - tile * A16_BN);  // row in tile, clamped
+    return (uint32_t)(rit * RB) + (vo - (uint32_t)(lrow * RB));
+  };
   auto issue_k_one = [&](int tile, int jj) {
     const int j = w + A16_WAVES * jj;
-    hx_g2l16_s(Kh + ((long)tile * A16_BN + j * RPD) * RB, k_vo, lds0 + (uint32_t)(tile % NS) * TILE + j * 1024);
+    const uint32_t lds = lds0 + (uint32_t)(tile % NS) * TILE + j * 1024;
+    if (TAIL) hx_g2l16_s(Kh + (long)tile * A16_BN * RB, tail_vo(k_vo, tile, j), lds);
+    else hx_g2l16_s(Kh + ((long)tile * A16_BN + j * RPD) * RB, k_vo, lds);
   };
   auto issue_v_one = [&](int tile, int jj) {
     const int j = w + A16_WAVES * jj;
-    hx_g2l16_s(Vh + ((long)tile * A16_BN + j * RPD) * RB, v_vo, lds0 + (uint32_t)(NS + tile % NS) * TILE + j * 1024);
+    const uint32_t lds = lds0 + (uint32_t)(NS + tile % NS) * TILE + j * 1024;
+    if (TAIL) hx_g2l16_s(Vh + (long)tile * A16_BN * RB, tail_vo(v_vo, tile, j), lds);
+    else hx_g2l16_s(Vh + ((long)tile * A16_BN + j * RPD) * RB, v_vo, lds);
   };
   auto issue_k = [&](int tile) {
 #pragma unroll
@@ -130,7 +140,7 @@ __global__ __launch_bounds__(64 * A16_WAVES, 2) void hx_attention16_kernel(const
   };
 
   const float c = (float)((1.0 / __builtin_sqrt((double)D)) * 1.44269504);
-  const int ntiles = N / A16_BN;
+  const int ntiles = (N + A16_BN - 1) / A16_BN;
 
   auto load_kfrag = [&](const uint8_t* sk, int mi) -> V8 {  // A operand of score MFMA mi = kb * KSTEPS + t
     return *(const V8*)(sk + (k_off[mi / KSTEPS] ^ (32 * (mi % KSTEPS))));
@@ -194,6 +204,13 @@ __global__ __launch_bounds__(64 * A16_WAVES, 2) void hx_attention16_kernel(const
         kf[1] = load_kfrag(sk, 1);
       }
       // ---- phase 0
+      if (TAIL && j == ntiles - 1) {  // keys past the end: score -inf, p = 0
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (j * A16_BN + 32 * kb + 8 * (r >> 2) + 4 * G + (r & 3) >= N) cur[kb][r] = -__builtin_inff();
+      }
       float t0 = cur[0][0], t1 = cur[1][0];
 #pragma unroll
       for (int r = 0; r < 16; r += 2) {
@@ -358,7 +375,7 @@ __global__ __launch_bounds__(256) void hx_attention_general(const T* __restrict_
 static bool att16_fast_ok(const void* q, const void* k, const void* v, const void* out, int64_t BH, int64_t M, int64_t N, int64_t D,
                           int dtype) {
   if (dtype != HX_BF16 && dtype != HX_F16) return false;
-  if ((D != 64 && D != 128) || N % A16_BN || N < A16_BN) return false;
+  if (D != 64 && D != 128) return false;
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) return false;
   if (N * D * 2 >= (1LL << 31) || M * D * 2 >= (1LL << 31)) return false;
   return true;
@@ -374,8 +391,12 @@ template <int D, bool BF>
 static void launch_att16(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t M, int64_t N, hipStream_t s) {
   const int qtiles = (int)((M + A16_BM - 1) / A16_BM);
   const int hpx = (int)((BH + 7) / 8);
-  hipLaunchKernelGGL((hx_attention16_kernel<D, BF>), dim3(8 * hpx * qtiles), dim3(64 * A16_WAVES), 0, s, (const uint8_t*)q, (const uint8_t*)k,
-                     (const uint8_t*)v, out, (int)M, (int)N, (int)BH, qtiles);
+  if (N % A16_BN)
+    hipLaunchKernelGGL((hx_attention16_kernel<D, BF, true>), dim3(8 * hpx * qtiles), dim3(64 * A16_WAVES), 0, s, (const uint8_t*)q,
+                       (const uint8_t*)k, (const uint8_t*)v, out, (int)M, (int)N, (int)BH, qtiles);
+  else
+    hipLaunchKernelGGL((hx_attention16_kernel<D, BF, false>), dim3(8 * hpx * qtiles), dim3(64 * A16_WAVES), 0, s, (const uint8_t*)q,
+                       (const uint8_t*)k, (const uint8_t*)v, out, (int)M, (int)N, (int)BH, qtiles);
 }
 
 extern "C" int hx_attention(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t M, int64_t N, int64_t D,

@@ -177,8 +177,8 @@ int hx_matmul_path(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, 
  * over key tiles as the reference's compiled kernel does (for 16-bit p the result does not depend on the tiling
  * beyond rounding noise; its eager mode is the one-tile case).
  * q [BH, M, D], k [BH, N, D], v [BH, N, D], out [BH, M, D], contiguous, all of `dtype` (HX_BF16 / HX_F16: MFMA kernel
- * when D is 64 or 128, N % 64 == 0 and the pointers are 16-byte aligned; HX_F32 and every other shape with D <= 256:
- * plain kernel).  hx_attention_path: 1 = MFMA kernel, 0 = plain. */
+ * when D is 64 or 128 and the pointers are 16-byte aligned, any M and N; HX_F32 and every other D <= 256: plain
+ * kernel).  hx_attention_path: 1 = MFMA kernel, 0 = plain. */
 int hx_attention(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t M, int64_t N, int64_t D,
                  int dtype, void* stream);
 int hx_attention_path(int64_t BH, int64_t M, int64_t N, int64_t D, int dtype, const void* q, const void* k, const void* v,

@@ -32,7 +32,7 @@ def _path(q, k):
 @pytest.mark.parametrize("shape_q,n,path", [
     ((2, 4, 256, 64), 256, 1), ((1, 2, 128, 128), 128, 1), ((2, 3, 1024, 64), 512, 1),   # seq_q != seq_k: test_examples.py:358-372
     ((1, 3, 100, 128), 192, 1), ((3, 1, 64), 64, 1), ((9, 33, 64), 1024, 1), ((1, 1, 200, 128), 2048, 1),
-    ((2, 2, 50, 64), 70, 0), ((1, 2, 40, 32), 64, 0), ((1, 1, 17, 80), 33, 0), ((2, 5, 256), 9, 0),
+    ((2, 2, 50, 64), 70, 1), ((1, 3, 130, 128), 1, 1), ((2, 1, 64, 128), 63, 1), ((2, 2, 33, 64), 1000, 1), ((1, 2, 40, 32), 64, 0), ((1, 1, 17, 80), 33, 0), ((2, 5, 256), 9, 0),
 ])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_shapes_vs_oracle(shape_q, n, path, dtype):
@@ -96,7 +96,7 @@ def test_seeded_random_sweep():
     for _ in range(12):
         d = (64, 128)[int(torch.randint(0, 2, (1,), generator=g))]
         bh = int(torch.randint(1, 20, (1,), generator=g)); m = int(torch.randint(1, 400, (1,), generator=g))
-        n = 64 * int(torch.randint(1, 12, (1,), generator=g))
+        n = int(torch.randint(1, 700, (1,), generator=g))
         dtype = (torch.float16, torch.bfloat16)[int(torch.randint(0, 2, (1,), generator=g))]
         q, k, v = _mk((bh, m, d), n, dtype, int(torch.randint(0, 1 << 30, (1,), generator=g)))
         out = hx.attention(q.to(DEV), k.to(DEV), v.to(DEV))
