@@ -85,24 +85,35 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
   const uint8_t* gA = A + (m0 + w * 64) * lda;                                  // wave-uniform
   const uint8_t* gB = BROW ? Bt + (long)(w * 32) * ldb + n0 : Bt + (n0 + w * 64) * ldb;  // wave-uniform
   const uint32_t lds0 = hx_lds_addr(&smem[0][0][0]) + (uint32_t)w * 64 * 128;
+  const uint8_t* gB0 = Bt + n0;  // row-major B, edge tiles: per-lane k rows
 
+  // k-tiles; with EDGE the last one may be partial (K % 16 == 0): its DMA re-reads valid chunks / rows instead of
+  // running off the operands, and the part past K is zeroed in LDS once it has landed (zero_tail below)
+  const int nk = EDGE ? (K + T256_BK - 1) / T256_BK : K / T256_BK;
+  const int ktail = K - (nk - 1) * T256_BK;  // valid k of the last tile: 128 unless EDGE
   // DMA instruction i (0..15) of a k-tile: i < 8 -> A rows 64w + 8i .., else B rows 64w + 8(i-8) ..
   auto issue_one = [&](int kt, int stage, int i) {
     const long kb = (long)kt * T256_BK;
     const uint32_t la = lds0 + (uint32_t)stage * 2 * T256_TILE_BYTES, lb = la + T256_TILE_BYTES;
     if (BROW && i >= 8) {  // 4 k-rows x 256 B; column clamping (EDGE) is already in the per-lane offsets
-      hx_g2l16_s(gB + (kb + (long)(i - 8) * 4) * ldb, (i & 1) ? b_vo1 : b_vo0, lb + (i - 8) * 1024);
+      if (EDGE) {  // k rows past K re-read row K-1; the whole of B is below 4 GB (checked by the host)
+        const uint32_t krow = (uint32_t)min((int)kb + w * 32 + (i - 8) * 4 + brow, K - 1);
+        hx_g2l16_s(hx_uniform_ptr(gB0), krow * (uint32_t)ldb + (((i & 1) ? b_vo1 : b_vo0) - (uint32_t)(brow * ldb)), lb + (i - 8) * 1024);
+      } else {
+        hx_g2l16_s(gB + (kb + (long)(i - 8) * 4) * ldb, (i & 1) ? b_vo1 : b_vo0, lb + (i - 8) * 1024);
+      }
     } else if (!EDGE) {
       if (i < 8) hx_g2l16_s(gA + (long)i * 8 * lda + kb, (i & 1) ? a_vo1 : a_vo0, la + i * 1024);
       else hx_g2l16_s(gB + (long)(i - 8) * 8 * ldb + kb, (i & 1) ? b_vo1 : b_vo0, lb + (i - 8) * 1024);
     } else {  // per-lane clamped row; the whole matrix is below 4 GB (checked by the host), so the offset fits 32 bits
       const int swz = (((i & 1) ? 4 : 0) + (lrow >> 1)) & 7;
+      const int chunk = min(lpos ^ swz, (kt == nk - 1 ? ktail / 16 : 8) - 1);  // chunks past K re-read the last valid one
       if (i < 8) {
         const uint32_t row = (uint32_t)min((int)m0 + w * 64 + i * 8 + lrow, M - 1);
-        hx_g2l16_s(A + kb, row * (uint32_t)lda + (uint32_t)((lpos ^ swz) * 16), la + i * 1024);
+        hx_g2l16_s(hx_uniform_ptr(A + kb), row * (uint32_t)lda + (uint32_t)(chunk * 16), la + i * 1024);
       } else {
         const uint32_t row = (uint32_t)min((int)n0 + w * 64 + (i - 8) * 8 + lrow, N - 1);
-        hx_g2l16_s(Bt + kb, row * (uint32_t)ldb + (uint32_t)((lpos ^ swz) * 16), lb + (i - 8) * 1024);
+        hx_g2l16_s(hx_uniform_ptr(Bt + kb), row * (uint32_t)ldb + (uint32_t)(chunk * 16), lb + (i - 8) * 1024);
       }
     }
   };
@@ -162,7 +173,21 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
   // No register set is double-buffered, so every k-tile runs the same code.  The last one reads "next" fragments that
   // nobody uses (from a stage that holds an older tile, or nothing yet when there is a single k-tile): cheaper than a
   // peeled copy of the tile, which costs the accumulators their fixed registers.
-  const int nk = K / T256_BK;
+  // Zero the part of the last k-tile past K, each wave in the rows it fetched itself (so its own vmcnt wait covers
+  // them): A and K-contiguous B rows 64w + lane, chunks ktail/16 .. 7; row-major B: whole k rows >= ktail.
+  auto zero_tail = [&](int stage) {
+    const v4i z = {0, 0, 0, 0};
+    const int row = w * 64 + lane;
+    for (int c = ktail / 16; c < 8; ++c) {
+      const int off = row * 128 + ((c ^ ((row >> 1) & 7)) * 16);
+      *(v4i*)(&smem[stage][0][0] + off) = z;
+      if (!BROW) *(v4i*)(&smem[stage][1][0] + off) = z;
+    }
+    if (BROW)
+      for (int r = w * 32 + (lane >> 4); r < w * 32 + 32; r += 4)
+        if (r >= ktail) *(v4i*)(&smem[stage][1][0] + r * 256 + (lane & 15) * 16) = z;
+  };
+  const bool has_tail = EDGE && ktail != T256_BK;
   v8i fa[8], fb[8];
   auto ktile = [&](int kt, auto with_dma) {
     constexpr bool dma = decltype(with_dma)::value;
@@ -175,6 +200,7 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
       __builtin_amdgcn_sched_barrier(0);
     }
     HX_WAIT_VM0();
+    if (has_tail && kt == nk - 2) zero_tail(stage ^ 1);  // the last tile has just landed in the other stage
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
@@ -189,6 +215,7 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
   issue(0, 0);
   if (nk > 1) issue(1, 1);
   if (nk > 1) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(16)); else HX_WAIT_VM0();
+  if (has_tail && nk == 1) zero_tail(0);
   __syncthreads();
 #pragma unroll
   for (int f = 0; f < 8; ++f) load_a(fa[f], 0, f);
@@ -563,19 +590,20 @@ static inline bool aligned(const void* p, size_t a) { return ((uintptr_t)p & (a 
 // 0 general, 1 tile256, 2 skinny, 3 tile256 with edge tiles (M or N not a multiple of 256)
 static int gemm_path_kmajor(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, const void* a, const void* b,
                             const void* c) {
-  const bool ok = (lda % 16 == 0) && (ldb % 16 == 0) && (K % 128 == 0) && aligned(a, 16) && aligned(b, 16) && K >= 128;
+  const bool ok = (lda % 16 == 0) && (ldb % 16 == 0) && (K % 16 == 0) && aligned(a, 16) && aligned(b, 16) && K >= 16;
   if (!ok) return 0;
-  if ((M <= 16 || (M <= 32 && K <= 8192)) && lda >= K && ldb >= K) return 2;
+  const bool ktail = K % 128 != 0;  // only the edge instantiation of the tile kernel pads a partial last k-tile
+  if (!ktail && (M <= 16 || (M <= 32 && K <= 8192)) && lda >= K && ldb >= K) return 2;
   if (lda >= (1LL << 27) || ldb >= (1LL << 27)) return 0;
-  if ((M % 256 == 0) && (N % 256 == 0) && (ldc % 8 == 0) && aligned(c, 16)) return 1;  // 16-byte row-aligned stores
+  if (!ktail && (M % 256 == 0) && (N % 256 == 0) && (ldc % 8 == 0) && aligned(c, 16)) return 1;  // 16-byte row-aligned stores
   if (M * lda < (1LL << 32) && N * ldb < (1LL << 32)) return 3;
   return 0;
 }
 
 // row-major B (N contiguous) on the tile kernel's transposing-read mode
 static bool gemm_path_rowmajor_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, const void* a, const void* b) {
-  return M > 16 && (lda % 16 == 0) && (ldb_k % 16 == 0) && (K % 128 == 0) && K >= 128 && (N % 16 == 0) && ldb_k >= N && aligned(a, 16) &&
-         aligned(b, 16) && lda < (1LL << 27) && ldb_k < (1LL << 27) && M * lda < (1LL << 32);
+  return M > 16 && (lda % 16 == 0) && (ldb_k % 16 == 0) && (K % 16 == 0) && K >= 16 && (N % 16 == 0) && ldb_k >= N && aligned(a, 16) &&
+         aligned(b, 16) && lda < (1LL << 27) && ldb_k < (1LL << 27) && M * lda < (1LL << 32) && K * ldb_k < (1LL << 32);
 }
 
 extern "C" int hx_fp8_gemm_path(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
@@ -591,7 +619,7 @@ static void launch_kmajor(int path, const void* a, const void* bt, void* c, int6
   typedef typename OutT<OUT>::T out_t;
   if (path == 4) {  // row-major B; ldb is its row stride
     const int tiles_m = (int)((M + 255) / 256), tiles_n = (int)((N + 255) / 256);
-    const bool edge = (M % 256 != 0) || (N % 256 != 0) || (ldc % 8 != 0) || !aligned(c, 16);
+    const bool edge = (M % 256 != 0) || (N % 256 != 0) || (K % 128 != 0) || (ldc % 8 != 0) || !aligned(c, 16);
     if (!edge)
       hipLaunchKernelGGL((hx_fp8_gemm_tile256<OUT, false, true>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
                          (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m,
@@ -669,7 +697,7 @@ extern "C" size_t hx_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, i
   // Only a row-major B (N contiguous) that the tile kernel cannot read in place (M <= 16: the skinny kernel wants K
   // contiguous; N or the row stride not a multiple of 16) but that could take a fast path after a transpose needs
   // scratch: N*K bytes.
-  if (M <= 0 || N <= 0 || K <= 0 || ldb_k == 1 || ldb_n != 1 || K % 128 != 0) return 0;
+  if (M <= 0 || N <= 0 || K <= 0 || ldb_k == 1 || ldb_n != 1 || K % 16 != 0) return 0;
   if (M > 16 && N % 16 == 0 && ldb_k % 16 == 0) return 0;
   return (size_t)(N * K);
 }

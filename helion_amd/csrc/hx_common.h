@@ -36,6 +36,12 @@ __device__ __forceinline__ void hx_g2l16(const void* gptr, void* lds_wave_base) 
 __device__ __forceinline__ void hx_g2l16_s(const void* sbase, uint32_t voff, uint32_t lds_wave_base) {
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_wave_base), "v"(voff), "s"(sbase) : "memory", "m0");
 }
+// A wave-uniform pointer the compiler cannot prove uniform (the "s" constraint above needs SGPRs)
+__device__ __forceinline__ const uint8_t* hx_uniform_ptr(const uint8_t* p) {
+  const uint64_t v = (uint64_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return (const uint8_t*)(((uint64_t)hi << 32) | lo);
+}
 __device__ __forceinline__ uint32_t hx_lds_addr(const void* p) {
   return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t*)p;
 }

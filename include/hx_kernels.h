@@ -1,5 +1,6 @@
 /* C ABI of libhx_kernels.so — hand-written gfx950 (MI355X) kernels behind the three Helion example
- * entry points fp8_gemm, fp8_attention_kernel and moe_matmul_ogs.
+ * entry points fp8_gemm, fp8_attention_kernel and moe_matmul_ogs, and of their 16-bit siblings matmul,
+ * matmul_split_k and attention.
  *
  * Conventions (all functions):
  *   - plain pointers and sizes only; every pointer is DEVICE memory owned by the caller;
@@ -49,8 +50,9 @@ const char* hx_last_error(void);
  * c: [M,N] of out_dtype (HX_F16 = reference default, HX_BF16, HX_F32), element (m,n) at c[m*ldc+n].
  * scale_a/scale_b: device pointers to one fp32 each, or NULL for 1.0 (the reference hard-codes
  *    1.0, helion/language/matmul_ops.py:232-233).
- * Chooses between the 256x256 MFMA tile kernel (with guarded edge tiles when M or N is ragged; it reads a
- * column-major B directly and a row-major B through transposing LDS loads), the skinny (M<=16, or M<=32 with K<=8192) wave-split-K kernel
+ * Chooses between the 256x256 MFMA tile kernel (with guarded edge tiles when M or N is ragged or K is not a multiple
+ * of 128 — K % 16 == 0 suffices, the last k-tile is zero-padded in LDS; it reads a column-major B directly and a
+ * row-major B through transposing LDS loads), the skinny (M<=16, or M<=32 with K<=8192) wave-split-K kernel
  * and a bounds-checked general kernel from the shape, strides and alignment.
  * workspace: optional device scratch of hx_fp8_gemm_workspace_bytes(...) bytes, 16-byte aligned. */
 int hx_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int64_t lda,

@@ -27,6 +27,7 @@ def _path(m, n, k):
     (16, 512, 1024, 2), (1, 16, 128, 2), (5, 48, 256, 2), (16, 1000, 384, 2), (9, 33, 8192 + 128, 2), (16, 64, 16384, 2),
     (17, 256, 256, 2), (32, 512, 8192, 2), (24, 100, 1152, 2), (31, 33, 384, 2),        # two 16-row blocks on the skinny kernel
     (1000, 1000, 1024, 3), (300, 200, 256, 3), (257, 255, 128, 3), (33, 256, 256, 3), (32, 64, 8192 + 128, 3), (255, 1, 128, 3),
+    (256, 256, 208, 3), (300, 200, 144, 3), (1000, 1000, 1040, 3), (64, 64, 16, 3), (16, 512, 1024 + 16, 3), (512, 256, 128 * 5 + 112, 3),  # K tails
     (100, 70, 50, 0), (256, 256, 200, 0), (3, 5, 7, 0), (64, 64, 0, 0),
 ])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16, torch.float32])
@@ -45,6 +46,9 @@ def test_shapes_vs_oracle(m, n, k, path, out_dtype):
     (300, 256, 208, 4, 0),            # ragged M and N (N % 16 == 0): clamped chunks, guarded stores
     (1000, 512, 1008, 4, 0),
     (17, 128, 16, 4, 0),              # one valid 16-byte chunk per row
+    (256, 400, 512, 4, 0),            # K % 128 != 0: the last k-tile is zero-padded in LDS
+    (300, 144, 208, 4, 0),
+    (100, 16, 48, 4, 0),
     (300, 256, 200, 0, 200 * 256),    # N % 16 != 0: transposed into the workspace, then the edge-tile kernel
     (16, 1024, 512, 0, 512 * 1024),   # skinny shape: transposed, then the skinny kernel
     (64, 100, 48, 0, 0),              # K % 128 != 0: general kernel
@@ -177,10 +181,10 @@ def test_random_shapes_layouts_and_dtypes_vs_oracle():
     rng = np.random.default_rng(1234)
     lib = _lib.load()
     seen = set()
-    for case in range(48):
+    for case in range(64):
         m = int(rng.choice([1, 7, 16, 17, 32, 33, 100, 256, 300, 513]))
         n = int(rng.choice([16, 48, 100, 256, 272, 400, 512, 1000]))
-        k = int(rng.choice([128, 256, 384, 1024, 200]))
+        k = int(rng.choice([128, 256, 384, 1024, 200, 16, 144, 1200]))
         row_major = bool(rng.integers(0, 2))
         od = [torch.float16, torch.bfloat16, torch.float32][int(rng.integers(0, 3))]
         g = torch.Generator().manual_seed(case)
