@@ -33,6 +33,8 @@ __device__ __forceinline__ int moe_wswz(int k) { return ((k & 3) << 1) | ((k >> 
 
 // MODE 0: grouped (MoE) GEMM: rows gathered through the tile table and idx, W of the tile's expert, 16-bit output.
 // MODE 1: dense C = act(A @ W + bias): row tile t covers rows 256t ..; 16-bit output.
+// BCOL (dense modes): W is given column-major, i.e. as W^T [N][K] with row stride ldb (an nn.Linear weight used as
+//         w.T): its tile sits in LDS like the A tile, rows = columns of W, and feeds the MFMA through plain 16-byte reads.
 // MODE 2: dense, raw fp32 accumulators of k-tiles [y*kt_per_split, ...) to the fp32 matrix number blockIdx.y at C
 //         (split-K partial sums, or the input of an epilogue applied elsewhere).
 struct G16Dense {
@@ -43,7 +45,7 @@ struct G16Dense {
   int kt_per_split;     // MODE 2: k-tiles per blockIdx.y
 };
 
-template <bool BF, int MODE>
+template <bool BF, int MODE, bool BCOL = false>
 __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restrict__ A, const uint8_t* __restrict__ W,
                                                         void* __restrict__ Cv, const int* __restrict__ num_tiles,
                                                         const MoeTile* __restrict__ table, const int32_t* __restrict__ idx, int T, int K,
@@ -115,6 +117,17 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restri
   const int cmax = (int)((min((long)N - n0, (long)MOE_BN) >> 3) - 1);
 #pragma unroll
   for (int j = 0; j < 4; ++j) w_vo[j] = (uint32_t)(wk_l * d.ldb * 2 + min(wpos ^ (moe_wswz(2 * j + wk_l) << 1), cmax) * 16);
+  // column-major W: wave w owns tile columns [64w, 64w+64) = rows of W^T, 8 instructions of 8 rows, exactly like A;
+  // columns past N re-read column N-1 and are never stored (W^T is below 4 GB, checked by the host)
+  uint32_t wc_vo[BCOL ? 8 : 1];
+  if (BCOL) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int col = (int)min(n0 + w * 64 + j * 8 + lrow, (long)N - 1);
+      const int swz = ((j & 1) ? 4 + (lrow >> 1) : (lrow >> 1)) & 7;
+      wc_vo[j] = (uint32_t)col * (uint32_t)(d.ldb * 2) + (uint32_t)((lpos ^ swz) * 16);
+    }
+  }
   const uint32_t lds0 = hx_lds_addr(&smem[0][0][0]);
 
   // DMA instruction i (0..15) of a k-tile: i < 8 -> gathered A rows 64w + 8i .., else W k-rows 16w + 2(i-8), +1
@@ -122,6 +135,7 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restri
     const uint32_t la = lds0 + (uint32_t)stage * 2 * MOE_TILE_BYTES + (uint32_t)w * 64 * 128;
     const uint32_t lw = lds0 + (uint32_t)stage * 2 * MOE_TILE_BYTES + MOE_TILE_BYTES + (uint32_t)w * 16 * 512;
     if (i < 8) hx_g2l16_s(A + (long)kt * 128, a_vo[i], la + i * 1024);
+    else if (BCOL) hx_g2l16_s(W + ((long)kt0 + kt) * 128, wc_vo[BCOL ? i - 8 : 0], lds0 + (uint32_t)stage * 2 * MOE_TILE_BYTES + MOE_TILE_BYTES + (uint32_t)w * 64 * 128 + (i - 8) * 1024);
     else hx_g2l16_s(We + ((long)kt * MOE_BK + 2 * (i - 8)) * d.ldb * 2, w_vo[(i - 8) & 3], lw + (i - 8) * 1024);
   };
   auto issue = [&](int kt, int stage) {
@@ -160,6 +174,8 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restri
   auto load_frag = [&](V8(&af)[4], V8(&wf)[4], int stage, int ks, int f) {
     if (f < 4) {
       af[f] = *(const V8*)(&smem[stage][0][0] + a_base + f * 4096 + (ax ^ (ks * 32)));
+    } else if (BCOL) {
+      wf[f - 4] = *(const V8*)(&smem[stage][1][0] + (wn * 128 + r31) * 128 + (f - 4) * 4096 + (ax ^ (ks * 32)));
     } else {
       const uint8_t* sw = &smem[stage][1][0];
       v4s part[2];

@@ -1,7 +1,7 @@
 // Dense matmul with a fused epilogue for gfx950 — device side of the reference's examples/matmul.py:25-56 and
 // examples/matmul_split_k.py:30-68:
 //   C = cast( act( fp32(A) @ fp32(B) + bias[None, :] ) ),   act = identity | relu,  fp32 accumulation.
-// A [M,K], B [K,N], bias [N] or absent.  bf16 / fp16 operands run the 256x256x64 MFMA tile kernel that the grouped
+// A [M,K], B [K,N] row-major or column-major, bias [N] or absent.  bf16 / fp16 operands run the 256x256x64 MFMA tile kernel that the grouped
 // (MoE) GEMM uses; K can be split over workgroups (blockIdx.y), the fp32 partial sums then go through the workspace and
 // a second kernel adds them up, applies the epilogue and casts.  The reference's split-K accumulates with atomics in
 // the output type and applies the epilogue to the first split only; its result for one split — which is what its eager
@@ -89,10 +89,12 @@ __global__ __launch_bounds__(256) void hx_matmul16_reduce(const float* __restric
 static bool mm_fast_ok(const void* a, const void* b, const void* c, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k,
                        int64_t ldb_n, int64_t ldc, const void* bias, int in_dtype) {
   if (in_dtype != HX_BF16 && in_dtype != HX_F16) return false;
-  if (ldb_n != 1 || K < MOE_BK || K % MOE_BK || N % 8 || lda % 8 || ldb_k % 8 || ldc % 4) return false;
+  if (K < MOE_BK || K % MOE_BK || N % 8 || lda % 8 || ldc % 4) return false;
   if ((((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)bias) & 15) != 0) return false;
-  if (M * lda * 2 >= (1LL << 32) || ldb_k * 4 >= (1LL << 31)) return false;
-  return true;
+  if (M * lda * 2 >= (1LL << 32)) return false;
+  if (ldb_n == 1) return ldb_k % 8 == 0 && ldb_k * 4 < (1LL << 31);               // row-major B
+  if (ldb_k == 1) return ldb_n % 8 == 0 && ldb_n >= K && N * ldb_n * 2 < (1LL << 32);  // column-major B (B^T rows of K)
+  return false;
 }
 
 static int mm_pick_split(int64_t M, int64_t N, int64_t K, int split_k) {
@@ -135,7 +137,7 @@ static void mm_launch_general(const void* a, const void* b, void* c, int64_t M, 
                      (long)lda, (long)ldb_k, (long)ldb_n, (long)ldc, bias, bias_f32, relu);
 }
 
-template <bool BF>
+template <bool BF, bool BCOL>
 static void mm_launch_fast(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k,
                            int64_t ldc, const void* bias, int bias_f32, int relu, int out_dtype, int splits, void* ws, hipStream_t s) {
   typedef typename Mfma16<BF>::T T16;
@@ -145,14 +147,14 @@ static void mm_launch_fast(const void* a, const void* b, void* c, int64_t M, int
   const bool partial = splits > 1 || (out_dtype == HX_F32 && (bias || relu));
   if (!partial && out_dtype != HX_F32) {
     d.ldc = ldc;
-    hipLaunchKernelGGL((hx_gemm16_tile256<BF, 1>), dim3(tiles_m * tiles_n), dim3(256), 0, s, (const uint8_t*)a, (const uint8_t*)b, c,
+    hipLaunchKernelGGL((hx_gemm16_tile256<BF, 1, BCOL>), dim3(tiles_m * tiles_n), dim3(256), 0, s, (const uint8_t*)a, (const uint8_t*)b, c,
                        (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M, (int)K, (int)N, tiles_m, tiles_n, 1, d);
     return;
   }
   const int nkt = (int)(K / MOE_BK);
   d.kt_per_split = (nkt + splits - 1) / splits;
   d.ldc = partial ? N : ldc;
-  hipLaunchKernelGGL((hx_gemm16_tile256<BF, 2>), dim3(tiles_m * tiles_n, splits), dim3(256), 0, s, (const uint8_t*)a, (const uint8_t*)b,
+  hipLaunchKernelGGL((hx_gemm16_tile256<BF, 2, BCOL>), dim3(tiles_m * tiles_n, splits), dim3(256), 0, s, (const uint8_t*)a, (const uint8_t*)b,
                      partial ? ws : c, (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M, (int)K, (int)N, tiles_m,
                      tiles_n, 1, d);
   if (!partial) return;
@@ -218,8 +220,15 @@ extern "C" int hx_matmul(const void* a, const void* b, void* c, int64_t M, int64
       }
       splits = 1;  // automatic split without room for it: one pass
     }
-    if (in_dtype == HX_BF16) mm_launch_fast<true>(a, b, c, M, N, K, lda, ldb_k, ldc, bias, bias_f32, relu, out_dtype, splits, workspace, s);
-    else mm_launch_fast<false>(a, b, c, M, N, K, lda, ldb_k, ldc, bias, bias_f32, relu, out_dtype, splits, workspace, s);
+    const bool bcol = ldb_n != 1;  // column-major B: its leading dimension is ldb_n
+    const int64_t ldb = bcol ? ldb_n : ldb_k;
+    if (in_dtype == HX_BF16) {
+      if (bcol) mm_launch_fast<true, true>(a, b, c, M, N, K, lda, ldb, ldc, bias, bias_f32, relu, out_dtype, splits, workspace, s);
+      else mm_launch_fast<true, false>(a, b, c, M, N, K, lda, ldb, ldc, bias, bias_f32, relu, out_dtype, splits, workspace, s);
+    } else {
+      if (bcol) mm_launch_fast<false, true>(a, b, c, M, N, K, lda, ldb, ldc, bias, bias_f32, relu, out_dtype, splits, workspace, s);
+      else mm_launch_fast<false, false>(a, b, c, M, N, K, lda, ldb, ldc, bias, bias_f32, relu, out_dtype, splits, workspace, s);
+    }
   } else if (in_dtype == HX_F32) {
     mm_launch_general<float, float>(a, b, c, M, N, K, lda, ldb_k, ldb_n, ldc, bias, 1, relu, s);
   } else if (in_dtype == HX_BF16) {

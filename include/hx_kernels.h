@@ -154,8 +154,9 @@ size_t hx_fp8_quantize_workspace_bytes(int64_t n);
  * `matmul_split_k(x, y, epilogue)` (examples/matmul_split_k.py:30-68) for the epilogues its examples and tests use
  * (identity, `acc + bias[tile[1]]`, `relu(acc + bias[tile[1]])`: examples/matmul.py:96-119, test/test_examples.py:143-200):
  *   c[M,N] = cast( act( fp32(a[M,K]) @ fp32(b[K,N]) + bias[N] ) ),  fp32 accumulation, act = relu if `relu` else identity.
- * in_dtype: HX_BF16 / HX_F16 (MFMA tile kernel when b is row-major (ldb_n == 1), K % 64 == 0, N % 8 == 0, lda % 8 == 0,
- * ldb_k % 8 == 0, ldc % 4 == 0 and all pointers are 16-byte aligned) or HX_F32 (plain fp32 kernel, as is everything the
+ * in_dtype: HX_BF16 / HX_F16 (MFMA tile kernel when b is row-major (ldb_n == 1) or column-major (ldb_k == 1, e.g. the
+ * transpose of a linear layer's [N, K] weight), K % 64 == 0, N % 8 == 0, lda % 8 == 0, its leading dimension % 8 == 0,
+ * ldc % 4 == 0 and all pointers are 16-byte aligned) or HX_F32 (plain fp32 kernel, as is everything the
  * tile kernel does not cover).  out_dtype: in_dtype, or HX_F32 for the raw accumulator an arbitrary epilogue can be
  * applied to by the caller.  bias: null or [N] in in_dtype or HX_F32 (bias_dtype).
  * split_k: 1 = every workgroup runs the whole K; n > 1 = K split n ways (fewer if K / 64 < n); 0 = the library picks

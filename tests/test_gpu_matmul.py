@@ -42,6 +42,23 @@ def test_shapes_and_epilogues_vs_oracle(m, k, n, path, dtype):
         assert rel_err(out, orc.matmul(x, y, **kw)) <= 1e-2
 
 
+@pytest.mark.parametrize("m,k,n", [(256, 256, 256), (300, 192, 200), (1000, 512, 1016), (64, 4096, 72), (1, 64, 8)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_column_major_y_in_place(m, k, n, dtype):
+    """y given as the transpose of an [n, k] weight (what `x @ w.T` of a linear layer passes): read in place by the tile
+    kernel, bit-identical to the row-major result (same MFMA operands in the same order)."""
+    x, y, bias = _mk(m, k, n, dtype, m + k + n)
+    xd, bd = x.to(DEV), bias.to(DEV)
+    w = y.t().contiguous().to(DEV)            # [n, k]
+    yc = w.t()                                # [k, n] with strides (1, k)
+    assert _path(xd, yc) == 1
+    for ep, kw in ((None, {}), (bias_relu(bd), dict(bias=bias, relu=True))):
+        out = hx.matmul(xd, yc, ep)
+        assert rel_err(out, orc.matmul(x, y, **kw)) <= 1e-2
+        assert torch.equal(out, hx.matmul(xd, y.to(DEV), ep))
+    assert torch.equal(hx.matmul_split_k(xd, yc, split_k=2), hx.matmul_split_k(xd, y.to(DEV), split_k=2))
+
+
 def test_callable_epilogues_match_fused_ones():
     """The reference's own lambdas (examples/matmul.py:98,108-110; test/test_examples.py:143-200, bias of shape [1, n]
     indexed by the whole tile tuple) give what the fused epilogue objects give."""
@@ -96,7 +113,9 @@ def test_strided_operands_and_tritonbench_wrappers():
     ref = orc.matmul(x, y, bias)
     wide = torch.zeros(300, 512, dtype=torch.bfloat16, device=DEV); wide[:, :256] = xd
     assert rel_err(hx.matmul(wide[:, :256], yd, bias_add(bd)), ref) <= 1e-2        # lda > K: read in place
-    yt = yd.t().contiguous().t()                                                    # column-major y: plain kernel
+    yt = yd.t().contiguous().t()[:, ::2]                                            # strided in both dimensions: plain kernel
+    assert rel_err(hx.matmul(xd, yt, bias_add(bd[::2])), orc.matmul(x, y[:, ::2], bias[::2])) <= 1e-2
+    yt = yd.t().contiguous().t()                                                    # column-major y: tile kernel
     assert rel_err(hx.matmul(xd, yt, bias_add(bd)), ref) <= 1e-2
     assert rel_err(hx.matmul_tritonbench(xd, yd, bd)(), ref) <= 1e-2
     assert rel_err(hx.matmul_tritonbench(xd, yd, None)(), orc.matmul(x, y)) <= 1e-2
