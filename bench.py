@@ -198,11 +198,11 @@ def bench_siblings(steps, warmup):
     out = {}
     n_it, n_w = min(steps, 30), min(warmup, 10)
 
-    def mfma(flops, ms, kernel, workload):
+    def mfma(flops, ms, kernel, workload, traffic=None):
         tf = flops / (ms * 1e-3) / 1e12
         return {"workload": workload, "ms_per_launch": ms, "value": tf, "unit": "TFLOP/s",
                 "roofline": {"bound": "mfma", "achieved": tf, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tf / PEAK_BF16_TFLOPS,
-                             "traffic": None, "kernel": kernel, "avg_launch_ms": ms, "algorithmic_flops_per_launch": float(flops)}}
+                             "traffic": traffic, "kernel": kernel, "avg_launch_ms": ms, "algorithmic_flops_per_launch": float(flops)}}
 
     g = torch.Generator(device="cuda").manual_seed(5)
     x = torch.randn(8192, 8192, device="cuda", generator=g).to(torch.bfloat16)
@@ -211,7 +211,7 @@ def bench_siblings(steps, warmup):
     ep = bias_relu(bias)
     ms, _ = _time_launches(lambda: hx.matmul(x, y, ep), n_it, n_w)
     out["matmul_bf16_bias_relu"] = mfma(2.0 * 8192**3, ms, "hx_gemm16_tile256<bf16, dense + epilogue>",
-                                        "matmul 8192^3 bf16, relu(acc + bias) fused, row-major operands")
+                                        "matmul 8192^3 bf16, relu(acc + bias) fused, row-major operands", _traffic("gemm16_dense_8192"))
     del x, y, bias
     x = torch.randn(64, 32768, device="cuda", generator=g).to(torch.float16)
     y = torch.randn(32768, 64, device="cuda", generator=g).to(torch.float16)
@@ -223,7 +223,7 @@ def bench_siblings(steps, warmup):
         q, k, v = (torch.randn(4, 32, 4096, d, device="cuda", generator=g).to(torch.bfloat16) for _ in range(3))
         ms, _ = _time_launches(lambda: hx.attention(q, k, v), n_it, n_w)
         out[f"attention_bf16_d{d}"] = mfma(4.0 * 4 * 32 * 4096 * 4096 * d, ms, f"hx_attention16_kernel<{d}, bf16>",
-                                           f"attention B4 H32 S4096 D{d} bf16 non-causal; flops counted as 4*B*H*S^2*D")
+                                           f"attention B4 H32 S4096 D{d} bf16 non-causal; flops counted as 4*B*H*S^2*D", _traffic(f"attention16_d{d}"))
         del q, k, v
     return out
 

@@ -122,15 +122,21 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
     for (int i = 0; i < 16; ++i) issue_one(kt, stage, i);
   };
 
-  // ---- MFMA operand addressing (16x16x128: lane = row/column lane%16, k = 32*(lane/16) .. +31 of the 128-byte k-tile)
+  // ---- MFMA operand addressing (16x16x128: lane = row/column lane%16, k-slots 32*(lane/16) .. +31)
+  // The product does not care which 32 of the 128 k a lane group multiplies as long as A and B agree, and the LDS
+  // serves a 16-byte read in four passes of the lanes {0-3, 12-15, 20-23, 24-27}, the same + 32, {4-7, 8-11, 16-19,
+  // 28-31}, the same + 32.  With lane group gq on k-block gq, rows 0-3 of group 0 and rows 4-7 of group 1 meet in one
+  // pass on the same banks (measured: every fragment read took twice its cycles); with k-blocks 0, 3, 1, 2 for groups
+  // 0..3 the sixteen lanes of every pass land in sixteen different 16-byte bank groups.
   const int r16 = lane & 15, gq = lane >> 4;
-  const int x16 = ((2 * gq) ^ ((r16 >> 1) & 7)) * 16;  // chunk 2gq of the row, swizzled; chunk 2gq+1 is at x16 ^ 16
+  const int kq = (gq >> 1) ^ ((gq & 1) * 3);             // k-block (32 k) of this lane group
+  const int x16 = ((2 * kq) ^ ((r16 >> 1) & 7)) * 16;  // chunk 2kq of the row, swizzled; chunk 2kq+1 is at x16 ^ 16
   const int a_base = (wm * 128 + r16) * 128;
   const int b_base = (wn * 128 + r16) * 128;
-  // row-major B: transposing read j (0..3) of column block bj fetches k = 32gq + 8j .. +7; this lane supplies 8 bytes of
+  // row-major B: transposing read j (0..3) of column block bj fetches k = 32kq + 8j .. +7; this lane supplies 8 bytes of
   // row (that k) + (lane%16)/2, columns 8*(lane&1) .. +7 of the block's 16-byte chunk, and receives column lane%16.
   // The chunk index wn*8 + bj enters by xor, which commutes with the swizzle's xor.
-  const int bt_off = (32 * gq + (r16 >> 1)) * 256 + ((((r16 >> 1) << 1) | (gq & 1)) * 16) + (lane & 1) * 8;
+  const int bt_off = (32 * kq + (r16 >> 1)) * 256 + ((((r16 >> 1) << 1) | (kq & 1)) * 16) + (lane & 1) * 8;
 
   // acc[bj][bi][r] is C[m0 + wm*128 + 16 bi + lane%16][n0 + wn*128 + 16 bj + 4*(lane/16) + r]
   v4f acc[8][8];
