@@ -55,12 +55,15 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restri
   // [stage][A|W][32 KB]
   __shared__ __attribute__((aligned(1024))) uint8_t smem[2][2][MOE_TILE_BYTES];
 
-  // XCD-contiguous grouped raster over (row tile, column tile), as in the fp8 GEMM
+  // Grouped raster over (row tile, column tile), 8 row tiles tall.  Workgroup i runs on XCD i % 8; each run of 256
+  // workgroups covers 256 consecutive tiles of that order, 32 consecutive ones (8 row tiles x 4 column tiles) per XCD,
+  // so one XCD's resident tiles share operand panels in its L2 and all eight XCDs work side by side on the same row
+  // tiles and on neighbouring column panels of the same expert — the set of panels in flight then fits the memory-side
+  // cache, which a contiguous range of the tile order per XCD (eight different experts at once) does not (C5: -6 %).
   int tile;
   {
-    const int nwg = gridDim.x, wg = blockIdx.x;
-    const int per = nwg >> 3, rem = nwg & 7, xcd = wg & 7, loc = wg >> 3;
-    tile = (xcd < rem) ? xcd * (per + 1) + loc : rem * (per + 1) + (xcd - rem) * per + loc;
+    const int nwg = gridDim.x, wg = blockIdx.x, chunk = wg >> 8;
+    tile = chunk < (nwg >> 8) ? (chunk << 8) + ((wg & 7) << 5) + ((wg >> 3) & 31) : wg;
   }
   const int GM = 8;
   const int group_size = GM * tiles_n;
