@@ -29,6 +29,23 @@ def i16(t):
     return t.contiguous().view(torch.int16).numpy()
 
 
+def siblings(g):
+    """16-bit siblings: matmul 96x64x72 with bias and relu, attention M=80 N=100 D=64 (ragged) and M=N=64 D=128, one head each."""
+    out = {}
+    for name, dt in {"bf16": torch.bfloat16, "f16": torch.float16}.items():
+        x = torch.randn(96, 64, generator=g).to(dt); y = torch.randn(64, 72, generator=g).to(dt)
+        bias = torch.randn(72, generator=g).to(dt)
+        out[f"mm_{name}_x"] = i16(x); out[f"mm_{name}_y"] = i16(y); out[f"mm_{name}_bias"] = i16(bias)
+        out[f"mm_{name}_out"] = i16(orc.matmul(x, y))
+        out[f"mm_{name}_out_bias_relu"] = i16(orc.matmul(x, y, bias, relu=True))
+        for tag, (bh, m, n, d) in {"d64": (1, 80, 100, 64), "d128": (1, 64, 64, 128)}.items():
+            q = torch.randn(bh, m, d, generator=g).to(dt); k = torch.randn(bh, n, d, generator=g).to(dt)
+            v = torch.randn(bh, n, d, generator=g).to(dt)
+            out[f"att_{name}_{tag}_q"] = i16(q); out[f"att_{name}_{tag}_k"] = i16(k); out[f"att_{name}_{tag}_v"] = i16(v)
+            out[f"att_{name}_{tag}_out"] = i16(orc.attention(q, k, v))
+    np.savez_compressed(HERE / "siblings_small.npz", **out)
+
+
 def main():
     g = torch.Generator().manual_seed(1234)
     # fp8 gemm: 48x40x96 (ragged, general kernel) and 16x64x256 (skinny) with scales
@@ -62,6 +79,7 @@ def main():
         out[f"{name}_A"] = i16(A); out[f"{name}_W"] = i16(W); out[f"{name}_expert"] = ex.numpy().astype(np.int64)
         out[f"{name}_out"] = i16(orc.moe_matmul_ogs(*orc.moe_args_gen(A, W, ex)))
     np.savez_compressed(HERE / "moe_small.npz", **out)
+    siblings(torch.Generator().manual_seed(4321))
     for f in sorted(HERE.glob("*.npz")):
         print(f.name, f.stat().st_size, "bytes")
 

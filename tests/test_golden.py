@@ -40,3 +40,15 @@ def test_moe_fixture():
         ex = torch.from_numpy(z[f"{name}_expert"].copy())
         got = orc.moe_matmul_ogs(*orc.moe_args_gen(A, W, ex)).view(torch.int16).numpy()
         assert np.array_equal(got, z[f"{name}_out"])
+
+
+def test_siblings_fixture():
+    z = np.load(G / "siblings_small.npz")
+    for name, dt in (("bf16", torch.bfloat16), ("f16", torch.float16)):
+        t = lambda key: torch.from_numpy(z[key].copy()).view(dt)
+        x, y, bias = t(f"mm_{name}_x"), t(f"mm_{name}_y"), t(f"mm_{name}_bias")
+        assert np.array_equal(orc.matmul(x, y).view(torch.int16).numpy(), z[f"mm_{name}_out"])
+        assert np.array_equal(orc.matmul(x, y, bias, relu=True).view(torch.int16).numpy(), z[f"mm_{name}_out_bias_relu"])
+        for tag in ("d64", "d128"):
+            q, k, v = (t(f"att_{name}_{tag}_{c}") for c in "qkv")
+            assert np.array_equal(orc.attention(q, k, v).view(torch.int16).numpy(), z[f"att_{name}_{tag}_out"])

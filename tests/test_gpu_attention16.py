@@ -1,6 +1,9 @@
 """GPU parity of hx_attention (the 16-bit sibling of the fp8 attention: examples/attention.py of the reference) against
 the CPU oracle, through the C ABI via the registered op.  Bar: max|out - ref| <= 2e-2 max|ref| after rounding to the
 output dtype."""
+import pathlib
+
+import numpy as np
 import pytest
 import torch
 
@@ -101,3 +104,13 @@ def test_seeded_random_sweep():
         q, k, v = _mk((bh, m, d), n, dtype, int(torch.randint(0, 1 << 30, (1,), generator=g)))
         out = hx.attention(q.to(DEV), k.to(DEV), v.to(DEV))
         assert rel_err(out, orc.attention(q, k, v)) <= 2e-2, (bh, m, n, d, dtype)
+
+
+def test_golden_fixture():
+    """Frozen oracle outputs (tests/golden/siblings_small.npz): an anchor that does not run the oracle code."""
+    z = np.load(pathlib.Path(__file__).resolve().parent / "golden" / "siblings_small.npz")
+    for name, dt in (("bf16", torch.bfloat16), ("f16", torch.float16)):
+        t = lambda key: torch.from_numpy(z[key].copy()).view(dt)
+        for tag in ("d64", "d128"):
+            q, k, v = (t(f"att_{name}_{tag}_{c}").to(DEV) for c in "qkv")
+            assert rel_err(hx.attention(q, k, v), t(f"att_{name}_{tag}_out")) <= 2e-2

@@ -1,6 +1,9 @@
 """GPU parity of hx_matmul (the 16-bit siblings of the fp8 GEMM: examples/matmul.py, examples/matmul_split_k.py of the
 reference) against the CPU oracle, through the C ABI via the registered op.  Bar: max|out - ref| <= 2e-2 max|ref|
 after rounding to the output type (the 16-bit kernels differ from the oracle only in fp32 summation order)."""
+import pathlib
+
+import numpy as np
 import pytest
 import torch
 
@@ -134,3 +137,13 @@ def test_errors_and_empty():
     k0 = hx.matmul(torch.zeros(4, 0, dtype=torch.float16, device=DEV), torch.zeros(0, 8, dtype=torch.float16, device=DEV),
                    bias_add(torch.ones(8, dtype=torch.float16, device=DEV)))
     assert torch.equal(k0, torch.ones(4, 8, dtype=torch.float16, device=DEV))      # empty sum + bias
+
+
+def test_golden_fixture():
+    """Frozen oracle outputs (tests/golden/siblings_small.npz): an anchor that does not run the oracle code."""
+    z = np.load(pathlib.Path(__file__).resolve().parent / "golden" / "siblings_small.npz")
+    for name, dt in (("bf16", torch.bfloat16), ("f16", torch.float16)):
+        t = lambda key: torch.from_numpy(z[key].copy()).view(dt)
+        x, y, bias = (t(f"mm_{name}_{c}").to(DEV) for c in ("x", "y", "bias"))
+        assert rel_err(hx.matmul(x, y), t(f"mm_{name}_out")) <= 1e-2
+        assert rel_err(hx.matmul(x, y, bias_relu(bias)), t(f"mm_{name}_out_bias_relu")) <= 1e-2
