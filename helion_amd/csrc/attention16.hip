@@ -418,7 +418,7 @@ extern "C" int hx_attention(const void* q, const void* k, const void* v, void* o
     hx_set_error("hx_attention: null pointer");
     return HX_ERR_BAD_ARG;
   }
-  if (BH >= 65536 || M >= (1LL << 31) || N >= (1LL << 31) || BH * M * D >= (1LL << 40) || BH * N * D >= (1LL << 40)) {
+  if (M >= (1LL << 31) || N >= (1LL << 31) || BH * M * D >= (1LL << 40) || BH * N * D >= (1LL << 40)) {
     hx_set_error("hx_attention: problem too large");
     return HX_ERR_UNSUPPORTED;
   }
@@ -432,8 +432,9 @@ extern "C" int hx_attention(const void* q, const void* k, const void* v, void* o
       else launch_att16<64, false>(q, k, v, out, BH, M, N, s);
     }
   } else {
-    if (D > 256) {
-      hx_set_error("hx_attention: head dimension %lld > 256 is not supported", (long long)D);
+    if (D > 256 || BH >= 65536) {
+      hx_set_error("hx_attention: unsupported shape D=%lld BH=%lld (plain kernel: head dimension <= 256, batch*heads < 65536)",
+                   (long long)D, (long long)BH);
       return HX_ERR_UNSUPPORTED;
     }
     const dim3 grid((unsigned)M, (unsigned)BH);

@@ -356,6 +356,68 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// general: any S, D <= 256, any V strides; one workgroup per query row, exact row max (two sweeps over the keys),
+// p quantised to e4m3 against it, l from the un-quantised p.  Correctness path for the shapes the MFMA kernel does
+// not take; it always computes the exact-max form.
+// ------------------------------------------------------------------------------------------
+template <int OUT>
+__global__ __launch_bounds__(256) void hx_fp8_attention_general(const uint8_t* __restrict__ Q, const uint8_t* __restrict__ Kt,
+                                                               const uint8_t* __restrict__ Vt, void* __restrict__ Out, int S, int D,
+                                                               long vsd, long vss) {
+  constexpr int CH = 1024;
+  __shared__ float sq[256];
+  __shared__ float sp[CH];
+  __shared__ float red[256];
+  const int tid = threadIdx.x;
+  const long bh = blockIdx.y, qi = blockIdx.x;
+  const uint8_t* Kh = Kt + bh * (long)S * D;
+  const uint8_t* Vh = Vt + bh * (long)S * D;
+  if (tid < D) sq[tid] = hx_e4m3_to_f32(Q[(bh * S + qi) * D + tid]);
+  __syncthreads();
+  auto score = [&](int key) {
+    const uint8_t* kr = Kh + (long)key * D;
+    float s = 0.f;
+    for (int d = 0; d < D; ++d) s = __builtin_fmaf(sq[d], hx_e4m3_to_f32(kr[d]), s);
+    return s;
+  };
+  auto block_reduce = [&](float v, bool is_max) {
+    red[tid] = v;
+    __syncthreads();
+    for (int st = 128; st > 0; st >>= 1) {
+      if (tid < st) red[tid] = is_max ? fmaxf(red[tid], red[tid + st]) : red[tid] + red[tid + st];
+      __syncthreads();
+    }
+    const float r = red[0];
+    __syncthreads();
+    return r;
+  };
+  const float c = (float)((1.0 / __builtin_sqrt((double)D)) * 1.44269504);
+  float smax = -__builtin_inff();
+  for (int key = tid; key < S; key += 256) smax = fmaxf(smax, score(key));
+  const float neg_m = -(block_reduce(smax, true) * c);
+  float lsum = 0.f, acc = 0.f;
+  for (int n0 = 0; n0 < S; n0 += CH) {
+    const int cn = min(CH, S - n0);
+    for (int i = tid; i < cn; i += 256) {
+      const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(score(n0 + i), c, neg_m));
+      lsum += p;
+      sp[i] = hx_e4m3_to_f32((uint8_t)(HX_CVT_PK_E4M3(p, 0.f, 0, false) & 0xFF));
+    }
+    __syncthreads();
+    if (tid < D)
+      for (int i = 0; i < cn; ++i) acc = __builtin_fmaf(sp[i], hx_e4m3_to_f32(Vh[(long)tid * vsd + (long)(n0 + i) * vss]), acc);
+    __syncthreads();
+  }
+  const float l = block_reduce(lsum, false);
+  if (tid < D) {
+    const float o = acc / l;
+    const long at = (bh * S + qi) * D + tid;
+    if (OUT == HX_F32) ((float*)Out)[at] = o;
+    else ((uint8_t*)Out)[at] = (uint8_t)(HX_CVT_PK_E4M3(o, 0.f, 0, false) & 0xFF);
+  }
+}
+
 template <int D, int OUT, bool EXACT, bool VSD>
 static void launch_att_kernel(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t S, hipStream_t s) {
   const int qtiles = (int)((S + ATT_BM - 1) / ATT_BM);
@@ -397,28 +459,35 @@ extern "C" int hx_fp8_attention(const void* q, const void* k, const void* v, voi
     hx_set_error("hx_fp8_attention: out_dtype must be HX_E4M3 or HX_F32, got %d", out_dtype);
     return HX_ERR_BAD_ARG;
   }
-  if ((D != 64 && D != 128) || (S % ATT_BN) != 0) {
-    hx_set_error("hx_fp8_attention: unsupported shape S=%lld D=%lld (need D in {64,128}, S %% 64 == 0)", (long long)S,
-                 (long long)D);
-    return HX_ERR_UNSUPPORTED;
-  }
-  bool vsd;
-  if (v_stride_s == 1 && (v_stride_d == S || D == 1)) vsd = false;       // [D][S] per head
-  else if (v_stride_d == 1 && (v_stride_s == D || S == 1)) vsd = true;   // [S][D] per head
-  else {
-    hx_set_error("hx_fp8_attention: v strides (d: %lld, s: %lld) are neither [D][S] (S, 1) nor [S][D] (1, D) per head",
-                 (long long)v_stride_d, (long long)v_stride_s);
-    return HX_ERR_UNSUPPORTED;
-  }
-  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) {
-    hx_set_error("hx_fp8_attention: pointers must be 16-byte aligned");
-    return HX_ERR_UNSUPPORTED;
-  }
   if (BH * S * D >= (1LL << 40) || S * D >= (1LL << 31)) {
     hx_set_error("hx_fp8_attention: problem too large");
     return HX_ERR_UNSUPPORTED;
   }
   hipStream_t s = (hipStream_t)stream;
+  bool vsd = false, fast = (D == 64 || D == 128) && (S % ATT_BN) == 0 && ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) == 0);
+  if (v_stride_s == 1 && (v_stride_d == S || D == 1)) vsd = false;       // [D][S] per head
+  else if (v_stride_d == 1 && (v_stride_s == D || S == 1)) vsd = true;   // [S][D] per head
+  else fast = false;
+  if (!fast) {  // any other shape, alignment or V striding within a head (heads are D*S elements apart)
+    if (D > 256 || D < 1 || BH >= 65536) {
+      hx_set_error("hx_fp8_attention: unsupported shape S=%lld D=%lld BH=%lld (MFMA kernel: D in {64,128}, S %% 64 == 0; plain kernel: D <= 256, BH < 65536)",
+                   (long long)S, (long long)D, (long long)BH);
+      return HX_ERR_UNSUPPORTED;
+    }
+    const dim3 grid((unsigned)S, (unsigned)BH);
+    if (out_dtype == HX_F32)
+      hipLaunchKernelGGL(hx_fp8_attention_general<HX_F32>, grid, dim3(256), 0, s, (const uint8_t*)q, (const uint8_t*)k, (const uint8_t*)v,
+                         out, (int)S, (int)D, (long)v_stride_d, (long)v_stride_s);
+    else
+      hipLaunchKernelGGL(hx_fp8_attention_general<HX_E4M3>, grid, dim3(256), 0, s, (const uint8_t*)q, (const uint8_t*)k,
+                         (const uint8_t*)v, out, (int)S, (int)D, (long)v_stride_d, (long)v_stride_s);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+      hx_set_error("hx_fp8_attention: launch failed: %s", hipGetErrorString(e));
+      return (int)e;
+    }
+    return 0;
+  }
   if (D == 128) {
     if (out_dtype == HX_F32) return launch_att<128, HX_F32>(q, k, v, out, BH, S, exact_max, vsd, s);
     return launch_att<128, HX_E4M3>(q, k, v, out, BH, S, exact_max, vsd, s);

@@ -82,7 +82,9 @@ int hx_fp8_gemm_path(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k
  * exact_max != 0: two passes, P is quantised to e4m3 against the exact row max (bit-faithful to
  *   the reference's ref-eager execution); exact_max == 0: one pass, online softmax, P quantised
  *   against the running max (what the reference's compiled kernel does).
- * Supported: D == 128 or 64, S % 64 == 0. */
+ * MFMA kernel: D == 128 or 64, S % 64 == 0, 16-byte aligned pointers, v in one of the two layouts above.  Every other
+ * shape with D <= 256 and BH < 65536 (and any v strides within a head) runs a plain kernel that always computes the
+ * exact-max form. */
 int hx_fp8_attention(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t S,
                      int64_t D, int64_t v_stride_d, int64_t v_stride_s, int out_dtype, int exact_max, void* stream);
 

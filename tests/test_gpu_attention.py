@@ -83,10 +83,25 @@ def test_tritonbench_thunk_and_layout():
     assert rel_err(out, orc.fp8_attention(q8, k8, v8, 2, 3)) <= 0.08
 
 
+@pytest.mark.parametrize("b,h,s,d", [(1, 2, 100, 64), (2, 1, 70, 80), (1, 3, 64, 32), (1, 1, 1, 16), (1, 2, 1100, 128), (1, 1, 130, 256)])
+def test_other_shapes_run_the_plain_kernel(b, h, s, d):
+    """Sequence lengths that are not a multiple of 64 and head dims other than 64 / 128: exact-max form, both V layouts,
+    both output types."""
+    q, k, v = inputs.attention_inputs(b, h, s, d, seed=s + d)
+    ref32 = orc.fp8_attention(q, k, v, b, h, torch.float32)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    out = hx.fp8_attention_kernel(qd, kd, vd, b, h, out_dtype=torch.float32)
+    assert rel_err(out, ref32) <= 2e-2
+    v_sd = vd.transpose(1, 2).contiguous().transpose(1, 2)           # [BH, D, S] view of [BH, S, D] memory
+    assert rel_err(hx.fp8_attention_kernel(qd, kd, v_sd, b, h, out_dtype=torch.float32), ref32) <= 2e-2
+    out8 = hx.fp8_attention_kernel(qd, kd, vd, b, h)
+    assert out8.dtype == E4M3 and rel_err(out8, orc.fp8_attention(q, k, v, b, h)) <= 0.08
+
+
 def test_unsupported_shapes_raise():
-    x = torch.zeros(1, 100, 64).to(E4M3).to(DEV)
+    x = torch.zeros(1, 64, 320).to(E4M3).to(DEV)
     with pytest.raises(ValueError, match="unsupported shape"):
-        hx.fp8_attention_kernel(x, x, torch.zeros(1, 64, 100).to(E4M3).to(DEV), 1, 1)
+        hx.fp8_attention_kernel(x, x, torch.zeros(1, 320, 64).to(E4M3).to(DEV), 1, 1)   # head dim > 256
     y = torch.zeros(2, 64, 64).to(E4M3).to(DEV)
     with pytest.raises(ValueError):
         hx.fp8_attention_kernel(y, y, y, 1, 1)  # batch*heads mismatch
