@@ -18,7 +18,18 @@ def _cases():
     A, W, ex = inputs.moe_inputs(300, 128, 256, 6, 2, seed=3)
     A, W, ex = A.to(DEV), W.to(DEV), ex.to(DEV)
     x = torch.randn(1000, 333, device=DEV, dtype=torch.bfloat16)
+    g = torch.Generator(device=DEV).manual_seed(4)
+    mx = torch.randn(300, 1024, device=DEV, generator=g).to(torch.float16)
+    my = torch.randn(1024, 264, device=DEV, generator=g).to(torch.float16)
+    mb = torch.randn(264, device=DEV, generator=g).to(torch.float16)
+    aq, ak, av = (torch.randn(2, 3, 200, 128, device=DEV, generator=g).to(torch.bfloat16) for _ in range(3))
+    from helion_amd.matmul import bias_relu
     return {
+        "matmul_bias_relu": lambda: hx.matmul(mx, my, bias_relu(mb)),
+        "matmul_split_k": lambda: hx.matmul_split_k(mx, my, split_k=4),
+        "attention16": lambda: hx.attention(aq, ak, av),
+        "attention16_ragged_keys": lambda: hx.attention(aq, ak[:, :, :150], av[:, :, :150]),
+        "fp8_attention_plain": lambda: hx.fp8_attention_kernel(q[:, :100], k[:, :100], v[:, :, :100], 1, 4, out_dtype=torch.float32),
         "fp8_gemm": lambda: hx.fp8_gemm(a, b, scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16),
         "fp8_gemm_row_major": lambda: hx.fp8_gemm(a, b.contiguous(), out_dtype=torch.float32),
         "fp8_gemm_skinny": lambda: hx.fp8_gemm(a[:16], b, out_dtype=torch.float32),
