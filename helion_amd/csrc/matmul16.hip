@@ -62,17 +62,28 @@ __global__ __launch_bounds__(256) void hx_matmul_general(const TI* __restrict__ 
   }
 }
 
-// C[m, n..n+3] = cast(act(sum_s part[s][m][n..] + bias[n..])); part is [S][M][N] fp32, N % 4 == 0
+// C[m, n..n+3] = cast(act(sum_s part[s][m][n..] + bias[n..])); part is [S][M][N] fp32, N % 4 == 0.
+// A workgroup covers 16 groups of 4 columns; 16 threads share each group's splits (s = lane, lane + 16, ...: many
+// splits of a small output would otherwise be one long chain of loads per thread) and are summed through LDS in a
+// fixed order, so the result does not depend on the launch.
 template <typename TB, typename TO>
 __global__ __launch_bounds__(256) void hx_matmul16_reduce(const float* __restrict__ part, int S, int M, int N, TO* __restrict__ C,
                                                          long ldc, const void* __restrict__ bias, int bias_f32, int relu) {
-  const long q = (long)blockIdx.x * 256 + threadIdx.x;  // group of 4 columns
+  __shared__ v4f red[16][16];
+  const int gl = threadIdx.x & 15, sl = threadIdx.x >> 4;
+  const long q = (long)blockIdx.x * 16 + gl;  // group of 4 columns
   const int nq = N >> 2;
-  if (q >= (long)M * nq) return;
-  const long m = q / nq, n = (q % nq) * 4;
+  const bool live = q < (long)M * nq;
+  const long m = live ? q / nq : 0, n = live ? (q % nq) * 4 : 0;
   const long plane = (long)M * N;
-  v4f v = *(const v4f*)(part + m * N + n);
-  for (int s = 1; s < S; ++s) v += *(const v4f*)(part + s * plane + m * N + n);
+  v4f v = {0.f, 0.f, 0.f, 0.f};
+  if (live)
+    for (int s = sl; s < S; s += 16) v += *(const v4f*)(part + s * plane + m * N + n);
+  red[sl][gl] = v;
+  __syncthreads();
+  if (sl != 0 || !live) return;
+#pragma unroll
+  for (int i = 1; i < 16; ++i) v += red[i][gl];
   if (bias) {
 #pragma unroll
     for (int b = 0; b < 4; ++b) v[b] += bias_f32 ? ((const float*)bias)[n + b] : (float)((const TB*)bias)[n + b];
@@ -159,7 +170,7 @@ static void mm_launch_fast(const void* a, const void* b, void* c, int64_t M, int
                      tiles_n, 1, d);
   if (!partial) return;
   const long groups = M * (N / 4);
-  const dim3 grid((unsigned)((groups + 255) / 256));
+  const dim3 grid((unsigned)((groups + 15) / 16));
   if (out_dtype == HX_F32)
     hipLaunchKernelGGL((hx_matmul16_reduce<T16, float>), grid, dim3(256), 0, s, (const float*)ws, splits, (int)M, (int)N, (float*)c, (long)ldc,
                        bias, bias_f32, relu);
