@@ -52,6 +52,23 @@ def test_ops_refuse_cpu_tensors():
                           torch.zeros(2, dtype=torch.int32), torch.zeros(4, dtype=torch.int32), torch.empty(4))
 
 
+def test_sibling_ops_refuse_cpu_tensors_and_epilogue_objects_are_plain_callables():
+    from helion_amd.matmul import bias_add, bias_relu, relu
+    x = torch.zeros(4, 4).half()
+    with pytest.raises(RuntimeError, match="GPU only"):
+        hx.matmul(x, x)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        hx.attention(x.reshape(1, 4, 4), x.reshape(1, 4, 4), x.reshape(1, 4, 4))
+    # the fused epilogues keep the reference's (acc, tile) calling convention (examples/matmul.py:30-34), so they can be
+    # handed to any matmul that takes such a callable
+    acc = torch.tensor([[-1.0, 2.0, 3.0]]); bias = torch.tensor([0.5, -4.0, 1.0]).half()
+    tile = (slice(0, 1), slice(0, 3))
+    assert torch.equal(bias_add(bias)(acc, tile), acc + bias.float())
+    assert torch.equal(bias_relu(bias)(acc, tile), torch.relu(acc + bias.float()))
+    assert torch.equal(bias_relu(bias.reshape(1, 3))(acc, tile), torch.relu(acc + bias.float()))
+    assert torch.equal(relu()(acc, tile), torch.relu(acc))
+
+
 def test_registered_ops_infer_shapes_on_meta_tensors():
     x = torch.empty(32, 64, dtype=torch.float8_e4m3fn, device="meta")
     y = torch.empty(64, 48, dtype=torch.float8_e4m3fn, device="meta")
@@ -65,6 +82,12 @@ def test_registered_ops_infer_shapes_on_meta_tensors():
     i32 = lambda n: torch.empty(n, dtype=torch.int32, device="meta")
     c = torch.ops.helion_amd.moe_matmul_ogs(A, W, i32(3), i32(4), i32(10), 5)
     assert c.shape == (10, 12) and c.dtype == torch.bfloat16
+    mx = torch.empty(32, 64, dtype=torch.float16, device="meta"); my = torch.empty(64, 48, dtype=torch.float16, device="meta")
+    mo = torch.ops.helion_amd.matmul(mx, my, None, True, torch.float32, 0)
+    assert mo.shape == (32, 48) and mo.dtype == torch.float32
+    aq = torch.empty(2, 3, 100, 64, dtype=torch.bfloat16, device="meta"); ak = torch.empty(2, 3, 70, 64, dtype=torch.bfloat16, device="meta")
+    ao = torch.ops.helion_amd.attention(aq, ak, ak)
+    assert ao.shape == (2, 3, 100, 64) and ao.dtype == torch.bfloat16
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
