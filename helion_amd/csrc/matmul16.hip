@@ -7,7 +7,7 @@
 // the output type and applies the epilogue to the first split only; its result for one split — which is what its eager
 // mode computes — is the formula above, and that is what every split count gives here.
 // Anything the tile kernel does not cover (fp32 operands, odd sizes, strided B) runs a plain fp32-FMA kernel.
-#include "gemm16_tile256.h"
+#include "gemm16_tile128.h"
 
 template <typename T>
 __device__ __forceinline__ float mm_ld(const T* p) { return (float)*p; }
@@ -108,19 +108,32 @@ static bool mm_fast_ok(const void* a, const void* b, const void* c, int64_t M, i
   return false;
 }
 
-static int mm_pick_split(int64_t M, int64_t N, int64_t K, int split_k) {
+// Tile size and K split for a problem the tile kernels take.  256x256 tiles unless they would leave most of the chip
+// idle; an automatic split (split_k <= 0) only while the workgroups do not fill the chip, every split keeps at least
+// eight k-tiles (a split costs a second launch) and the fp32 partial sums, which are written and read again, stay below
+// half the operand bytes.
+struct MmPlan {
+  int tile, splits;
+};
+static MmPlan mm_plan(int64_t M, int64_t N, int64_t K, int split_k) {
   const int64_t nkt = K / MOE_BK;
+  const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
+  MmPlan p;
+  p.tile = t256 >= 128 ? 256 : 128;
+  const int64_t tiles = ((M + p.tile - 1) / p.tile) * ((N + p.tile - 1) / p.tile);
+  const int64_t room = p.tile == 256 ? 256 : 512;  // resident workgroups: one or two per CU
   int64_t s = split_k;
-  if (s <= 0) {  // enough workgroups for the chip, at least four k-tiles each
-    const int64_t tiles = ((M + MOE_BM - 1) / MOE_BM) * ((N + MOE_BN - 1) / MOE_BN);
+  if (s <= 0) {
     s = 1;
-    while (tiles * s * 2 <= 256 && nkt / (s * 2) >= 4) s *= 2;
+    const int64_t cap = (M + N) * K;  // half the operand bytes
+    while (tiles * s * 2 <= room && nkt / (s * 2) >= 8 && (s * 2) * M * N * 4 <= cap) s *= 2;
   }
   if (s > nkt) s = nkt;
   if (s > 65535) s = 65535;
   if (s < 1) s = 1;
   const int64_t per = (nkt + s - 1) / s;
-  return (int)((nkt + per - 1) / per);
+  p.splits = (int)((nkt + per - 1) / per);
+  return p;
 }
 
 extern "C" int hx_matmul_splits(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc, int in_dtype,
@@ -128,14 +141,14 @@ extern "C" int hx_matmul_splits(int64_t M, int64_t N, int64_t K, int64_t lda, in
   if (M <= 0 || N <= 0 || K <= 0) return 1;
   // alignment of the pointers is not known here; the launcher re-checks and falls back to one split
   if (!mm_fast_ok(nullptr, nullptr, nullptr, M, N, K, lda, ldb_k, ldb_n, ldc, nullptr, in_dtype)) return 1;
-  return mm_pick_split(M, N, K, split_k);
+  return mm_plan(M, N, K, split_k).splits;
 }
 
 extern "C" size_t hx_matmul_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
                                             int in_dtype, int out_dtype, int has_epilogue, int split_k) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
   if (!mm_fast_ok(nullptr, nullptr, nullptr, M, N, K, lda, ldb_k, ldb_n, ldc, nullptr, in_dtype)) return 0;
-  const int s = mm_pick_split(M, N, K, split_k);
+  const int s = mm_plan(M, N, K, split_k).splits;
   const bool partial = s > 1 || (out_dtype == HX_F32 && has_epilogue);
   return partial ? (size_t)s * M * N * 4 : 0;
 }
@@ -150,24 +163,34 @@ static void mm_launch_general(const void* a, const void* b, void* c, int64_t M, 
 
 template <bool BF, bool BCOL>
 static void mm_launch_fast(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k,
-                           int64_t ldc, const void* bias, int bias_f32, int relu, int out_dtype, int splits, void* ws, hipStream_t s) {
+                           int64_t ldc, const void* bias, int bias_f32, int relu, int out_dtype, int tile, int splits, void* ws,
+                           hipStream_t s) {
   typedef typename Mfma16<BF>::T T16;
-  const int tiles_m = (int)((M + MOE_BM - 1) / MOE_BM), tiles_n = (int)((N + MOE_BN - 1) / MOE_BN);
+  const int tiles_m = (int)((M + tile - 1) / tile), tiles_n = (int)((N + tile - 1) / tile);
   G16Dense d = {};
   d.lda = lda; d.ldb = ldb_k; d.bias = bias; d.bias_f32 = bias_f32; d.relu = relu;
   const bool partial = splits > 1 || (out_dtype == HX_F32 && (bias || relu));
   if (!partial && out_dtype != HX_F32) {
     d.ldc = ldc;
-    hipLaunchKernelGGL((hx_gemm16_tile256<BF, 1, BCOL>), dim3(tiles_m * tiles_n), dim3(256), 0, s, (const uint8_t*)a, (const uint8_t*)b, c,
-                       (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M, (int)K, (int)N, tiles_m, tiles_n, 1, d);
+    if (tile == 256)
+      hipLaunchKernelGGL((hx_gemm16_tile256<BF, 1, BCOL>), dim3(tiles_m * tiles_n), dim3(256), 0, s, (const uint8_t*)a, (const uint8_t*)b, c,
+                         (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M, (int)K, (int)N, tiles_m, tiles_n, 1, d);
+    else
+      hipLaunchKernelGGL((hx_gemm16_tile128<BF, 1, BCOL>), dim3(tiles_m * tiles_n), dim3(256), 0, s, (const uint8_t*)a, (const uint8_t*)b, c,
+                         (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M, (int)K, (int)N, tiles_m, tiles_n, 1, d);
     return;
   }
   const int nkt = (int)(K / MOE_BK);
   d.kt_per_split = (nkt + splits - 1) / splits;
   d.ldc = partial ? N : ldc;
-  hipLaunchKernelGGL((hx_gemm16_tile256<BF, 2, BCOL>), dim3(tiles_m * tiles_n, splits), dim3(256), 0, s, (const uint8_t*)a, (const uint8_t*)b,
-                     partial ? ws : c, (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M, (int)K, (int)N, tiles_m,
-                     tiles_n, 1, d);
+  if (tile == 256)
+    hipLaunchKernelGGL((hx_gemm16_tile256<BF, 2, BCOL>), dim3(tiles_m * tiles_n, splits), dim3(256), 0, s, (const uint8_t*)a,
+                       (const uint8_t*)b, partial ? ws : c, (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M,
+                       (int)K, (int)N, tiles_m, tiles_n, 1, d);
+  else
+    hipLaunchKernelGGL((hx_gemm16_tile128<BF, 2, BCOL>), dim3(tiles_m * tiles_n, splits), dim3(256), 0, s, (const uint8_t*)a,
+                       (const uint8_t*)b, partial ? ws : c, (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M,
+                       (int)K, (int)N, tiles_m, tiles_n, 1, d);
   if (!partial) return;
   const long groups = M * (N / 4);
   const dim3 grid((unsigned)((groups + 15) / 16));
@@ -221,7 +244,8 @@ extern "C" int hx_matmul(const void* a, const void* b, void* c, int64_t M, int64
   const int bias_f32 = (bias_dtype == HX_F32 || in_dtype == HX_F32) ? 1 : 0;
   bool fast = mm_fast_ok(a, b, c, M, N, K, lda, ldb_k, ldb_n, ldc, bias, in_dtype);
   if (fast) {
-    int splits = mm_pick_split(M, N, K, split_k);
+    const MmPlan plan = mm_plan(M, N, K, split_k);
+    int splits = plan.splits;
     const bool partial = splits > 1 || (out_dtype == HX_F32 && (bias || relu));
     const size_t need = partial ? (size_t)splits * M * N * 4 : 0;
     if (need && (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15))) {
@@ -234,11 +258,11 @@ extern "C" int hx_matmul(const void* a, const void* b, void* c, int64_t M, int64
     const bool bcol = ldb_n != 1;  // column-major B: its leading dimension is ldb_n
     const int64_t ldb = bcol ? ldb_n : ldb_k;
     if (in_dtype == HX_BF16) {
-      if (bcol) mm_launch_fast<true, true>(a, b, c, M, N, K, lda, ldb, ldc, bias, bias_f32, relu, out_dtype, splits, workspace, s);
-      else mm_launch_fast<true, false>(a, b, c, M, N, K, lda, ldb, ldc, bias, bias_f32, relu, out_dtype, splits, workspace, s);
+      if (bcol) mm_launch_fast<true, true>(a, b, c, M, N, K, lda, ldb, ldc, bias, bias_f32, relu, out_dtype, plan.tile, splits, workspace, s);
+      else mm_launch_fast<true, false>(a, b, c, M, N, K, lda, ldb, ldc, bias, bias_f32, relu, out_dtype, plan.tile, splits, workspace, s);
     } else {
-      if (bcol) mm_launch_fast<false, true>(a, b, c, M, N, K, lda, ldb, ldc, bias, bias_f32, relu, out_dtype, splits, workspace, s);
-      else mm_launch_fast<false, false>(a, b, c, M, N, K, lda, ldb, ldc, bias, bias_f32, relu, out_dtype, splits, workspace, s);
+      if (bcol) mm_launch_fast<false, true>(a, b, c, M, N, K, lda, ldb, ldc, bias, bias_f32, relu, out_dtype, plan.tile, splits, workspace, s);
+      else mm_launch_fast<false, false>(a, b, c, M, N, K, lda, ldb, ldc, bias, bias_f32, relu, out_dtype, plan.tile, splits, workspace, s);
     }
   } else if (in_dtype == HX_F32) {
     mm_launch_general<float, float>(a, b, c, M, N, K, lda, ldb_k, ldb_n, ldc, bias, 1, relu, s);

@@ -11,7 +11,7 @@
 //   3. hx_moe_tile256 / hx_moe_general : the grouped GEMM over (row tile, column tile) pairs;
 //   4. hx_moe_zero_rows  : zero-fills rows whose flag is still clear.
 // Padded rows of a tile are never stored, so there is no read-modify-write and no write race.
-#include "gemm16_tile256.h"
+#include "gemm16_tile128.h"
 
 // workspace layout: [0] int num_tiles | [16 ..) MoeTile table[max_tiles] | flags[T] bytes
 static inline size_t moe_table_bytes(int64_t max_tiles) { return 16 + (size_t)max_tiles * sizeof(MoeTile); }
@@ -140,7 +140,11 @@ static int launch_moe(const void* A, const void* W, void* C, const int32_t* coun
                       int64_t T, int64_t K, int64_t N, int64_t E, int64_t a_div, void* ws, hipStream_t s) {
   typedef typename Mfma16<BF>::T T16;
   const bool fast = (K % MOE_BK == 0) && (N % 8 == 0) && K >= MOE_BK && (((T + a_div - 1) / a_div) * K * 2 < (1LL << 32)) && (N * 4 < (1LL << 31)) && (((uintptr_t)A | (uintptr_t)W | (uintptr_t)C) & 15) == 0;
-  const int bm = fast ? MOE_BM : 64;
+  // 128-row tiles while the experts are small (less padding in each expert's last row tile) or the 256-row tiles would
+  // not fill the chip; 256-row tiles otherwise (half the operand traffic per flop)
+  const int64_t tn256 = (N + MOE_BN - 1) / MOE_BN;
+  const bool small = E > 0 && (T / E < 512 || ((T + MOE_BM - 1) / MOE_BM + E / 2) * tn256 < 192);
+  const int bm = fast ? (small ? G128_BM : MOE_BM) : 64;
   const int max_tiles = (int)moe_max_tiles(T, E, bm);
   int* num_tiles = (int*)ws;
   MoeTile* table = (MoeTile*)((uint8_t*)ws + 16);
@@ -154,11 +158,19 @@ static int launch_moe(const void* A, const void* W, void* C, const int32_t* coun
   hipLaunchKernelGGL(hx_moe_mark, dim3(max_tiles < 1024 ? max_tiles : 1024), dim3(256), 0, s, (const int*)num_tiles,
                      (const MoeTile*)table, idx, (int)T, flags);
   if (fast) {
-    const int tiles_n = (int)((N + MOE_BN - 1) / MOE_BN);
     G16Dense d = {};
     d.lda = K; d.ldb = N; d.ldc = N;
-    hipLaunchKernelGGL((hx_gemm16_tile256<BF, 0>), dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W, (void*)C,
-                       (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, max_tiles, tiles_n, (int)a_div, d);
+    if (bm == MOE_BM) {
+      const int tiles_n = (int)tn256;
+      hipLaunchKernelGGL((hx_gemm16_tile256<BF, 0>), dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W,
+                         (void*)C, (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, max_tiles, tiles_n,
+                         (int)a_div, d);
+    } else {
+      const int tiles_n = (int)((N + G128_BN - 1) / G128_BN);
+      hipLaunchKernelGGL((hx_gemm16_tile128<BF, 0>), dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W,
+                         (void*)C, (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, max_tiles, tiles_n,
+                         (int)a_div, d);
+    }
   } else {
     dim3 grid((unsigned)max_tiles, (unsigned)((N + 63) / 64));
     hipLaunchKernelGGL(hx_moe_general<T16>, grid, dim3(256), 0, s, (const T16*)A, (const T16*)W, (T16*)C, (const int*)num_tiles,

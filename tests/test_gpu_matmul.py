@@ -32,7 +32,8 @@ def _path(x, y):
 
 @pytest.mark.parametrize("m,k,n,path", [
     (256, 256, 256, 1), (1024, 1024, 1024, 1), (512, 64, 768, 1), (300, 192, 200, 1), (1, 64, 8, 1), (1000, 512, 1016, 1),
-    (128, 128, 128, 1), (64, 100, 64, 0), (33, 64, 7, 0), (5, 3, 2, 0),
+    (128, 128, 128, 1), (4096, 128, 2048, 1), (3000, 64, 4000, 1),   # the last two: enough tiles for the 256x256 kernel
+    (64, 100, 64, 0), (33, 64, 7, 0), (5, 3, 2, 0),
 ])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_shapes_and_epilogues_vs_oracle(m, k, n, path, dtype):
@@ -45,7 +46,7 @@ def test_shapes_and_epilogues_vs_oracle(m, k, n, path, dtype):
         assert rel_err(out, orc.matmul(x, y, **kw)) <= 1e-2
 
 
-@pytest.mark.parametrize("m,k,n", [(256, 256, 256), (300, 192, 200), (1000, 512, 1016), (64, 4096, 72), (1, 64, 8)])
+@pytest.mark.parametrize("m,k,n", [(256, 256, 256), (300, 192, 200), (1000, 512, 1016), (64, 4096, 72), (1, 64, 8), (4096, 128, 2056)])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_column_major_y_in_place(m, k, n, dtype):
     """y given as the transpose of an [n, k] weight (what `x @ w.T` of a linear layer passes): read in place by the tile
