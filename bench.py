@@ -216,7 +216,7 @@ def bench_siblings(steps, warmup):
     x = torch.randn(64, 32768, device="cuda", generator=g).to(torch.float16)
     y = torch.randn(32768, 64, device="cuda", generator=g).to(torch.float16)
     ms, _ = _time_launches(lambda: hx.matmul_split_k(x, y), n_it, n_w)
-    out["matmul_split_k_fp16"] = mfma(2.0 * 64 * 64 * 32768, ms, "hx_gemm16_tile256<f16, split-K partials> + hx_matmul16_reduce",
+    out["matmul_split_k_fp16"] = mfma(2.0 * 64 * 64 * 32768, ms, "hx_gemm16_tile128<f16, split-K partials> + hx_matmul16_reduce",
                                       "matmul_split_k 64 x 32768 x 64 fp16 (the example's shape; launch-latency sized)")
     del x, y
     for d in (128, 64):
