@@ -4,6 +4,7 @@
 // Three kernels:
 //   hx_fp8_gemm_tile256 : 256x256x128 workgroup tile, 4 waves (2x2) of 128x128, 32x32x64 fp8 MFMA,
 //                         A/B k-tiles DMA'd global->LDS (double buffered, XOR-swizzled 16B chunks).
+//   hx_fp8_gemm_tileN128 : 128x128 / 256x128 tiles with a deeper LDS ring, for problems with too few 256x256 tiles.
 //   hx_fp8_gemm_skinny_direct : M <= 32, K <= 8192; HBM-bound streaming of B^T through registers into
 //                         16x16x128 MFMA, K split across the 8 waves of a workgroup, partials summed in LDS.
 //   hx_fp8_gemm_skinny  : M <= 16, larger K; same split, A panel staged through LDS in 8 KB chunks of K.
@@ -314,6 +315,139 @@ __global__ __launch_bounds__(256) void hx_transpose_u8(const uint8_t* __restrict
 }
 
 // ------------------------------------------------------------------------------------------
+// tileN128: BM x 128 x 128 workgroup tile (BM = 128 or 256), for problems that 256x256 tiles cut into too few pieces
+// to occupy the chip: a decode batch of 33..256 rows against a wide weight matrix (one row tile: the kernel is then a
+// weight-streaming loop and wants every CU busy and several k-tiles in flight per CU), or a mid-size square product.
+// Column-major B (B^T rows of K).  4 waves (2x2) of (BM/2) x 64, 16x16x128 MFMAs, same LDS tile layout and k-block
+// assignment as tile256.  LDS ring of NS stages of (A BM x 128 B + B 128 x 128 B): NS - 1 k-tiles in flight; the
+// fragments of k-tile kt+1 are read into a second register set before the MFMAs of tile kt.  Rows and columns past
+// M / N re-read the last valid one and are never stored, so ragged M and N need no second instantiation.
+// ------------------------------------------------------------------------------------------
+template <int OUT, int BM>
+__global__ __launch_bounds__(256) void hx_fp8_gemm_tileN128(const uint8_t* __restrict__ A, const uint8_t* __restrict__ Bt,
+                                                           typename OutT<OUT>::T* __restrict__ C, int M, int N, int K, long lda,
+                                                           long ldb, long ldc, const float* __restrict__ scale_a,
+                                                           const float* __restrict__ scale_b, int tiles_m) {
+  typedef typename OutT<OUT>::T out_t;
+  constexpr int NS = BM == 128 ? 4 : 3;                  // 128 KB or 144 KB of LDS
+  constexpr int STAGE = (BM + 128) * 128;                // bytes of one stage: A tile, then B tile
+  constexpr int WMB = BM / 32;                           // 16-row blocks per wave
+  constexpr int AJ = BM / 32, IPW = AJ + 4;              // DMA instructions per wave per k-tile: A, B
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[NS][STAGE];
+
+  const int tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m;
+  const long m0 = (long)tm * BM, n0 = (long)tn * 128;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = w >> 1, wn = w & 1;
+
+  // ---- DMA: instruction j of a tile covers rows 8j .. 8j+7; wave w issues j = w, w+4, ...  The swizzle of a lane's
+  // row, ((8j + lrow) >> 1) & 7 = (4 (w & 1) + (lrow >> 1)) & 7, is the same for all of them.
+  const int lrow = lane >> 3, lpos = lane & 7;
+  const uint32_t chunk = (uint32_t)((lpos ^ ((4 * (w & 1) + (lrow >> 1)) & 7)) * 16);
+  uint32_t a_vo[AJ], b_vo[4];
+#pragma unroll
+  for (int jj = 0; jj < AJ; ++jj) a_vo[jj] = (uint32_t)min((int)m0 + 8 * (w + 4 * jj) + lrow, M - 1) * (uint32_t)lda + chunk;
+#pragma unroll
+  for (int jj = 0; jj < 4; ++jj) b_vo[jj] = (uint32_t)min((int)n0 + 8 * (w + 4 * jj) + lrow, N - 1) * (uint32_t)ldb + chunk;
+  const uint32_t lds0 = hx_lds_addr(&smem[0][0]);
+  const int nk = K / T256_BK;
+  // instruction i (0 .. IPW-1) of this wave for k-tile kt; past the end: the last tile again, so that every step
+  // issues IPW instructions and the counted waits stay exact
+  auto issue_one = [&](int kt, int i) {
+    const int t = min(kt, nk - 1);
+    const uint32_t base = lds0 + (uint32_t)(kt % NS) * STAGE;
+    if (i < AJ) hx_g2l16_s(hx_uniform_ptr(A + (long)t * T256_BK), a_vo[i], base + (w + 4 * i) * 1024);
+    else hx_g2l16_s(hx_uniform_ptr(Bt + (long)t * T256_BK), b_vo[i - AJ], base + BM * 128 + (w + 4 * (i - AJ)) * 1024);
+  };
+  auto issue = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < IPW; ++i) issue_one(kt, i);
+  };
+
+  // ---- MFMA operands: lane (r16, gq) reads chunks 2kq, 2kq + 1 of its row (kq: k-block of the lane group, as in tile256)
+  const int r16 = lane & 15, gq = lane >> 4;
+  const int kq = (gq >> 1) ^ ((gq & 1) * 3);
+  const int x16 = ((2 * kq) ^ ((r16 >> 1) & 7)) * 16;
+  const int a_base = (wm * (BM / 2) + r16) * 128;
+  const int b_base = BM * 128 + (wn * 64 + r16) * 128;
+  auto load_frags = [&](v8i(&fa)[WMB], v8i(&fb)[4], int kt) {
+    const uint8_t* st = &smem[kt % NS][0];
+#pragma unroll
+    for (int f = 0; f < WMB; ++f) {
+      const v4i lo = *(const v4i*)(st + a_base + f * 2048 + x16), hi = *(const v4i*)(st + a_base + f * 2048 + (x16 ^ 16));
+      fa[f] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    }
+#pragma unroll
+    for (int f = 0; f < 4; ++f) {
+      const v4i lo = *(const v4i*)(st + b_base + f * 2048 + x16), hi = *(const v4i*)(st + b_base + f * 2048 + (x16 ^ 16));
+      fb[f] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    }
+  };
+  // acc[bj][bi][r] is C[m0 + wm*BM/2 + 16 bi + lane%16][n0 + wn*64 + 16 bj + 4*(lane/16) + r]
+  v4f acc[4][WMB];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < WMB; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+  // the MFMAs of one k-tile with the DMA instructions of tile dkt between them, one after every other MFMA (a burst of
+  // them right after the barrier would hold the in-order instruction stream up)
+  auto mma = [&](v8i(&fa)[WMB], v8i(&fb)[4], int dkt) {
+#pragma unroll
+    for (int i = 0; i < 4 * WMB; ++i) {
+      acc[i & 3][i >> 2] = hx_mfma_16x16x128_e4m3(fb[i & 3], fa[i >> 2], acc[i & 3][i >> 2]);
+      if ((i & 1) && (i >> 1) < IPW) issue_one(dkt, i >> 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // step kt: tile kt is in `cur`; tiles kt+1 .. kt+NS-1 are landed or in flight
+  auto step = [&](v8i(&ca)[WMB], v8i(&cb)[4], v8i(&na)[WMB], v8i(&nb)[4], int kt) {
+    __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 2) * IPW));  // this wave's part of tile kt+1 has landed
+    __syncthreads();             // ... everybody's has, and every wave holds tile kt in registers: its stage is free
+    if (kt + 1 < nk) load_frags(na, nb, kt + 1);
+    mma(ca, cb, kt + NS);
+  };
+  for (int t = 0; t < NS; ++t) issue(t);
+  __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 1) * IPW));
+  __syncthreads();
+  v8i fa0[WMB], fb0[4], fa1[WMB], fb1[4];
+  load_frags(fa0, fb0, 0);
+  int kt = 0;
+  for (; kt + 1 < nk; kt += 2) {
+    step(fa0, fb0, fa1, fb1, kt);
+    step(fa1, fb1, fa0, fb0, kt + 1);
+  }
+  if (kt < nk) step(fa0, fb0, fa1, fb1, kt);
+  HX_WAIT_VM0();  // no DMA may still be writing this workgroup's LDS when it ends
+
+  float alpha = 1.f;
+  if (scale_a) alpha = *scale_a;
+  if (scale_b) alpha = alpha * *scale_b;
+  typedef out_t ov4 __attribute__((ext_vector_type(4)));
+  const bool vec_ok = (ldc % 4 == 0) && (((uintptr_t)C & (4 * sizeof(out_t) - 1)) == 0);
+#pragma unroll
+  for (int bi = 0; bi < WMB; ++bi) {
+    const long m = m0 + wm * (BM / 2) + 16 * bi + r16;
+    if (m >= M) continue;
+#pragma unroll
+    for (int bj = 0; bj < 4; ++bj) {
+      const long n = n0 + wn * 64 + 16 * bj + 4 * gq;
+      out_t* dst = C + m * ldc + n;
+      if (n + 4 <= N && vec_ok) {
+        ov4 o;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[r] = (out_t)(acc[bj][bi][r] * alpha);
+        *(ov4*)dst = o;
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (n + r < N) dst[r] = (out_t)(acc[bj][bi][r] * alpha);
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
 // skinny (M <= 16): one workgroup = 8 waves; the workgroup owns column groups of 16 columns and
 // streams the 16 x K bytes of B^T for each exactly once from HBM.  K is split across the waves in
 // 128-byte steps (wave w takes steps w, w+8, ...); each wave accumulates a 16x16 fp32 partial with
@@ -593,7 +727,8 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_general(const uint8_t* __rest
 // ------------------------------------------------------------------------------------------
 static inline bool aligned(const void* p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
-// 0 general, 1 tile256, 2 skinny, 3 tile256 with edge tiles (M or N not a multiple of 256)
+// 0 general, 1 tile256, 2 skinny, 3 tile256 with edge tiles (M or N not a multiple of 256, K not of 128),
+// 5 tileN128 (too few 256x256 tiles to occupy the chip)
 static int gemm_path_kmajor(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, const void* a, const void* b,
                             const void* c) {
   const bool ok = (lda % 16 == 0) && (ldb % 16 == 0) && (K % 16 == 0) && aligned(a, 16) && aligned(b, 16) && K >= 16;
@@ -601,6 +736,7 @@ static int gemm_path_kmajor(int64_t M, int64_t N, int64_t K, int64_t lda, int64_
   const bool ktail = K % 128 != 0;  // only the edge instantiation of the tile kernel pads a partial last k-tile
   if (!ktail && (M <= 16 || (M <= 32 && K <= 8192)) && lda >= K && ldb >= K) return 2;
   if (lda >= (1LL << 27) || ldb >= (1LL << 27)) return 0;
+  if (!ktail && ((M + 255) / 256) * ((N + 255) / 256) < 192 && M * lda < (1LL << 32) && N * ldb < (1LL << 32)) return 5;
   if (!ktail && (M % 256 == 0) && (N % 256 == 0) && (ldc % 8 == 0) && aligned(c, 16)) return 1;  // 16-byte row-aligned stores
   if (M * lda < (1LL << 32) && N * ldb < (1LL << 32)) return 3;
   return 0;
@@ -634,6 +770,15 @@ static void launch_kmajor(int path, const void* a, const void* bt, void* c, int6
       hipLaunchKernelGGL((hx_fp8_gemm_tile256<OUT, true, true>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
                          (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m,
                          tiles_n);
+  } else if (path == 5) {
+    const int tiles_n = (int)((N + 127) / 128);
+    if (M > 128 && M <= 256)  // one 256-row tile instead of a full and a mostly padded 128-row tile
+      hipLaunchKernelGGL((hx_fp8_gemm_tileN128<OUT, 256>), dim3(tiles_n), dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
+                         (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, 1);
+    else
+      hipLaunchKernelGGL((hx_fp8_gemm_tileN128<OUT, 128>), dim3((unsigned)((M + 127) / 128) * tiles_n), dim3(256), 0, stream,
+                         (const uint8_t*)a, (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa,
+                         sb, (int)((M + 127) / 128));
   } else if (path == 1 || path == 3) {
     const int tiles_m = (int)((M + 255) / 256), tiles_n = (int)((N + 255) / 256);
     if (path == 1)

@@ -48,12 +48,15 @@ def test_gemm_path_selection():
     assert lib.hx_fp8_gemm_path(16, 28672, 8192, 8192, 1, 8192, 28672, A, A, A) == 2
     assert lib.hx_fp8_gemm_path(1, 512, 256, 256, 1, 256, 512, A, A, A) == 2
     assert lib.hx_fp8_gemm_path(32, 28672, 8192, 8192, 1, 8192, 28672, A, A, A) == 2   # up to 32 rows when K <= 8192
-    assert lib.hx_fp8_gemm_path(33, 28672, 8192, 8192, 1, 8192, 28672, A, A, A) == 3
+    assert lib.hx_fp8_gemm_path(33, 28672, 8192, 8192, 1, 8192, 28672, A, A, A) == 5   # a decode batch: 128-column tiles
+    assert lib.hx_fp8_gemm_path(2048, 2048, 2048, 2048, 1, 2048, 2048, A, A, A) == 5   # 64 tiles of 256x256 would idle the chip
+    assert lib.hx_fp8_gemm_path(4096, 4096, 4096, 4096, 1, 4096, 4096, A, A, A) == 1
     assert lib.hx_fp8_gemm_path(256, 256, 256, 256, 256, 1, 256, A, A, A) == 4  # row-major B, read in place
     assert lib.hx_fp8_gemm_path(16, 256, 256, 256, 256, 1, 256, A, A, A) == 0   # row-major B for the skinny shape: via workspace
     assert lib.hx_fp8_gemm_path(100, 72, 128, 128, 72, 1, 72, A, A, A) == 0     # row-major B, N % 16 != 0
     assert lib.hx_fp8_gemm_path(100, 70, 50, 50, 1, 50, 70, A, A, A) == 0  # ragged K
-    assert lib.hx_fp8_gemm_path(1000, 1000, 1024, 1024, 1, 1024, 1000, A, A, A) == 3  # ragged M/N: guarded edge tiles
+    assert lib.hx_fp8_gemm_path(5000, 5000, 1024, 1024, 1, 1024, 5000, A, A, A) == 3  # ragged M/N: guarded edge tiles
+    assert lib.hx_fp8_gemm_path(1000, 1000, 1040, 1040, 1, 1040, 1000, A, A, A) == 3  # K % 128 != 0
     assert lib.hx_fp8_gemm_workspace_bytes(256, 512, 384, 512, 1) == 0          # row-major B the tile kernel reads in place
     assert lib.hx_fp8_gemm_workspace_bytes(8, 512, 384, 512, 1) == 512 * 384    # skinny shape: transpose scratch
     assert lib.hx_fp8_gemm_workspace_bytes(256, 512, 384, 1, 384) == 0

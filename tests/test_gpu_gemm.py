@@ -23,10 +23,13 @@ def _path(m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k,path", [
-    (256, 256, 256, 1), (512, 512, 512, 1), (1024, 1024, 1024, 1), (256, 768, 128, 1), (768, 256, 1152, 1),
+    (4096, 4096, 128, 1), (2048, 6144, 256, 1),                                                      # enough full 256x256 tiles
+    (256, 256, 256, 5), (512, 512, 512, 5), (1024, 1024, 1024, 5), (256, 768, 128, 5), (768, 256, 1152, 5),   # too few: 128-column tiles
+    (48, 1024, 512, 5), (100, 3000, 256, 5), (129, 520, 384, 5), (256, 1000, 128, 5), (200, 136, 1280, 5), (33, 256, 256, 5),
+    (1000, 1000, 1024, 5), (300, 200, 256, 5), (257, 255, 128, 5), (32, 64, 8192 + 128, 5), (255, 1, 128, 5),
     (16, 512, 1024, 2), (1, 16, 128, 2), (5, 48, 256, 2), (16, 1000, 384, 2), (9, 33, 8192 + 128, 2), (16, 64, 16384, 2),
     (17, 256, 256, 2), (32, 512, 8192, 2), (24, 100, 1152, 2), (31, 33, 384, 2),        # two 16-row blocks on the skinny kernel
-    (1000, 1000, 1024, 3), (300, 200, 256, 3), (257, 255, 128, 3), (33, 256, 256, 3), (32, 64, 8192 + 128, 3), (255, 1, 128, 3),
+    (4000, 4100, 256, 3), (3000, 5000, 128, 3),                                          # ragged M, N on the 256x256 kernel
     (256, 256, 208, 3), (300, 200, 144, 3), (1000, 1000, 1040, 3), (64, 64, 16, 3), (16, 512, 1024 + 16, 3), (512, 256, 128 * 5 + 112, 3),  # K tails
     (100, 70, 50, 0), (256, 256, 200, 0), (3, 5, 7, 0), (64, 64, 0, 0),
 ])
@@ -197,4 +200,4 @@ def test_random_shapes_layouts_and_dtypes_vs_oracle():
         out = hx.fp8_gemm(xd, yd, scale_a=sa.to(DEV), scale_b=sb.to(DEV), out_dtype=od)
         ref = orc.fp8_gemm(x, y, sa, sb, od)
         assert rel_err(out, ref) <= (1e-2 if od != torch.float32 else 1e-4), (case, m, n, k, row_major, od)
-    assert seen >= {0, 2, 3, 4}   # the aligned tile path (1) has its own cases above
+    assert seen >= {0, 2, 3, 4, 5}   # the aligned 256x256 tile path (1) has its own cases above
