@@ -4,15 +4,18 @@
 // entry points use it while 256x256 tiles would leave most of the chip idle (a 2048^3 product has only 64 of them) and
 // for grouped GEMMs whose experts hold few rows (less padding in the last row tile of every expert).
 //
-// 4 waves (2x2) of 64x64, 32x32x16 MFMAs, 2 LDS stages of (A 16 KB + W 16 KB) = 64 KB, two workgroups per CU.
+// 4 waves (2x2) of 64x64, 32x32x16 MFMAs, NS LDS stages of (A 16 KB + W 16 KB): NS = 2 (64 KB, two workgroups per CU)
+// for compute-heavy problems, NS = 4 (128 KB, three k-tiles in flight per CU) when there is at most one workgroup per
+// CU anyway and the kernel is a weight-streaming loop (a decode batch against a wide weight matrix).
 //   A tile [128 rows][128 B]   : as in the 256 kernel (rows gathered by the DMA in the grouped mode).
 //   W tile [64 k][256 B]       : row = k, 16 chunks of 8 columns, chunk stored at pos = chunk ^ ((k & 3) << 2): one
 //                                transposing read has 32 lanes fetch 4 consecutive k rows x 64 contiguous bytes, and
 //                                the xor puts the four rows into different 64-byte quarters of the bank window.
 //   W tile, column-major W     : [128 columns][128 B], exactly like the A tile.
 // The fragments of a whole k-tile (4 k-steps) are read into registers at once, one k-tile ahead of the MFMAs that use
-// them, so the LDS stage of a tile is free for the DMA of tile kt+2 as soon as every wave has passed the barrier of
-// tile kt; two register sets alternate.
+// them, so the LDS stage of a tile is free for the DMA of tile kt+NS as soon as every wave has passed the barrier of
+// tile kt; two register sets alternate.  Past the last k-tile the DMA fetches the last tile again, so every step
+// issues the same number of instructions and the counted waits stay exact.
 #pragma once
 #include "gemm16_tile256.h"
 
@@ -20,14 +23,14 @@
 #define G128_BN 128
 #define G128_TILE_BYTES (128 * 128)
 
-template <bool BF, int MODE, bool BCOL = false>
-__global__ __launch_bounds__(256, 2) void hx_gemm16_tile128(const uint8_t* __restrict__ A, const uint8_t* __restrict__ W,
+template <bool BF, int MODE, bool BCOL = false, int NS = 2>
+__global__ __launch_bounds__(256, NS == 2 ? 2 : 1) void hx_gemm16_tile128(const uint8_t* __restrict__ A, const uint8_t* __restrict__ W,
                                                            void* __restrict__ Cv, const int* __restrict__ num_tiles,
                                                            const MoeTile* __restrict__ table, const int32_t* __restrict__ idx, int T,
                                                            int K, int N, int max_tiles, int tiles_n, int a_div, G16Dense d) {
   typedef typename Mfma16<BF>::T out_t;
   typedef typename Mfma16<BF>::V8 V8;
-  __shared__ __attribute__((aligned(1024))) uint8_t smem[2][2][G128_TILE_BYTES];  // [stage][A | W]
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[NS][2][G128_TILE_BYTES];  // [stage][A | W]
 
   // the raster of the 256 kernel: 8 row tiles tall, every 256 consecutive tiles spread over the XCDs in blocks of 32
   int tile;
@@ -94,7 +97,8 @@ __global__ __launch_bounds__(256, 2) void hx_gemm16_tile128(const uint8_t* __res
     }
   }
   const uint32_t lds0 = hx_lds_addr(&smem[0][0][0]);
-  auto issue = [&](int kt, int stage) {  // this wave's 8 DMA instructions of k-tile kt
+  auto issue = [&](int kt_unclamped) {  // this wave's 8 DMA instructions of k-tile kt into stage kt % NS
+    const int kt = min(kt_unclamped, nk - 1), stage = kt_unclamped % NS;
     const uint32_t la = lds0 + (uint32_t)stage * 2 * G128_TILE_BYTES + (uint32_t)w * 32 * 128;
     const uint32_t lw = lds0 + (uint32_t)stage * 2 * G128_TILE_BYTES + G128_TILE_BYTES;
 #pragma unroll
@@ -164,18 +168,15 @@ __global__ __launch_bounds__(256, 2) void hx_gemm16_tile128(const uint8_t* __res
   };
   // one k-tile: `cur` holds tile kt; tile kt+1 is in flight into the other stage
   auto ktile = [&](V8(&ca)[4][2], V8(&cw)[4][2], V8(&na)[4][2], V8(&nw)[4][2], int kt) {
-    if (kt + 1 < nk) {
-      HX_WAIT_VM0();    // this wave's part of tile kt+1 has landed (tile kt+2 is not issued yet)
-      __syncthreads();  // ... everybody's has, and every wave holds tile kt in registers: its stage is free
-      if (kt + 2 < nk) issue(kt + 2, kt & 1);
-      load_frags(na, nw, (kt + 1) & 1);
-    }
+    __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 2) * 8));  // this wave's part of tile kt+1 has landed
+    __syncthreads();  // ... everybody's has, and every wave holds tile kt in registers: its stage is free
+    issue(kt + NS);
+    if (kt + 1 < nk) load_frags(na, nw, (kt + 1) % NS);
     mma(ca, cw);
   };
   V8 fa0[4][2], fw0[4][2], fa1[4][2], fw1[4][2];
-  issue(0, 0);
-  if (nk > 1) issue(1, 1);
-  if (nk > 1) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(8)); else HX_WAIT_VM0();
+  for (int t = 0; t < NS; ++t) issue(t);
+  __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 1) * 8));
   __syncthreads();
   load_frags(fa0, fw0, 0);
   int kt = 0;
@@ -184,6 +185,7 @@ __global__ __launch_bounds__(256, 2) void hx_gemm16_tile128(const uint8_t* __res
     ktile(fa1, fw1, fa0, fw0, kt + 1);
   }
   if (kt < nk) ktile(fa0, fw0, fa1, fw1, kt);
+  HX_WAIT_VM0();  // no DMA may still be writing this workgroup's LDS when it ends
 
   // ---- epilogue: acc[bj][bi][4a+b] is C[row_of(wm*64 + bi*32 + lane%32)][n0 + wn*64 + bj*32 + 8a + 4g + b].
   // N % 8 == 0 and a piece starts at a multiple of 4: it is either wholly inside the row or wholly outside.

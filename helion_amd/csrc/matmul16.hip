@@ -121,7 +121,9 @@ static MmPlan mm_plan(int64_t M, int64_t N, int64_t K, int split_k) {
   MmPlan p;
   p.tile = t256 >= 128 ? 256 : 128;
   const int64_t tiles = ((M + p.tile - 1) / p.tile) * ((N + p.tile - 1) / p.tile);
-  const int64_t room = p.tile == 256 ? 256 : 512;  // resident workgroups: one or two per CU
+  // resident workgroups to aim for: one per CU (with 128x128 tiles a deep LDS ring then keeps several k-tiles in flight;
+  // two workgroups per CU with a shallow ring are for problems that have the tiles anyway)
+  const int64_t room = 256;
   int64_t s = split_k;
   if (s <= 0) {
     s = 1;
@@ -175,9 +177,14 @@ static void mm_launch_fast(const void* a, const void* b, void* c, int64_t M, int
     if (tile == 256)
       hipLaunchKernelGGL((hx_gemm16_tile256<BF, 1, BCOL>), dim3(tiles_m * tiles_n), dim3(256), 0, s, (const uint8_t*)a, (const uint8_t*)b, c,
                          (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M, (int)K, (int)N, tiles_m, tiles_n, 1, d);
+    else if (tiles_m * tiles_n <= 256)
+      hipLaunchKernelGGL((hx_gemm16_tile128<BF, 1, BCOL, 4>), dim3(tiles_m * tiles_n), dim3(256), 0, s, (const uint8_t*)a, (const uint8_t*)b,
+                         c, (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M, (int)K, (int)N, tiles_m, tiles_n, 1,
+                         d);
     else
-      hipLaunchKernelGGL((hx_gemm16_tile128<BF, 1, BCOL>), dim3(tiles_m * tiles_n), dim3(256), 0, s, (const uint8_t*)a, (const uint8_t*)b, c,
-                         (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M, (int)K, (int)N, tiles_m, tiles_n, 1, d);
+      hipLaunchKernelGGL((hx_gemm16_tile128<BF, 1, BCOL, 2>), dim3(tiles_m * tiles_n), dim3(256), 0, s, (const uint8_t*)a, (const uint8_t*)b,
+                         c, (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M, (int)K, (int)N, tiles_m, tiles_n, 1,
+                         d);
     return;
   }
   const int nkt = (int)(K / MOE_BK);
@@ -187,8 +194,12 @@ static void mm_launch_fast(const void* a, const void* b, void* c, int64_t M, int
     hipLaunchKernelGGL((hx_gemm16_tile256<BF, 2, BCOL>), dim3(tiles_m * tiles_n, splits), dim3(256), 0, s, (const uint8_t*)a,
                        (const uint8_t*)b, partial ? ws : c, (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M,
                        (int)K, (int)N, tiles_m, tiles_n, 1, d);
+  else if ((long)tiles_m * tiles_n * splits <= 256)
+    hipLaunchKernelGGL((hx_gemm16_tile128<BF, 2, BCOL, 4>), dim3(tiles_m * tiles_n, splits), dim3(256), 0, s, (const uint8_t*)a,
+                       (const uint8_t*)b, partial ? ws : c, (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M,
+                       (int)K, (int)N, tiles_m, tiles_n, 1, d);
   else
-    hipLaunchKernelGGL((hx_gemm16_tile128<BF, 2, BCOL>), dim3(tiles_m * tiles_n, splits), dim3(256), 0, s, (const uint8_t*)a,
+    hipLaunchKernelGGL((hx_gemm16_tile128<BF, 2, BCOL, 2>), dim3(tiles_m * tiles_n, splits), dim3(256), 0, s, (const uint8_t*)a,
                        (const uint8_t*)b, partial ? ws : c, (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M,
                        (int)K, (int)N, tiles_m, tiles_n, 1, d);
   if (!partial) return;
