@@ -176,6 +176,19 @@ def bench_next_rows(steps, warmup):
     out["fp8_quantize_per_tensor"] = hbm(x.numel() * 5, ms, "hx_amax_partial + hx_amax_final + hx_cast_e4m3_kernel<bf16>",
                                          "amax -> scale -> e4m3 of a bf16 8192x8192 operand (bytes: 2 reads + 1 write)")
     del x
+    # a decode batch of 64 rows against the C3 weight matrix: the 128-column tile kernel as a weight-streaming loop
+    bufs = [(torch.randn(28672, 8192, device="cuda") * 0.5).to(torch.float8_e4m3fn).T for _ in range(4)]
+    xa = (torch.randn(64, 8192, device="cuda") * 0.5).to(torch.float8_e4m3fn)
+    turn = [0]
+
+    def decode64():
+        turn[0] = (turn[0] + 1) % len(bufs)
+        return hx.fp8_gemm(xa, bufs[turn[0]], out_dtype=torch.bfloat16)
+
+    ms, _ = _time_launches(decode64, n_it, n_w)
+    out["decode_gemm_m64"] = hbm(28672 * 8192 + 64 * 8192 + 2 * 64 * 28672, ms, "hx_fp8_gemm_tileN128<bf16, 128>",
+                                 "fp8_gemm M64 N28672 K8192 bf16 out, 4 rotating weight buffers (HBM-cold)")
+    del bufs, xa
     # routing tables at the C5 row count and at 1M rows
     _, _, ex = inputs.moe_c5("cuda")
     ms, _ = _time_launches(lambda: hx.moe_routing(ex, 8), n_it, n_w)

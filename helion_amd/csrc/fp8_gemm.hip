@@ -322,12 +322,15 @@ __global__ __launch_bounds__(256) void hx_transpose_u8(const uint8_t* __restrict
 // assignment as tile256.  LDS ring of NS stages of (A BM x 128 B + B 128 x 128 B): NS - 1 k-tiles in flight; the
 // fragments of k-tile kt+1 are read into a second register set before the MFMAs of tile kt.  Rows and columns past
 // M / N re-read the last valid one and are never stored, so ragged M and N need no second instantiation.
+// bn (a multiple of 16, 64..128) is the column pitch of the tiles: with a single row tile the host picks it so that
+// the column tiles come to about one per CU (N = 28672: 112 columns, 256 tiles); the columns of a tile past bn
+// re-read its last column (an L2 hit, no HBM traffic) and are not stored.
 // ------------------------------------------------------------------------------------------
 template <int OUT, int BM>
 __global__ __launch_bounds__(256) void hx_fp8_gemm_tileN128(const uint8_t* __restrict__ A, const uint8_t* __restrict__ Bt,
                                                            typename OutT<OUT>::T* __restrict__ C, int M, int N, int K, long lda,
                                                            long ldb, long ldc, const float* __restrict__ scale_a,
-                                                           const float* __restrict__ scale_b, int tiles_m) {
+                                                           const float* __restrict__ scale_b, int tiles_m, int bn) {
   typedef typename OutT<OUT>::T out_t;
   constexpr int NS = BM == 128 ? 4 : 3;                  // 128 KB or 144 KB of LDS
   constexpr int STAGE = (BM + 128) * 128;                // bytes of one stage: A tile, then B tile
@@ -336,7 +339,8 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tileN128(const uint8_t* __res
   __shared__ __attribute__((aligned(1024))) uint8_t smem[NS][STAGE];
 
   const int tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m;
-  const long m0 = (long)tm * BM, n0 = (long)tn * 128;
+  const long m0 = (long)tm * BM, n0 = (long)tn * bn;
+  const int nlast = (int)min(n0 + bn, (long)N) - 1;  // last column this tile owns
   const int tid = threadIdx.x, lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = w >> 1, wn = w & 1;
@@ -349,7 +353,7 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tileN128(const uint8_t* __res
 #pragma unroll
   for (int jj = 0; jj < AJ; ++jj) a_vo[jj] = (uint32_t)min((int)m0 + 8 * (w + 4 * jj) + lrow, M - 1) * (uint32_t)lda + chunk;
 #pragma unroll
-  for (int jj = 0; jj < 4; ++jj) b_vo[jj] = (uint32_t)min((int)n0 + 8 * (w + 4 * jj) + lrow, N - 1) * (uint32_t)ldb + chunk;
+  for (int jj = 0; jj < 4; ++jj) b_vo[jj] = (uint32_t)min((int)n0 + 8 * (w + 4 * jj) + lrow, nlast) * (uint32_t)ldb + chunk;
   const uint32_t lds0 = hx_lds_addr(&smem[0][0]);
   const int nk = K / T256_BK;
   // instruction i (0 .. IPW-1) of this wave for k-tile kt; past the end: the last tile again, so that every step
@@ -433,7 +437,7 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tileN128(const uint8_t* __res
     for (int bj = 0; bj < 4; ++bj) {
       const long n = n0 + wn * 64 + 16 * bj + 4 * gq;
       out_t* dst = C + m * ldc + n;
-      if (n + 4 <= N && vec_ok) {
+      if (n + 3 <= nlast && vec_ok) {
         ov4 o;
 #pragma unroll
         for (int r = 0; r < 4; ++r) o[r] = (out_t)(acc[bj][bi][r] * alpha);
@@ -441,7 +445,7 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tileN128(const uint8_t* __res
       } else {
 #pragma unroll
         for (int r = 0; r < 4; ++r)
-          if (n + r < N) dst[r] = (out_t)(acc[bj][bi][r] * alpha);
+          if (n + r <= nlast) dst[r] = (out_t)(acc[bj][bi][r] * alpha);
       }
     }
   }
@@ -771,14 +775,20 @@ static void launch_kmajor(int path, const void* a, const void* bt, void* c, int6
                          (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m,
                          tiles_n);
   } else if (path == 5) {
-    const int tiles_n = (int)((N + 127) / 128);
+    // column pitch of the tiles: 128, except that a single row tile (a decode batch) gets about one column tile per CU
+    int bn = 128;
+    if (M <= 128) {  // (with a 256-row tile the MFMA work on the unused columns costs more than the idle CUs)
+      const int64_t blocks = (N + 15) / 16, per = (blocks + 255) / 256;  // 16-column blocks per tile for <= 256 tiles
+      if (per <= 8) bn = (int)(16 * (per < 4 ? 4 : per));
+    }
+    const int tiles_n = (int)((N + bn - 1) / bn);
     if (M > 128 && M <= 256)  // one 256-row tile instead of a full and a mostly padded 128-row tile
       hipLaunchKernelGGL((hx_fp8_gemm_tileN128<OUT, 256>), dim3(tiles_n), dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
-                         (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, 1);
+                         (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, 1, bn);
     else
       hipLaunchKernelGGL((hx_fp8_gemm_tileN128<OUT, 128>), dim3((unsigned)((M + 127) / 128) * tiles_n), dim3(256), 0, stream,
                          (const uint8_t*)a, (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa,
-                         sb, (int)((M + 127) / 128));
+                         sb, (int)((M + 127) / 128), bn);
   } else if (path == 1 || path == 3) {
     const int tiles_m = (int)((M + 255) / 256), tiles_n = (int)((N + 255) / 256);
     if (path == 1)
