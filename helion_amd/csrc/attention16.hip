@@ -15,6 +15,7 @@
 // the last tile re-reads row N-1 for the missing keys and their scores are set to -inf before the softmax.
 #include "hx_common.h"
 
+#include <cmath>
 #include <type_traits>
 
 #define A16_BN 64
@@ -38,7 +39,7 @@ __device__ __forceinline__ int a16_vswz(int row) {
 template <int D, bool BF, bool TAIL>
 __global__ __launch_bounds__(64 * A16_WAVES, 2) void hx_attention16_kernel(const uint8_t* __restrict__ Q, const uint8_t* __restrict__ Kp,
                                                                 const uint8_t* __restrict__ Vp, void* __restrict__ Out, int M, int N,
-                                                                int BH, int qtiles) {
+                                                                int BH, int qtiles, float c) {
   typedef typename Mfma16<BF>::T T16;
   typedef typename Mfma16<BF>::V8 V8;
   constexpr int RB = 2 * D;                                  // bytes of a row
@@ -139,7 +140,6 @@ __global__ __launch_bounds__(64 * A16_WAVES, 2) void hx_attention16_kernel(const
     return __builtin_bit_cast(V8, both);
   };
 
-  const float c = (float)((1.0 / __builtin_sqrt((double)D)) * 1.44269504);
   const int ntiles = (N + A16_BN - 1) / A16_BN;
 
   auto load_kfrag = [&](const uint8_t* sk, int mi) -> V8 {  // A operand of score MFMA mi = kb * KSTEPS + t
@@ -317,7 +317,7 @@ __global__ __launch_bounds__(64 * A16_WAVES, 2) void hx_attention16_kernel(const
 // ------------------------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void hx_attention_general(const T* __restrict__ Q, const T* __restrict__ Kp, const T* __restrict__ Vp,
-                                                           T* __restrict__ Out, int M, int N, int D) {
+                                                           T* __restrict__ Out, int M, int N, int D, float c) {
   constexpr int CH = 1024;
   __shared__ float sq[256];
   __shared__ float sp[CH];
@@ -329,7 +329,6 @@ __global__ __launch_bounds__(256) void hx_attention_general(const T* __restrict_
   const T* Vh = Vp + bh * (long)N * D;
   if (tid < D) sq[tid] = (float)q[tid];
   __syncthreads();
-  const float c = (float)((1.0 / __builtin_sqrt((double)D)) * 1.44269504);
   float m = -__builtin_inff(), l = 0.f, acc = 0.f;
   for (int n0 = 0; n0 < N; n0 += CH) {
     const int cn = min(CH, N - n0);
@@ -388,25 +387,29 @@ extern "C" int hx_attention_path(int64_t BH, int64_t M, int64_t N, int64_t D, in
 }
 
 template <int D, bool BF>
-static void launch_att16(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t M, int64_t N, hipStream_t s) {
+static void launch_att16(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t M, int64_t N, float c, hipStream_t s) {
   const int qtiles = (int)((M + A16_BM - 1) / A16_BM);
   const int hpx = (int)((BH + 7) / 8);
   if (N % A16_BN)
     hipLaunchKernelGGL((hx_attention16_kernel<D, BF, true>), dim3(8 * hpx * qtiles), dim3(64 * A16_WAVES), 0, s, (const uint8_t*)q,
-                       (const uint8_t*)k, (const uint8_t*)v, out, (int)M, (int)N, (int)BH, qtiles);
+                       (const uint8_t*)k, (const uint8_t*)v, out, (int)M, (int)N, (int)BH, qtiles, c);
   else
     hipLaunchKernelGGL((hx_attention16_kernel<D, BF, false>), dim3(8 * hpx * qtiles), dim3(64 * A16_WAVES), 0, s, (const uint8_t*)q,
-                       (const uint8_t*)k, (const uint8_t*)v, out, (int)M, (int)N, (int)BH, qtiles);
+                       (const uint8_t*)k, (const uint8_t*)v, out, (int)M, (int)N, (int)BH, qtiles, c);
 }
 
 extern "C" int hx_attention(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t M, int64_t N, int64_t D,
-                            int dtype, void* stream) {
+                            int64_t scale_dim, int dtype, void* stream) {
   if (BH < 0 || M < 0 || N < 0 || D < 0) {
     hx_set_error("hx_attention: negative size");
     return HX_ERR_BAD_ARG;
   }
   if (dtype != HX_BF16 && dtype != HX_F16 && dtype != HX_F32) {
     hx_set_error("hx_attention: dtype must be HX_BF16, HX_F16 or HX_F32, got %d", dtype);
+    return HX_ERR_BAD_ARG;
+  }
+  if (scale_dim < 0) {
+    hx_set_error("hx_attention: negative scale_dim");
     return HX_ERR_BAD_ARG;
   }
   if (BH == 0 || M == 0 || D == 0) return 0;
@@ -423,13 +426,15 @@ extern "C" int hx_attention(const void* q, const void* k, const void* v, void* o
     return HX_ERR_UNSUPPORTED;
   }
   hipStream_t s = (hipStream_t)stream;
+  // the softmax scale in base 2, evaluated the way the reference does: double arithmetic, rounded to fp32 once
+  const float c = (float)((1.0 / sqrt((double)(scale_dim > 0 ? scale_dim : D))) * 1.44269504);
   if (att16_fast_ok(q, k, v, out, BH, M, N, D, dtype)) {
     if (D == 128) {
-      if (dtype == HX_BF16) launch_att16<128, true>(q, k, v, out, BH, M, N, s);
-      else launch_att16<128, false>(q, k, v, out, BH, M, N, s);
+      if (dtype == HX_BF16) launch_att16<128, true>(q, k, v, out, BH, M, N, c, s);
+      else launch_att16<128, false>(q, k, v, out, BH, M, N, c, s);
     } else {
-      if (dtype == HX_BF16) launch_att16<64, true>(q, k, v, out, BH, M, N, s);
-      else launch_att16<64, false>(q, k, v, out, BH, M, N, s);
+      if (dtype == HX_BF16) launch_att16<64, true>(q, k, v, out, BH, M, N, c, s);
+      else launch_att16<64, false>(q, k, v, out, BH, M, N, c, s);
     }
   } else {
     if (D > 256 || BH >= 65536) {
@@ -440,13 +445,13 @@ extern "C" int hx_attention(const void* q, const void* k, const void* v, void* o
     const dim3 grid((unsigned)M, (unsigned)BH);
     if (dtype == HX_BF16)
       hipLaunchKernelGGL(hx_attention_general<__bf16>, grid, dim3(256), 0, s, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
-                         (__bf16*)out, (int)M, (int)N, (int)D);
+                         (__bf16*)out, (int)M, (int)N, (int)D, c);
     else if (dtype == HX_F16)
       hipLaunchKernelGGL(hx_attention_general<_Float16>, grid, dim3(256), 0, s, (const _Float16*)q, (const _Float16*)k,
-                         (const _Float16*)v, (_Float16*)out, (int)M, (int)N, (int)D);
+                         (const _Float16*)v, (_Float16*)out, (int)M, (int)N, (int)D, c);
     else
       hipLaunchKernelGGL(hx_attention_general<float>, grid, dim3(256), 0, s, (const float*)q, (const float*)k, (const float*)v,
-                         (float*)out, (int)M, (int)N, (int)D);
+                         (float*)out, (int)M, (int)N, (int)D, c);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {

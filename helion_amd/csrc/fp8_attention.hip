@@ -22,6 +22,8 @@
 // (ds_read_b64_tr_b8: 8 keys x 16 columns per 16 lanes), so neither layout needs a copy.
 #include "hx_common.h"
 
+#include <cmath>
+
 #define ATT_BN 64      // keys per tile
 #define ATT_WAVES 4
 #define ATT_BM (32 * ATT_WAVES)
@@ -54,7 +56,7 @@ __device__ __forceinline__ void att_wait_tiles(int newer) {
 template <int D, int OUT, bool EXACT, bool VSD>
 __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t* __restrict__ Q, const uint8_t* __restrict__ Kt,
                                                                   const uint8_t* __restrict__ Vt, void* __restrict__ Out, int S,
-                                                                  int BH, int qtiles) {
+                                                                  int BH, int qtiles, float c) {
   constexpr int KSTEPS = D / 64;  // MFMA k-steps for S = K Q^T
   constexpr int DB = D / 32;      // 32-row blocks of O^T
   constexpr int KROWS_PER_DMA = 1024 / D;
@@ -163,7 +165,6 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
     return (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   };
 
-  const float c = (float)((1.0 / __builtin_sqrt((double)D)) * 1.44269504);
   const int ntiles = S / ATT_BN;
 
   auto scores = [&](const uint8_t* sk, v16f(&s)[2]) {
@@ -364,7 +365,7 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
 template <int OUT>
 __global__ __launch_bounds__(256) void hx_fp8_attention_general(const uint8_t* __restrict__ Q, const uint8_t* __restrict__ Kt,
                                                                const uint8_t* __restrict__ Vt, void* __restrict__ Out, int S, int D,
-                                                               long vsd, long vss) {
+                                                               long vsd, long vss, float c) {
   constexpr int CH = 1024;
   __shared__ float sq[256];
   __shared__ float sp[CH];
@@ -392,7 +393,6 @@ __global__ __launch_bounds__(256) void hx_fp8_attention_general(const uint8_t* _
     __syncthreads();
     return r;
   };
-  const float c = (float)((1.0 / __builtin_sqrt((double)D)) * 1.44269504);
   float smax = -__builtin_inff();
   for (int key = tid; key < S; key += 256) smax = fmaxf(smax, score(key));
   const float neg_m = -(block_reduce(smax, true) * c);
@@ -419,22 +419,22 @@ __global__ __launch_bounds__(256) void hx_fp8_attention_general(const uint8_t* _
 }
 
 template <int D, int OUT, bool EXACT, bool VSD>
-static void launch_att_kernel(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t S, hipStream_t s) {
+static void launch_att_kernel(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t S, float c, hipStream_t s) {
   const int qtiles = (int)((S + ATT_BM - 1) / ATT_BM);
   const int hpx = (int)((BH + 7) / 8);
   const int grid = 8 * hpx * qtiles;
   hipLaunchKernelGGL((hx_fp8_attention_kernel<D, OUT, EXACT, VSD>), dim3(grid), dim3(256), 0, s, (const uint8_t*)q, (const uint8_t*)k,
-                     (const uint8_t*)v, out, (int)S, (int)BH, qtiles);
+                     (const uint8_t*)v, out, (int)S, (int)BH, qtiles, c);
 }
 
 template <int D, int OUT>
-static int launch_att(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t S, int exact, bool vsd, hipStream_t s) {
+static int launch_att(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t S, int exact, bool vsd, float c, hipStream_t s) {
   if (exact) {
-    if (vsd) launch_att_kernel<D, OUT, true, true>(q, k, v, out, BH, S, s);
-    else launch_att_kernel<D, OUT, true, false>(q, k, v, out, BH, S, s);
+    if (vsd) launch_att_kernel<D, OUT, true, true>(q, k, v, out, BH, S, c, s);
+    else launch_att_kernel<D, OUT, true, false>(q, k, v, out, BH, S, c, s);
   } else {
-    if (vsd) launch_att_kernel<D, OUT, false, true>(q, k, v, out, BH, S, s);
-    else launch_att_kernel<D, OUT, false, false>(q, k, v, out, BH, S, s);
+    if (vsd) launch_att_kernel<D, OUT, false, true>(q, k, v, out, BH, S, c, s);
+    else launch_att_kernel<D, OUT, false, false>(q, k, v, out, BH, S, c, s);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
@@ -445,8 +445,9 @@ static int launch_att(const void* q, const void* k, const void* v, void* out, in
 }
 
 extern "C" int hx_fp8_attention(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t S, int64_t D,
-                                int64_t v_stride_d, int64_t v_stride_s, int out_dtype, int exact_max, void* stream) {
-  if (BH < 0 || S < 0 || D < 0) {
+                                int64_t scale_dim, int64_t v_stride_d, int64_t v_stride_s, int out_dtype, int exact_max,
+                                void* stream) {
+  if (BH < 0 || S < 0 || D < 0 || scale_dim < 0) {
     hx_set_error("hx_fp8_attention: negative size");
     return HX_ERR_BAD_ARG;
   }
@@ -464,6 +465,8 @@ extern "C" int hx_fp8_attention(const void* q, const void* k, const void* v, voi
     return HX_ERR_UNSUPPORTED;
   }
   hipStream_t s = (hipStream_t)stream;
+  // the softmax scale in base 2, evaluated the way the reference does: double arithmetic, rounded to fp32 once
+  const float c = (float)((1.0 / sqrt((double)(scale_dim > 0 ? scale_dim : (D > 0 ? D : 1)))) * 1.44269504);
   bool vsd = false, fast = (D == 64 || D == 128) && (S % ATT_BN) == 0 && ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) == 0);
   if (v_stride_s == 1 && (v_stride_d == S || D == 1)) vsd = false;       // [D][S] per head
   else if (v_stride_d == 1 && (v_stride_s == D || S == 1)) vsd = true;   // [S][D] per head
@@ -477,10 +480,10 @@ extern "C" int hx_fp8_attention(const void* q, const void* k, const void* v, voi
     const dim3 grid((unsigned)S, (unsigned)BH);
     if (out_dtype == HX_F32)
       hipLaunchKernelGGL(hx_fp8_attention_general<HX_F32>, grid, dim3(256), 0, s, (const uint8_t*)q, (const uint8_t*)k, (const uint8_t*)v,
-                         out, (int)S, (int)D, (long)v_stride_d, (long)v_stride_s);
+                         out, (int)S, (int)D, (long)v_stride_d, (long)v_stride_s, c);
     else
       hipLaunchKernelGGL(hx_fp8_attention_general<HX_E4M3>, grid, dim3(256), 0, s, (const uint8_t*)q, (const uint8_t*)k,
-                         (const uint8_t*)v, out, (int)S, (int)D, (long)v_stride_d, (long)v_stride_s);
+                         (const uint8_t*)v, out, (int)S, (int)D, (long)v_stride_d, (long)v_stride_s, c);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
       hx_set_error("hx_fp8_attention: launch failed: %s", hipGetErrorString(e));
@@ -489,9 +492,9 @@ extern "C" int hx_fp8_attention(const void* q, const void* k, const void* v, voi
     return 0;
   }
   if (D == 128) {
-    if (out_dtype == HX_F32) return launch_att<128, HX_F32>(q, k, v, out, BH, S, exact_max, vsd, s);
-    return launch_att<128, HX_E4M3>(q, k, v, out, BH, S, exact_max, vsd, s);
+    if (out_dtype == HX_F32) return launch_att<128, HX_F32>(q, k, v, out, BH, S, exact_max, vsd, c, s);
+    return launch_att<128, HX_E4M3>(q, k, v, out, BH, S, exact_max, vsd, c, s);
   }
-  if (out_dtype == HX_F32) return launch_att<64, HX_F32>(q, k, v, out, BH, S, exact_max, vsd, s);
-  return launch_att<64, HX_E4M3>(q, k, v, out, BH, S, exact_max, vsd, s);
+  if (out_dtype == HX_F32) return launch_att<64, HX_F32>(q, k, v, out, BH, S, exact_max, vsd, c, s);
+  return launch_att<64, HX_E4M3>(q, k, v, out, BH, S, exact_max, vsd, c, s);
 }

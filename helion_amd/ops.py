@@ -83,6 +83,15 @@ def fp8_attention_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batch: i
         raise ValueError(f"shape mismatch: q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)} (v must be [BH, D, S])")
     if out_dtype not in (torch.float8_e4m3fn, torch.float32):
         raise TypeError(f"unsupported out_dtype {out_dtype}")
+    d_true = d
+    if d not in (64, 128) and 0 < d < 128 and s % 64 == 0:
+        # zero-pad the head dimension to what the MFMA kernel takes: q.k and the other output columns are unchanged,
+        # the softmax scale still comes from the true head dimension
+        dp = 64 if d < 64 else 128
+        q = torch.nn.functional.pad(q.view(torch.uint8), (0, dp - d)).view(torch.float8_e4m3fn)
+        k = torch.nn.functional.pad(k.view(torch.uint8), (0, dp - d)).view(torch.float8_e4m3fn)
+        v = torch.nn.functional.pad(v.contiguous().view(torch.uint8), (0, 0, 0, dp - d)).view(torch.float8_e4m3fn)
+        d = dp
     q, k = q.contiguous(), k.contiguous()
     # v is logically [BH, D, S].  The reference's preprocessing hands it over as a permuted view of [BH, S, D]
     # memory (strides (S*D, 1, D)); the kernel reads that layout directly, so only other stridings are copied.
@@ -92,10 +101,10 @@ def fp8_attention_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batch: i
     if bh == 0 or s == 0:
         return out
     lib = _lib.load()
-    rc = lib.hx_fp8_attention(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), bh, s, d, v.stride(1), v.stride(2),
-                              _DT[out_dtype], 1 if exact_max else 0, _stream_ptr(q.device))
+    rc = lib.hx_fp8_attention(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), bh, s, d, d_true, v.stride(1),
+                              v.stride(2), _DT[out_dtype], 1 if exact_max else 0, _stream_ptr(q.device))
     _lib.check(rc, "hx_fp8_attention")
-    return out
+    return out if d == d_true else out[..., :d_true].contiguous()
 
 
 @fp8_attention_op.register_fake
@@ -323,17 +332,23 @@ def attention_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Ten
         raise ValueError("attention: no keys (softmax over an empty set)")
     if q.numel() == 0:
         return torch.empty_like(q, memory_format=torch.contiguous_format)
-    q3 = q.reshape(-1, m_dim, d).contiguous()
-    k3 = k.reshape(-1, n_dim, d).contiguous()
-    v3 = v.reshape(-1, n_dim, d).contiguous()
+    q3, k3, v3 = q.reshape(-1, m_dim, d), k.reshape(-1, n_dim, d), v.reshape(-1, n_dim, d)
     bh = q3.shape[0]
     if k3.shape[0] != bh or v3.shape[0] != bh:
         raise ValueError("attention: q, k, v disagree on the batch dimensions")
+    dp = d
+    if q.dtype != torch.float32 and d not in (64, 128) and d < 128:
+        # zero-pad the head dimension to what the MFMA kernel takes (scores and the other output columns are unchanged;
+        # the softmax scale still comes from the true head dimension)
+        dp = 64 if d < 64 else 128
+        q3, k3, v3 = (torch.nn.functional.pad(t, (0, dp - d)) for t in (q3, k3, v3))
+    q3, k3, v3 = q3.contiguous(), k3.contiguous(), v3.contiguous()
     out = torch.empty_like(q3)
-    if out.numel():
-        rc = _lib.load().hx_attention(q3.data_ptr(), k3.data_ptr(), v3.data_ptr(), out.data_ptr(), bh, m_dim, n_dim, d,
-                                      _DT[q.dtype], _stream_ptr(q.device))
-        _lib.check(rc, "hx_attention")
+    rc = _lib.load().hx_attention(q3.data_ptr(), k3.data_ptr(), v3.data_ptr(), out.data_ptr(), bh, m_dim, n_dim, dp, d,
+                                  _DT[q.dtype], _stream_ptr(q.device))
+    _lib.check(rc, "hx_attention")
+    if dp != d:
+        out = out[..., :d].contiguous()
     return out.view(q.shape)
 
 

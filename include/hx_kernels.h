@@ -83,11 +83,14 @@ int hx_fp8_gemm_path(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k
  * exact_max != 0: two passes, P is quantised to e4m3 against the exact row max (bit-faithful to
  *   the reference's ref-eager execution); exact_max == 0: one pass, online softmax, P quantised
  *   against the running max (what the reference's compiled kernel does).
+ * scale_dim: the head dimension the softmax scale 1/sqrt(.) is taken from; 0 = D.  (A caller whose head dimension is
+ *   not 64 or 128 can zero-pad q, k and v to one of them, pass the true one here and drop the padded output columns:
+ *   zero columns change neither q.k nor the other output columns.  The Python op does this.)
  * MFMA kernel: D == 128 or 64, S % 64 == 0, 16-byte aligned pointers, v in one of the two layouts above.  Every other
  * shape with D <= 256 and BH < 65536 (and any v strides within a head) runs a plain kernel that always computes the
  * exact-max form. */
-int hx_fp8_attention(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t S,
-                     int64_t D, int64_t v_stride_d, int64_t v_stride_s, int out_dtype, int exact_max, void* stream);
+int hx_fp8_attention(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t S, int64_t D,
+                     int64_t scale_dim, int64_t v_stride_d, int64_t v_stride_s, int out_dtype, int exact_max, void* stream);
 
 /* Replaces the device side of `moe_matmul_ogs(A, W, expert_token_counts, expert_token_offsets,
  * sorted_to_orig_token_idx, max_T_per_expert_tensor)` (reference: examples/moe_matmul_ogs.py:25-80;
@@ -182,11 +185,12 @@ int hx_matmul_path(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, 
  * P16 = p cast to the value dtype before the P.V product (:73-74), everything else fp32, softmax evaluated online
  * over key tiles as the reference's compiled kernel does (for 16-bit p the result does not depend on the tiling
  * beyond rounding noise; its eager mode is the one-tile case).
+ * scale_dim: the head dimension the softmax scale is taken from, 0 = D (see hx_fp8_attention).
  * q [BH, M, D], k [BH, N, D], v [BH, N, D], out [BH, M, D], contiguous, all of `dtype` (HX_BF16 / HX_F16: MFMA kernel
  * when D is 64 or 128 and the pointers are 16-byte aligned, any M and N; HX_F32 and every other D <= 256: plain
  * kernel).  hx_attention_path: 1 = MFMA kernel, 0 = plain. */
 int hx_attention(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t M, int64_t N, int64_t D,
-                 int dtype, void* stream);
+                 int64_t scale_dim, int dtype, void* stream);
 int hx_attention_path(int64_t BH, int64_t M, int64_t N, int64_t D, int dtype, const void* q, const void* k, const void* v,
                       const void* out);
 

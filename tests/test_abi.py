@@ -65,11 +65,11 @@ def test_gemm_path_selection():
 
 def test_attention_and_moe_argument_errors():
     lib = _lib.load()
-    assert lib.hx_fp8_attention(1, 1, 1, 1, -1, 64, 64, 64, 1, 3, 1, None) == -1
-    assert lib.hx_fp8_attention(16, 16, 16, 16, 2, 128, 320, 128, 1, 3, 1, None) == -2  # head dim > 256: no kernel takes it
+    assert lib.hx_fp8_attention(1, 1, 1, 1, -1, 64, 64, 0, 64, 1, 3, 1, None) == -1
+    assert lib.hx_fp8_attention(16, 16, 16, 16, 2, 128, 320, 0, 128, 1, 3, 1, None) == -2  # head dim > 256: no kernel takes it
     assert b"unsupported shape" in lib.hx_last_error()
-    assert lib.hx_fp8_attention(16, 16, 16, 16, 2, 128, 64, 128, 1, 1, 1, None) == -1  # bf16 output not offered
-    assert lib.hx_fp8_attention(None, None, None, None, 0, 128, 64, 128, 1, 3, 1, None) == 0
+    assert lib.hx_fp8_attention(16, 16, 16, 16, 2, 128, 64, 0, 128, 1, 1, 1, None) == -1  # bf16 output not offered
+    assert lib.hx_fp8_attention(None, None, None, None, 0, 128, 64, 0, 128, 1, 3, 1, None) == 0
     assert lib.hx_moe_workspace_bytes(1000, 30) >= 1000
     assert lib.hx_moe_grouped_gemm(16, 16, 16, 16, 16, 16, 8, 8, 8, 2, 8, 2, None, 0, None) == -1  # f32 tag
     assert lib.hx_moe_grouped_gemm(16, 16, 16, 16, 16, 16, 8, 8, 8, 2, 8, 1, None, 0, None) == -3  # no workspace
@@ -113,11 +113,11 @@ def test_sibling_argument_errors_are_reported_without_a_launch():
     assert lib.hx_matmul_splits(8192, 8192, 8192, 8192, 8192, 1, 8192, 1, 0) == 1
     assert lib.hx_matmul_workspace_bytes(64, 64, 32768, 32768, 64, 1, 64, 0, 0, 0, 4) == 4 * 64 * 64 * 4
     assert lib.hx_matmul_workspace_bytes(8192, 8192, 8192, 8192, 8192, 1, 8192, 1, 1, 1, 1) == 0
-    assert lib.hx_attention(None, None, None, None, -1, 4, 4, 64, 1, None) == -1
-    assert lib.hx_attention(A, A, A, A, 2, 64, 0, 64, 1, None) == -1                                     # no keys
-    assert lib.hx_attention(A, A, A, A, 2, 64, 64, 64, 3, None) == -1                                    # e4m3: not this entry
-    assert lib.hx_attention(A, A, A, A, 2, 64, 64, 320, 2, None) == -2                                   # fp32 head dim > 256
-    assert lib.hx_attention(None, None, None, None, 0, 64, 64, 64, 1, None) == 0
+    assert lib.hx_attention(None, None, None, None, -1, 4, 4, 64, 0, 1, None) == -1
+    assert lib.hx_attention(A, A, A, A, 2, 64, 0, 64, 0, 1, None) == -1                                     # no keys
+    assert lib.hx_attention(A, A, A, A, 2, 64, 64, 64, 0, 3, None) == -1                                    # e4m3: not this entry
+    assert lib.hx_attention(A, A, A, A, 2, 64, 64, 320, 0, 2, None) == -2                                   # fp32 head dim > 256
+    assert lib.hx_attention(None, None, None, None, 0, 64, 64, 64, 0, 1, None) == 0
     assert lib.hx_attention_path(2, 100, 70, 128, 1, A, A, A, A) == 1
     assert lib.hx_attention_path(2, 100, 70, 96, 1, A, A, A, A) == 0
     assert lib.hx_attention_path(2, 100, 70, 128, 2, A, A, A, A) == 0

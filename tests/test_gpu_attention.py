@@ -98,6 +98,20 @@ def test_other_shapes_run_the_plain_kernel(b, h, s, d):
     assert out8.dtype == E4M3 and rel_err(out8, orc.fp8_attention(q, k, v, b, h)) <= 0.08
 
 
+@pytest.mark.parametrize("d", [32, 96])
+def test_other_head_dims_are_zero_padded_onto_the_mfma_kernel(d):
+    b, h, s = 1, 3, 256
+    q, k, v = inputs.attention_inputs(b, h, s, d, seed=d)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    out = hx.fp8_attention_kernel(qd, kd, vd, b, h, out_dtype=torch.float32)
+    assert out.shape == (b, h, s, d) and out.is_contiguous()
+    assert rel_err(out, orc.fp8_attention(q, k, v, b, h, torch.float32)) <= 2e-2
+    v_sd = vd.transpose(1, 2).contiguous().transpose(1, 2)           # the [S][D] memory order
+    assert rel_err(hx.fp8_attention_kernel(qd, kd, v_sd, b, h, out_dtype=torch.float32), orc.fp8_attention(q, k, v, b, h, torch.float32)) <= 2e-2
+    out8 = hx.fp8_attention_kernel(qd, kd, vd, b, h)
+    assert rel_err(out8, orc.fp8_attention(q, k, v, b, h)) <= 0.08
+
+
 def test_unsupported_shapes_raise():
     x = torch.zeros(1, 64, 320).to(E4M3).to(DEV)
     with pytest.raises(ValueError, match="unsupported shape"):

@@ -59,6 +59,19 @@ def test_peaked_softmax_and_running_max_updates(dtype):
     assert rel_err(out_p, orc.attention(q, k, v)) <= 2e-2
 
 
+@pytest.mark.parametrize("d", [32, 80, 96, 112])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_other_head_dims_are_zero_padded_onto_the_mfma_kernel(d, dtype):
+    """Head dims below 128 other than 64: the op pads q, k, v with zero columns and passes the true head dim for the
+    softmax scale; same result as the oracle on the unpadded tensors, and as sdpa."""
+    q, k, v = _mk((2, 3, 150, d), 200, dtype, d)
+    out = hx.attention(q.to(DEV), k.to(DEV), v.to(DEV))
+    assert out.shape == q.shape and out.is_contiguous()
+    assert rel_err(out, orc.attention(q, k, v)) <= 2e-2
+    want = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float())
+    assert rel_err(out, want.to(dtype)) <= 2e-2
+
+
 def test_fp32_inputs_and_sdpa_relation():
     """test/test_examples.py:342-356,374-388 feed fp32 tensors of shape (1, 32, 512, 64): plain kernel."""
     q, k, v = _mk((1, 4, 128, 64), 128, torch.float32, 11)
