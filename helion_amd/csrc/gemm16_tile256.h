@@ -55,8 +55,9 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restri
   // [stage][A|W][32 KB]
   __shared__ __attribute__((aligned(1024))) uint8_t smem[2][2][MOE_TILE_BYTES];
 
-  // Grouped raster over (row tile, column tile), 8 row tiles tall.  Workgroup i runs on XCD i % 8; each run of 256
-  // workgroups covers 256 consecutive tiles of that order, 32 consecutive ones (8 row tiles x 4 column tiles) per XCD,
+  // Grouped raster over (row tile, column tile), 4 row tiles tall (measured against 2, 6, 8 and 16).  Workgroup i runs on
+  // XCD i % 8; each run of 256 workgroups covers 256 consecutive tiles of that order, 32 consecutive ones (4 row tiles x
+  // 8 column tiles) per XCD,
   // so one XCD's resident tiles share operand panels in its L2 and all eight XCDs work side by side on the same row
   // tiles and on neighbouring column panels of the same expert — the set of panels in flight then fits the memory-side
   // cache, which a contiguous range of the tile order per XCD (eight different experts at once) does not (C5: -6 %).
@@ -65,7 +66,7 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restri
     const int nwg = gridDim.x, wg = blockIdx.x, chunk = wg >> 8;
     tile = chunk < (nwg >> 8) ? (chunk << 8) + ((wg & 7) << 5) + ((wg >> 3) & 31) : wg;
   }
-  const int GM = 8;
+  const int GM = 4;
   const int group_size = GM * tiles_n;
   const int gid = tile / group_size;
   const int first_m = gid * GM;
