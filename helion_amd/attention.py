@@ -7,7 +7,7 @@ import math
 
 import torch
 
-from .ops import attention_op
+from .ops import attention_call
 
 
 def attention(q_in: torch.Tensor, k_in: torch.Tensor, v_in: torch.Tensor) -> torch.Tensor:
@@ -15,7 +15,7 @@ def attention(q_in: torch.Tensor, k_in: torch.Tensor, v_in: torch.Tensor) -> tor
     q: [..., seq_q, head_dim]; k, v: [..., seq_k, head_dim]; output: the shape and dtype of q.  As in the reference the
     softmax runs in base 2 with fp32 statistics and the probabilities are cast to the value dtype before the P.V
     product."""
-    return attention_op(q_in, k_in, v_in)
+    return attention_call(q_in, k_in, v_in)
 
 
 # examples/attention.py:89-98: the reference re-registers the same body with dynamic shapes; one kernel serves both here

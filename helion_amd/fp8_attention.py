@@ -6,7 +6,7 @@ from typing import Callable
 
 import torch
 
-from .ops import cast_e4m3_x3_op, fp8_attention_op
+from .ops import cast_e4m3_x3_call, fp8_attention_call
 
 
 def fp8_attention_kernel(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batch: int, heads: int, *,
@@ -16,7 +16,7 @@ def fp8_attention_kernel(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batc
     [batch, heads, seq, dim] float8_e4m3fn.  ``exact_max=True`` (default) quantises the un-normalised
     probabilities against the exact row max, which is what the reference computes when its kernel body
     is executed with one tile per loop; ``exact_max=False`` is the single-pass online softmax."""
-    return fp8_attention_op(q, k, v, batch, heads, out_dtype, exact_max)
+    return fp8_attention_call(q, k, v, batch, heads, out_dtype, exact_max)
 
 
 def preprocess_fp8_attention_inputs(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
@@ -26,7 +26,7 @@ def preprocess_fp8_attention_inputs(q: torch.Tensor, k: torch.Tensor, v: torch.T
     batch, heads, seq_len, head_dim = q.shape
     if (q.is_cuda and q.dtype == k.dtype == v.dtype and q.dtype in (torch.float16, torch.bfloat16, torch.float32)
             and q.shape == k.shape == v.shape and q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
-        q_fp8, k_fp8, v_fp8 = cast_e4m3_x3_op(q, k, v)
+        q_fp8, k_fp8, v_fp8 = cast_e4m3_x3_call(q, k, v)
         return (q_fp8.reshape(batch * heads, seq_len, head_dim), k_fp8.reshape(batch * heads, seq_len, head_dim),
                 v_fp8.permute(0, 1, 3, 2).reshape(batch * heads, head_dim, seq_len))
     q_fp8 = q.to(torch.float8_e4m3fn)

@@ -4,7 +4,7 @@ from __future__ import annotations
 
 import torch
 
-from .ops import fp8_gemm_op, fp8_quantize_op
+from .ops import fp8_gemm_call, fp8_quantize_call
 
 
 def fp8_gemm(x: torch.Tensor, y: torch.Tensor, *, scale_a: torch.Tensor | None = None,
@@ -13,13 +13,13 @@ def fp8_gemm(x: torch.Tensor, y: torch.Tensor, *, scale_a: torch.Tensor | None =
     examples/fp8_gemm.py:29-57).  x: [m,k] float8_e4m3fn, y: [k,n] float8_e4m3fn with any strides
     (column-major y, strides (1,k), is the fast layout).  Keyword-only extensions, all defaulting to
     the reference behaviour: per-tensor fp32 scales (one-element device tensors) and ``out_dtype``."""
-    return fp8_gemm_op(x, y, scale_a, scale_b, out_dtype)
+    return fp8_gemm_call(x, y, scale_a, scale_b, out_dtype)
 
 
 def fp8_gemm_scaled(x: torch.Tensor, y: torch.Tensor, scale_a: torch.Tensor, scale_b: torch.Tensor,
                     out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """``cast((x @ y) * scale_a * scale_b)`` — the per-tensor-scaled form torch._scaled_mm computes."""
-    return fp8_gemm_op(x, y, scale_a, scale_b, out_dtype)
+    return fp8_gemm_call(x, y, scale_a, scale_b, out_dtype)
 
 
 def fp8_quantize_per_tensor(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
@@ -27,7 +27,7 @@ def fp8_quantize_per_tensor(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor
     (1 for an all-zero tensor) and ``q = (x * (448 / max|x|)).to(float8_e4m3fn)``, so ``q.float() * scale ~ x``.
     Three launches, no host synchronisation.  (The reference's example only ever passes unit scales,
     examples/fp8_gemm.py:74-78; this is the producer of real ones.)"""
-    return fp8_quantize_op(x)
+    return fp8_quantize_call(x)
 
 
 def reference_fp8_gemm_pytorch(x_fp8: torch.Tensor, y_fp8: torch.Tensor) -> torch.Tensor:

@@ -13,7 +13,7 @@ from typing import Callable
 import torch
 from torch import Tensor
 
-from .ops import matmul_op
+from .ops import matmul_call
 
 
 class BiasEpilogue:
@@ -45,12 +45,12 @@ def relu() -> BiasEpilogue:
 def _run(x: Tensor, y: Tensor, epilogue: Callable | None, split_k: int) -> Tensor:
     dt = torch.promote_types(x.dtype, y.dtype)
     if epilogue is None:
-        return matmul_op(x, y, None, False, dt, split_k)
+        return matmul_call(x, y, None, False, dt, split_k)
     if isinstance(epilogue, BiasEpilogue):
-        return matmul_op(x, y, epilogue.bias, epilogue.relu, dt, split_k)
+        return matmul_call(x, y, epilogue.bias, epilogue.relu, dt, split_k)
     # arbitrary callable: the kernel hands back the fp32 accumulator (examples/matmul.py:51-55: acc is fp32 and the
     # epilogue's result is cast on the store); the one-tile view of the reference's eager mode is tile = whole dims
-    acc = matmul_op(x, y, None, False, torch.float32, split_k)
+    acc = matmul_call(x, y, None, False, torch.float32, split_k)
     m, n = acc.shape
     return epilogue(acc, (slice(0, m), slice(0, n))).to(dt)
 

@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import torch
 
-from .ops import moe_matmul_ogs_op, moe_matmul_topk_op, moe_routing_op
+from .ops import moe_matmul_ogs_call, moe_matmul_topk_call, moe_routing_call
 
 
 def moe_matmul_ogs(A: torch.Tensor, W: torch.Tensor, expert_token_counts: torch.Tensor,
@@ -12,7 +12,7 @@ def moe_matmul_ogs(A: torch.Tensor, W: torch.Tensor, expert_token_counts: torch.
     """``C[r] = A[r] @ W[e]`` for every row r routed to expert e (reference: examples/moe_matmul_ogs.py:25-80).
     A: [T,K], W: [E,K,N]; returns [T,N] in promote_types(A.dtype, W.dtype).  As in the reference only the
     *numel* of ``max_T_per_expert_tensor`` is used."""
-    return moe_matmul_ogs_op(A, W, expert_token_counts, expert_token_offsets, sorted_to_orig_token_idx,
+    return moe_matmul_ogs_call(A, W, expert_token_counts, expert_token_offsets, sorted_to_orig_token_idx,
                              int(max_T_per_expert_tensor.numel()))
 
 
@@ -23,7 +23,7 @@ def moe_matmul_ogs_helion_kernel_args_gen(A: torch.Tensor, W: torch.Tensor, top1
     E = W.size(0)
     device = A.device
     if A.is_cuda and E <= 512 and top1_expert_per_token.dtype in (torch.int32, torch.int64):
-        counts, offsets, idx, max_count = moe_routing_op(top1_expert_per_token, E)
+        counts, offsets, idx, max_count = moe_routing_call(top1_expert_per_token, E)
         return (A, W, counts, offsets, idx, torch.empty(int(max_count.item()), device=device))
     sorted_to_orig_token_idx = torch.argsort(top1_expert_per_token, stable=True).to(torch.int32)
     expert_token_counts = torch.bincount(top1_expert_per_token, minlength=E).to(torch.int32)
@@ -40,13 +40,13 @@ def moe_matmul_topk(A: torch.Tensor, W: torch.Tensor, expert_ids: torch.Tensor, 
     ``expert_ids`` holds T_tok*top_k ids (token-major, i.e. ``topk_indices.reshape(-1)``), the result is
     [T_tok*top_k, N] with row r = A[r // top_k] @ W[expert_ids[r]].  Equals
     ``moe_matmul_ogs(*moe_matmul_ogs_helion_kernel_args_gen(A.repeat_interleave(top_k, 0), W, expert_ids))``."""
-    return moe_matmul_topk_op(A, W, expert_ids, int(top_k))
+    return moe_matmul_topk_call(A, W, expert_ids, int(top_k))
 
 
 def moe_routing(expert_ids: torch.Tensor, num_experts: int):
     """(counts, offsets, sorted_to_orig_idx, max_count) as int32 device tensors from one kernel; the tensor form
     of examples/moe_matmul_ogs.py:98-113 with ``max_count`` left on the device."""
-    return moe_routing_op(expert_ids, int(num_experts))
+    return moe_routing_call(expert_ids, int(num_experts))
 
 
 def moe_matmul_ogs_reference(A: torch.Tensor, W: torch.Tensor, top1_expert_per_token: torch.Tensor) -> torch.Tensor:

@@ -15,6 +15,15 @@ def _stream_ptr(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
+def eager(op_impl, op, *args):
+    """Call the op's implementation directly for plain CUDA tensors in eager mode (the dispatcher round trip of a
+    custom op costs more than a small kernel), and through the registered op when tracing / compiling or for anything
+    else (fake or meta tensors get shape inference there, CPU tensors their error)."""
+    if not torch.compiler.is_compiling() and all(type(a) is torch.Tensor and a.is_cuda for a in args if isinstance(a, torch.Tensor)):
+        return op_impl(*args)
+    return op(*args)
+
+
 def _require_cuda(*tensors: torch.Tensor) -> None:
     for t in tensors:
         if t is not None and not t.is_cuda:
@@ -22,8 +31,7 @@ def _require_cuda(*tensors: torch.Tensor) -> None:
 
 
 # ------------------------------------------------------------------------------ fp8 gemm
-@torch.library.custom_op("helion_amd::fp8_gemm", mutates_args=())
-def fp8_gemm_op(x: torch.Tensor, y: torch.Tensor, scale_a: torch.Tensor | None, scale_b: torch.Tensor | None,
+def _fp8_gemm_impl(x: torch.Tensor, y: torch.Tensor, scale_a: torch.Tensor | None, scale_b: torch.Tensor | None,
                 out_dtype: torch.dtype) -> torch.Tensor:
     _require_cuda(x, y, scale_a, scale_b)
     if x.dtype != torch.float8_e4m3fn or y.dtype != torch.float8_e4m3fn:
@@ -61,14 +69,16 @@ def fp8_gemm_op(x: torch.Tensor, y: torch.Tensor, scale_a: torch.Tensor | None, 
     return out
 
 
+fp8_gemm_op = torch.library.custom_op("helion_amd::fp8_gemm", mutates_args=())(_fp8_gemm_impl)
+
+
 @fp8_gemm_op.register_fake
 def _(x, y, scale_a, scale_b, out_dtype):
     return x.new_empty((x.shape[0], y.shape[1]), dtype=out_dtype)
 
 
 # ------------------------------------------------------------------------------ fp8 attention
-@torch.library.custom_op("helion_amd::fp8_attention", mutates_args=())
-def fp8_attention_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batch: int, heads: int,
+def _fp8_attention_impl(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batch: int, heads: int,
                      out_dtype: torch.dtype, exact_max: bool) -> torch.Tensor:
     _require_cuda(q, k, v)
     for t in (q, k, v):
@@ -107,14 +117,16 @@ def fp8_attention_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batch: i
     return out if d == d_true else out[..., :d_true].contiguous()
 
 
+fp8_attention_op = torch.library.custom_op("helion_amd::fp8_attention", mutates_args=())(_fp8_attention_impl)
+
+
 @fp8_attention_op.register_fake
 def _(q, k, v, batch, heads, out_dtype, exact_max):
     return q.new_empty((batch, heads, q.shape[1], q.shape[2]), dtype=out_dtype)
 
 
 # ------------------------------------------------------------------------------ moe grouped gemm
-@torch.library.custom_op("helion_amd::moe_matmul_ogs", mutates_args=())
-def moe_matmul_ogs_op(A: torch.Tensor, W: torch.Tensor, expert_token_counts: torch.Tensor,
+def _moe_matmul_ogs_impl(A: torch.Tensor, W: torch.Tensor, expert_token_counts: torch.Tensor,
                       expert_token_offsets: torch.Tensor, sorted_to_orig_token_idx: torch.Tensor,
                       max_T_per_expert: int) -> torch.Tensor:
     _require_cuda(A, W, expert_token_counts, expert_token_offsets, sorted_to_orig_token_idx)
@@ -147,14 +159,16 @@ def moe_matmul_ogs_op(A: torch.Tensor, W: torch.Tensor, expert_token_counts: tor
     return C
 
 
+moe_matmul_ogs_op = torch.library.custom_op("helion_amd::moe_matmul_ogs", mutates_args=())(_moe_matmul_ogs_impl)
+
+
 @moe_matmul_ogs_op.register_fake
 def _(A, W, expert_token_counts, expert_token_offsets, sorted_to_orig_token_idx, max_T_per_expert):
     return A.new_empty((A.shape[0], W.shape[2]), dtype=torch.promote_types(A.dtype, W.dtype))
 
 
 # ------------------------------------------------------------------------------ moe routing tables
-@torch.library.custom_op("helion_amd::moe_routing", mutates_args=())
-def moe_routing_op(expert_ids: torch.Tensor, num_experts: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+def _moe_routing_impl(expert_ids: torch.Tensor, num_experts: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """(counts [E], offsets [E+1], idx [T], max_count [1]), all int32 on the device, no host synchronisation."""
     _require_cuda(expert_ids)
     if expert_ids.dim() != 1 or expert_ids.dtype not in (torch.int32, torch.int64):
@@ -176,6 +190,9 @@ def moe_routing_op(expert_ids: torch.Tensor, num_experts: int) -> tuple[torch.Te
     return counts, offsets, idx, max_count
 
 
+moe_routing_op = torch.library.custom_op("helion_amd::moe_routing", mutates_args=())(_moe_routing_impl)
+
+
 @moe_routing_op.register_fake
 def _(expert_ids, num_experts):
     i32 = dict(dtype=torch.int32)
@@ -184,8 +201,7 @@ def _(expert_ids, num_experts):
 
 
 # ------------------------------------------------------------------------------ moe top-k matmul (routing fused in)
-@torch.library.custom_op("helion_amd::moe_matmul_topk", mutates_args=())
-def moe_matmul_topk_op(A: torch.Tensor, W: torch.Tensor, expert_ids: torch.Tensor, top_k: int) -> torch.Tensor:
+def _moe_matmul_topk_impl(A: torch.Tensor, W: torch.Tensor, expert_ids: torch.Tensor, top_k: int) -> torch.Tensor:
     _require_cuda(A, W, expert_ids)
     if A.dim() != 2 or W.dim() != 3:
         raise ValueError("moe_matmul_topk expects A [T_tok,K] and W [E,K,N]")
@@ -215,14 +231,16 @@ def moe_matmul_topk_op(A: torch.Tensor, W: torch.Tensor, expert_ids: torch.Tenso
     return C
 
 
+moe_matmul_topk_op = torch.library.custom_op("helion_amd::moe_matmul_topk", mutates_args=())(_moe_matmul_topk_impl)
+
+
 @moe_matmul_topk_op.register_fake
 def _(A, W, expert_ids, top_k):
     return A.new_empty((A.shape[0] * top_k, W.shape[2]), dtype=torch.promote_types(A.dtype, W.dtype))
 
 
 # ------------------------------------------------------------------------------ casts / quantisation in front of the fp8 kernels
-@torch.library.custom_op("helion_amd::cast_e4m3_x3", mutates_args=())
-def cast_e4m3_x3_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+def _cast_e4m3_x3_impl(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Three equally sized contiguous fp16/bf16/fp32 tensors -> e4m3 (same shapes), one launch."""
     _require_cuda(q, k, v)
     if not (q.dtype == k.dtype == v.dtype) or q.dtype not in _DT or q.dtype == torch.float8_e4m3fn:
@@ -238,14 +256,16 @@ def cast_e4m3_x3_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> tuple[
     return outs[0], outs[1], outs[2]
 
 
+cast_e4m3_x3_op = torch.library.custom_op("helion_amd::cast_e4m3_x3", mutates_args=())(_cast_e4m3_x3_impl)
+
+
 @cast_e4m3_x3_op.register_fake
 def _(q, k, v):
     f8 = torch.float8_e4m3fn
     return q.new_empty(q.shape, dtype=f8), k.new_empty(k.shape, dtype=f8), v.new_empty(v.shape, dtype=f8)
 
 
-@torch.library.custom_op("helion_amd::fp8_quantize", mutates_args=())
-def fp8_quantize_op(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+def _fp8_quantize_impl(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     """(e4m3 tensor of x's shape, 0-d fp32 scale) with x ~ q * scale; scale = max|x| / 448."""
     _require_cuda(x)
     if x.dtype not in (torch.float16, torch.bfloat16, torch.float32):
@@ -262,14 +282,16 @@ def fp8_quantize_op(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     return q, scale
 
 
+fp8_quantize_op = torch.library.custom_op("helion_amd::fp8_quantize", mutates_args=())(_fp8_quantize_impl)
+
+
 @fp8_quantize_op.register_fake
 def _(x):
     return x.new_empty(x.shape, dtype=torch.float8_e4m3fn), x.new_empty((), dtype=torch.float32)
 
 
 # ------------------------------------------------------------------------------ dense matmul (+ bias, relu, split-K)
-@torch.library.custom_op("helion_amd::matmul", mutates_args=())
-def matmul_op(x: torch.Tensor, y: torch.Tensor, bias: torch.Tensor | None, relu: bool, out_dtype: torch.dtype,
+def _matmul_impl(x: torch.Tensor, y: torch.Tensor, bias: torch.Tensor | None, relu: bool, out_dtype: torch.dtype,
               split_k: int) -> torch.Tensor:
     _require_cuda(x, y, bias)
     if x.dim() != 2 or y.dim() != 2:
@@ -311,14 +333,16 @@ def matmul_op(x: torch.Tensor, y: torch.Tensor, bias: torch.Tensor | None, relu:
     return out
 
 
+matmul_op = torch.library.custom_op("helion_amd::matmul", mutates_args=())(_matmul_impl)
+
+
 @matmul_op.register_fake
 def _(x, y, bias, relu, out_dtype, split_k):
     return x.new_empty((x.shape[0], y.shape[1]), dtype=out_dtype)
 
 
 # ------------------------------------------------------------------------------ 16-bit attention
-@torch.library.custom_op("helion_amd::attention", mutates_args=())
-def attention_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+def _attention_impl(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
     _require_cuda(q, k, v)
     if q.dtype not in (torch.float16, torch.bfloat16, torch.float32) or k.dtype != q.dtype or v.dtype != q.dtype:
         raise TypeError(f"attention expects q, k, v of one dtype out of float16, bfloat16, float32; got {q.dtype}, {k.dtype}, {v.dtype}")
@@ -352,6 +376,27 @@ def attention_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Ten
     return out.view(q.shape)
 
 
+attention_op = torch.library.custom_op("helion_amd::attention", mutates_args=())(_attention_impl)
+
+
 @attention_op.register_fake
 def _(q, k, v):
     return torch.empty_like(q, memory_format=torch.contiguous_format)
+
+
+# ------------------------------------------------------------------------------ what the Python entry points call
+def _caller(impl, op):
+    def call(*args):
+        return eager(impl, op, *args)
+    return call
+
+
+fp8_gemm_call = _caller(_fp8_gemm_impl, fp8_gemm_op)
+fp8_attention_call = _caller(_fp8_attention_impl, fp8_attention_op)
+moe_matmul_ogs_call = _caller(_moe_matmul_ogs_impl, moe_matmul_ogs_op)
+moe_routing_call = _caller(_moe_routing_impl, moe_routing_op)
+moe_matmul_topk_call = _caller(_moe_matmul_topk_impl, moe_matmul_topk_op)
+cast_e4m3_x3_call = _caller(_cast_e4m3_x3_impl, cast_e4m3_x3_op)
+fp8_quantize_call = _caller(_fp8_quantize_impl, fp8_quantize_op)
+matmul_call = _caller(_matmul_impl, matmul_op)
+attention_call = _caller(_attention_impl, attention_op)

@@ -75,3 +75,14 @@ def test_graph_capture_and_replay():
         torch.cuda.synchronize()
         for n in cases:
             assert torch.equal(outs[n], want[n]), (n, replay)
+
+
+def test_entry_points_trace_under_torch_compile():
+    """In eager mode the entry points call the implementation directly; while tracing they go through the registered
+    ops (shape inference on fake tensors).  Dynamo with the pass-through backend: no code generation involved."""
+    cases = _cases()
+    for name in ("fp8_gemm", "matmul_bias_relu", "attention16", "fp8_attention"):
+        fn = cases[name]
+        want = fn()
+        got = torch.compile(fn, backend="eager", fullgraph=True)()
+        assert torch.equal(got, want), name
