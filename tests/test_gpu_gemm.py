@@ -25,6 +25,7 @@ def _path(m, n, k):
 @pytest.mark.parametrize("m,n,k,path", [
     (4096, 4096, 128, 1), (2048, 6144, 256, 1),                                                      # enough full 256x256 tiles
     (256, 256, 256, 5), (512, 512, 512, 5), (1024, 1024, 1024, 5), (256, 768, 128, 5), (768, 256, 1152, 5),   # too few: 128-column tiles
+    (64, 28672, 256, 5), (128, 40000, 128, 5), (90, 20000, 128, 5),      # one row tile: column pitch 112 / 128 / 80
     (48, 1024, 512, 5), (100, 3000, 256, 5), (129, 520, 384, 5), (256, 1000, 128, 5), (200, 136, 1280, 5), (33, 256, 256, 5),
     (1000, 1000, 1024, 5), (300, 200, 256, 5), (257, 255, 128, 5), (32, 64, 8192 + 128, 5), (255, 1, 128, 5),
     (16, 512, 1024, 2), (1, 16, 128, 2), (5, 48, 256, 2), (16, 1000, 384, 2), (9, 33, 8192 + 128, 2), (16, 64, 16384, 2),
