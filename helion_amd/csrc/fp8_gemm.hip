@@ -731,6 +731,17 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_general(const uint8_t* __rest
 // ------------------------------------------------------------------------------------------
 static inline bool aligned(const void* p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
+// Which tile for a K-contiguous problem: 256x256 (returns 0), 256x128 or 128x128 (returns the tile's rows).  All three
+// run one workgroup per CU, so a launch takes ceil(tiles / 256) rounds of K / 128 k-tile steps; per step the 128x128
+// tile costs about 0.6 and the 256x128 tile about 0.8 of the 256x256 tile's when fed from L2 (measured), and a single
+// row tile that streams weights from HBM costs what the stream costs.
+static int tileN128_rows(int64_t M, int64_t N) {
+  auto rounds = [&](int64_t bm, int64_t bn) { return (((M + bm - 1) / bm) * ((N + bn - 1) / bn) + 255) / 256; };
+  if (M <= 128) return 128;
+  if (M <= 256) return 256;
+  return 60 * rounds(128, 128) < 106 * rounds(256, 256) ? 128 : 0;
+}
+
 // 0 general, 1 tile256, 2 skinny, 3 tile256 with edge tiles (M or N not a multiple of 256, K not of 128),
 // 5 tileN128 (too few 256x256 tiles to occupy the chip)
 static int gemm_path_kmajor(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, const void* a, const void* b,
@@ -740,7 +751,10 @@ static int gemm_path_kmajor(int64_t M, int64_t N, int64_t K, int64_t lda, int64_
   const bool ktail = K % 128 != 0;  // only the edge instantiation of the tile kernel pads a partial last k-tile
   if (!ktail && (M <= 16 || (M <= 32 && K <= 8192)) && lda >= K && ldb >= K) return 2;
   if (lda >= (1LL << 27) || ldb >= (1LL << 27)) return 0;
-  if (!ktail && ((M + 255) / 256) * ((N + 255) / 256) < 192 && M * lda < (1LL << 32) && N * ldb < (1LL << 32)) return 5;
+  // 128-column tiles or 256x256 tiles?  Both run one workgroup per CU, so a launch takes ceil(tiles / 256) rounds of K / 128
+  // k-tile steps; a step of the small tile costs about 0.6 of a step of the large one when it is fed from L2 (measured),
+  // and far less when a single row tile streams weights from HBM.
+  if (!ktail && M * lda < (1LL << 32) && N * ldb < (1LL << 32) && tileN128_rows(M, N) != 0) return 5;
   if (!ktail && (M % 256 == 0) && (N % 256 == 0) && (ldc % 8 == 0) && aligned(c, 16)) return 1;  // 16-byte row-aligned stores
   if (M * lda < (1LL << 32) && N * ldb < (1LL << 32)) return 3;
   return 0;
@@ -782,9 +796,10 @@ static void launch_kmajor(int path, const void* a, const void* bt, void* c, int6
       if (per <= 8) bn = (int)(16 * (per < 4 ? 4 : per));
     }
     const int tiles_n = (int)((N + bn - 1) / bn);
-    if (M > 128 && M <= 256)  // one 256-row tile instead of a full and a mostly padded 128-row tile
-      hipLaunchKernelGGL((hx_fp8_gemm_tileN128<OUT, 256>), dim3(tiles_n), dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
-                         (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, 1, bn);
+    if (tileN128_rows(M, N) == 256)
+      hipLaunchKernelGGL((hx_fp8_gemm_tileN128<OUT, 256>), dim3((unsigned)((M + 255) / 256) * tiles_n), dim3(256), 0, stream,
+                         (const uint8_t*)a, (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa,
+                         sb, (int)((M + 255) / 256), bn);
     else
       hipLaunchKernelGGL((hx_fp8_gemm_tileN128<OUT, 128>), dim3((unsigned)((M + 127) / 128) * tiles_n), dim3(256), 0, stream,
                          (const uint8_t*)a, (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa,

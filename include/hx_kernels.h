@@ -65,8 +65,9 @@ size_t hx_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t ldb_
 
 /* Which kernel hx_fp8_gemm would launch for these arguments: 0 general (or, given a workspace, transpose + fast
  * path), 1 tile256, 2 skinny, 3 tile256 with guarded edge tiles (M or N not a multiple of 256), 4 tile256 reading a
- * row-major B in place (edges included), 5 the 128-column tile kernel (column-major B, K % 128 == 0, fewer than 192
- * 256x256 tiles: decode batches of 33..256 rows, mid-size products).
+ * row-major B in place (edges included), 5 the 128-column tile kernel (column-major B, K % 128 == 0, taken while its
+ * rounds of tiles are estimated to finish before those of 256x256 tiles: decode batches of 33..256 rows, small and
+ * mid-size products).
  * (Diagnostic; lets tests assert that the fast paths are the ones exercised.) */
 int hx_fp8_gemm_path(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n,
                      int64_t ldc, const void* a, const void* b, const void* c);
