@@ -731,10 +731,11 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_general(const uint8_t* __rest
 // ------------------------------------------------------------------------------------------
 static inline bool aligned(const void* p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
-// Which tile for a K-contiguous problem: 256x256 (returns 0), 256x128 or 128x128 (returns the tile's rows).  All three
-// run one workgroup per CU, so a launch takes ceil(tiles / 256) rounds of K / 128 k-tile steps; per step the 128x128
-// tile costs about 0.6 and the 256x128 tile about 0.8 of the 256x256 tile's when fed from L2 (measured), and a single
-// row tile that streams weights from HBM costs what the stream costs.
+// Which tile for a K-contiguous problem: 256x256 (returns 0) or 128 columns wide (returns the tile's rows: one row tile
+// of 128 or 256 rows for a decode batch that streams weights from HBM, 128 otherwise).  Both kernels run one workgroup
+// per CU, so a launch takes ceil(tiles / 256) rounds of K / 128 k-tile steps; per step the 128x128 tile costs about 0.6
+// of the 256x256 tile's when fed from L2 (measured: it is bound by what a CU can pull from L2, not by the MFMAs).  A
+// 256x128 tile for more than 256 rows measured no better than either.
 static int tileN128_rows(int64_t M, int64_t N) {
   auto rounds = [&](int64_t bm, int64_t bn) { return (((M + bm - 1) / bm) * ((N + bn - 1) / bn) + 255) / 256; };
   if (M <= 128) return 128;

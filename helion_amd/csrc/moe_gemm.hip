@@ -8,10 +8,11 @@
 //   1. hx_moe_prep       : builds the tile table (tile -> expert, first sorted row, row count) from
 //                          counts/offsets on the device and clears the row-covered flags;
 //   2. hx_moe_mark       : flags every row some expert covers;
-//   3. hx_moe_tile256 / hx_moe_general : the grouped GEMM over (row tile, column tile) pairs;
+//   3. hx_gemm16_tile256 / _tile128 / _rows32 or hx_moe_general : the grouped GEMM over (row tile, column tile) pairs;
 //   4. hx_moe_zero_rows  : zero-fills rows whose flag is still clear.
 // Padded rows of a tile are never stored, so there is no read-modify-write and no write race.
 #include "gemm16_tile128.h"
+#include "gemm16_rows32.h"
 
 // workspace layout: [0] int num_tiles | [16 ..) MoeTile table[max_tiles] | flags[T] bytes
 static inline size_t moe_table_bytes(int64_t max_tiles) { return 16 + (size_t)max_tiles * sizeof(MoeTile); }
@@ -129,8 +130,8 @@ __global__ __launch_bounds__(256) void hx_moe_general(const T16* __restrict__ A,
 // ------------------------------------------------------------------------------------------
 extern "C" size_t hx_moe_workspace_bytes(int64_t T, int64_t E) {
   if (T < 0 || E < 0) return 0;
-  // sized for the smaller row tile (64), which needs the longer table
-  size_t b = moe_table_bytes(moe_max_tiles(T, E, 64));
+  // sized for the smallest row tile (32), which needs the longest table
+  size_t b = moe_table_bytes(moe_max_tiles(T, E, 32));
   b = (b + 255) & ~(size_t)255;
   return b + (size_t)T + 256;
 }
@@ -144,11 +145,13 @@ static int launch_moe(const void* A, const void* W, void* C, const int32_t* coun
   // not fill the chip; 256-row tiles otherwise (half the operand traffic per flop)
   const int64_t tn256 = (N + MOE_BN - 1) / MOE_BN;
   const bool small = E > 0 && (T / E < 512 || ((T + MOE_BM - 1) / MOE_BM + E / 2) * tn256 < 192);
-  const int bm = fast ? (small ? G128_BM : MOE_BM) : 64;
+  // a handful of rows in all: 32-row tiles (a quarter of the A bytes per stage, more weight bytes in flight per CU)
+  const bool few = T <= R32_BM;
+  const int bm = fast ? (few ? R32_BM : small ? G128_BM : MOE_BM) : 64;
   const int max_tiles = (int)moe_max_tiles(T, E, bm);
   int* num_tiles = (int*)ws;
   MoeTile* table = (MoeTile*)((uint8_t*)ws + 16);
-  size_t tb = moe_table_bytes(moe_max_tiles(T, E, 64));
+  size_t tb = moe_table_bytes(moe_max_tiles(T, E, 32));
   tb = (tb + 255) & ~(size_t)255;
   uint8_t* flags = (uint8_t*)ws + tb;
 
@@ -160,7 +163,12 @@ static int launch_moe(const void* A, const void* W, void* C, const int32_t* coun
   if (fast) {
     G16Dense d = {};
     d.lda = K; d.ldb = N; d.ldc = N;
-    if (bm == MOE_BM) {
+    if (bm == R32_BM) {
+      const int tiles_n = (int)((N + R32_BN - 1) / R32_BN);
+      hipLaunchKernelGGL((hx_gemm16_rows32<BF, 3>), dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W,
+                         (void*)C, (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, max_tiles, tiles_n,
+                         (int)a_div, d);
+    } else if (bm == MOE_BM) {
       const int tiles_n = (int)tn256;
       hipLaunchKernelGGL((hx_gemm16_tile256<BF, 0>), dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W,
                          (void*)C, (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, max_tiles, tiles_n,

@@ -32,6 +32,10 @@ def _run(A, W, ex):
     (600, 64, 1408, 8, 2, torch.float16),      # N = 5.5 tiles
     (256, 64, 8, 2, 1, torch.bfloat16),        # a single column tile with one valid 16-byte chunk
     (300, 192, 200, 5, 1, torch.bfloat16),     # N % 8 == 0, nothing else aligned
+    (32, 256, 512, 8, 1, torch.bfloat16),      # a decode batch: the 32-row tile kernel
+    (16, 512, 264, 4, 2, torch.float16),       # ... top-2, ragged last column tile
+    (7, 64, 128, 3, 1, torch.bfloat16),        # ... one k-tile, fewer rows than experts' tiles
+    (24, 1024, 1408, 40, 1, torch.bfloat16),   # ... more experts than rows
 ])
 def test_shapes_vs_oracle(T, K, N, E, topk, dtype):
     A, W, ex = inputs.moe_inputs(T // topk, K, N, E, topk, seed=T + K, dtype=dtype)
