@@ -326,13 +326,13 @@ __global__ __launch_bounds__(256) void hx_transpose_u8(const uint8_t* __restrict
 // the column tiles come to about one per CU (N = 28672: 112 columns, 256 tiles); the columns of a tile past bn
 // re-read its last column (an L2 hit, no HBM traffic) and are not stored.
 // ------------------------------------------------------------------------------------------
-template <int OUT, int BM>
+template <int OUT, int BM, bool PAIR = false>
 __global__ __launch_bounds__(256) void hx_fp8_gemm_tileN128(const uint8_t* __restrict__ A, const uint8_t* __restrict__ Bt,
                                                            typename OutT<OUT>::T* __restrict__ C, int M, int N, int K, long lda,
                                                            long ldb, long ldc, const float* __restrict__ scale_a,
                                                            const float* __restrict__ scale_b, int tiles_m, int bn) {
   typedef typename OutT<OUT>::T out_t;
-  constexpr int NS = BM == 128 ? 4 : 3;                  // 128 KB or 144 KB of LDS
+  constexpr int NS = BM == 64 ? 6 : BM == 128 ? 4 : 3;   // 144, 128 or 144 KB of LDS
   constexpr int STAGE = (BM + 128) * 128;                // bytes of one stage: A tile, then B tile
   constexpr int WMB = BM / 32;                           // 16-row blocks per wave
   constexpr int AJ = BM / 32, IPW = AJ + 4;              // DMA instructions per wave per k-tile: A, B
@@ -394,34 +394,53 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tileN128(const uint8_t* __res
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < WMB; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
-  // the MFMAs of one k-tile with the DMA instructions of tile dkt between them, one after every other MFMA (a burst of
-  // them right after the barrier would hold the in-order instruction stream up)
-  auto mma = [&](v8i(&fa)[WMB], v8i(&fb)[4], int dkt) {
+  // the MFMAs of one k-tile with the DMA instructions of tile dkt between them, one after every other MFMA (after
+  // every MFMA where there are fewer than two per instruction): a burst of them right after the barrier would hold the
+  // in-order instruction stream up
+  constexpr int EVERY = 4 * WMB >= 2 * IPW ? 2 : 1;
+  constexpr int PER = (2 * IPW + 4 * WMB - 1) / (4 * WMB);  // PAIR: DMA instructions after each MFMA of an issuing step
+  static_assert(4 * WMB >= EVERY * IPW, "every DMA instruction of a k-tile has an MFMA to follow");
+  // PAIR: the DMA of two consecutive k-tiles is issued in the same step, at every other step and row piece by row
+  // piece, so that memory sees both 128-byte halves of 256 contiguous bytes of a row back to back (a single row tile
+  // streams its weights from HBM, and lone 128-byte pieces 8 KB apart cost a DRAM row activation each: 50.5 -> 47.5 us
+  // for 33..64 rows against 28672 x 8192 weights).  It needs the six-stage ring of the 64-row tile: with four stages
+  // the wait for the first tile of a pair leaves nothing in flight, and 65..128 rows measured slower paired.
+  auto mma = [&](v8i(&fa)[WMB], v8i(&fb)[4], int dkt, bool two) {
 #pragma unroll
     for (int i = 0; i < 4 * WMB; ++i) {
       acc[i & 3][i >> 2] = hx_mfma_16x16x128_e4m3(fb[i & 3], fa[i >> 2], acc[i & 3][i >> 2]);
-      if ((i & 1) && (i >> 1) < IPW) issue_one(dkt, i >> 1);
+      if (!PAIR) {
+        if (i % EVERY == EVERY - 1 && i / EVERY < IPW) issue_one(dkt, i / EVERY);
+      } else if (two) {  // row piece by row piece: (dkt-1, 0), (dkt, 0), (dkt-1, 1), ...; the counted waits rely on that order
+#pragma unroll
+        for (int q = PER * i; q < PER * (i + 1) && q < 2 * IPW; ++q) issue_one((q & 1) ? dkt : dkt - 1, q >> 1);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-  // step kt: tile kt is in `cur`; tiles kt+1 .. kt+NS-1 are landed or in flight
-  auto step = [&](v8i(&ca)[WMB], v8i(&cb)[4], v8i(&na)[WMB], v8i(&nb)[4], int kt) {
-    __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 2) * IPW));  // this wave's part of tile kt+1 has landed
+  // step kt: tile kt is in `cur`; tiles kt+1 .. are landed or in flight.  Without PAIR every step issues tile kt+NS;
+  // with it the even steps issue tiles kt+NS-1 and kt+NS (the stages of tiles kt-1 and kt) and the odd steps none.
+  auto step = [&](v8i(&ca)[WMB], v8i(&cb)[4], v8i(&na)[WMB], v8i(&nb)[4], int kt, bool even) {
+    // this wave's part of tile kt+1 has landed
+    // (PAIR, even step: tile kt+1 is the first of its pair, so only the last instruction of that pair, which belongs to
+    // the second tile, and the pairs issued since may be outstanding)
+    if (PAIR && even) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(PAIR ? (NS - 4) * IPW + 1 : 0));
+    else __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 2) * IPW));
     __syncthreads();             // ... everybody's has, and every wave holds tile kt in registers: its stage is free
     if (kt + 1 < nk) load_frags(na, nb, kt + 1);
-    mma(ca, cb, kt + NS);
+    mma(ca, cb, kt + NS, even);
   };
-  for (int t = 0; t < NS; ++t) issue(t);
-  __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 1) * IPW));
+  for (int t = 0; t < (PAIR ? NS - 1 : NS); ++t) issue(t);
+  __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((PAIR ? NS - 2 : NS - 1) * IPW));
   __syncthreads();
   v8i fa0[WMB], fb0[4], fa1[WMB], fb1[4];
   load_frags(fa0, fb0, 0);
   int kt = 0;
   for (; kt + 1 < nk; kt += 2) {
-    step(fa0, fb0, fa1, fb1, kt);
-    step(fa1, fb1, fa0, fb0, kt + 1);
+    step(fa0, fb0, fa1, fb1, kt, true);
+    step(fa1, fb1, fa0, fb0, kt + 1, false);
   }
-  if (kt < nk) step(fa0, fb0, fa1, fb1, kt);
+  if (kt < nk) step(fa0, fb0, fa1, fb1, kt, true);
   HX_WAIT_VM0();  // no DMA may still be writing this workgroup's LDS when it ends
 
   float alpha = 1.f;
@@ -738,6 +757,7 @@ static inline bool aligned(const void* p, size_t a) { return ((uintptr_t)p & (a 
 // 256x128 tile for more than 256 rows measured no better than either.
 static int tileN128_rows(int64_t M, int64_t N) {
   auto rounds = [&](int64_t bm, int64_t bn) { return (((M + bm - 1) / bm) * ((N + bn - 1) / bn) + 255) / 256; };
+  if (M <= 64) return 64;
   if (M <= 128) return 128;
   if (M <= 256) return 256;
   return 60 * rounds(128, 128) < 106 * rounds(256, 256) ? 128 : 0;
@@ -797,7 +817,10 @@ static void launch_kmajor(int path, const void* a, const void* bt, void* c, int6
       if (per <= 8) bn = (int)(16 * (per < 4 ? 4 : per));
     }
     const int tiles_n = (int)((N + bn - 1) / bn);
-    if (tileN128_rows(M, N) == 256)
+    if (tileN128_rows(M, N) == 64)
+      hipLaunchKernelGGL((hx_fp8_gemm_tileN128<OUT, 64, true>), dim3((unsigned)tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
+                         (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, 1, bn);
+    else if (tileN128_rows(M, N) == 256)
       hipLaunchKernelGGL((hx_fp8_gemm_tileN128<OUT, 256>), dim3((unsigned)((M + 255) / 256) * tiles_n), dim3(256), 0, stream,
                          (const uint8_t*)a, (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa,
                          sb, (int)((M + 255) / 256), bn);

@@ -27,6 +27,7 @@ def _path(m, n, k):
     (256, 256, 256, 5), (512, 512, 512, 5), (1024, 1024, 1024, 5), (256, 768, 128, 5), (768, 256, 1152, 5),   # too few: 128-column tiles
     (64, 28672, 256, 5), (128, 40000, 128, 5), (90, 20000, 128, 5),      # one row tile: column pitch 112 / 128 / 80
     (48, 1024, 512, 5), (100, 3000, 256, 5), (129, 520, 384, 5), (256, 1000, 128, 5), (200, 136, 1280, 5), (33, 256, 256, 5),
+    (64, 256, 128 * 7, 5), (40, 300, 128 * 12, 5), (96, 264, 128 * 9, 5), (80, 1024, 2048, 5), (128, 512, 128 * 11, 5),  # k-tiles issued in pairs
     (1000, 1000, 1024, 5), (300, 200, 256, 5), (257, 255, 128, 5), (32, 64, 8192 + 128, 5), (255, 1, 128, 5),
     (16, 512, 1024, 2), (1, 16, 128, 2), (5, 48, 256, 2), (16, 1000, 384, 2), (9, 33, 8192 + 128, 2), (16, 64, 16384, 2),
     (17, 256, 256, 2), (32, 512, 8192, 2), (24, 100, 1152, 2), (31, 33, 384, 2),        # two 16-row blocks on the skinny kernel
