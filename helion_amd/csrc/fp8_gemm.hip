@@ -399,12 +399,18 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tileN128(const uint8_t* __res
   // in-order instruction stream up
   constexpr int EVERY = 4 * WMB >= 2 * IPW ? 2 : 1;
   constexpr int PER = (2 * IPW + 4 * WMB - 1) / (4 * WMB);  // PAIR: DMA instructions after each MFMA of an issuing step
+  // PAIR: instructions that may still be outstanding when tile kt+1 must have landed, at even / odd steps.  Pairs go out
+  // at even steps as (kt+NS-1, kt+NS), interleaved, so the tile needed is the first of its pair (the pair's last
+  // instruction is not its own) at even steps for an even NS and at odd steps for an odd NS.
+  constexpr int W_EVEN = NS % 2 == 0 ? IPW * (NS - 4) + 1 : IPW * (NS - 3);
+  constexpr int W_ODD = NS % 2 == 0 ? IPW * (NS - 2) : IPW * (NS - 3) + 1;
   static_assert(4 * WMB >= EVERY * IPW, "every DMA instruction of a k-tile has an MFMA to follow");
   // PAIR: the DMA of two consecutive k-tiles is issued in the same step, at every other step and row piece by row
   // piece, so that memory sees both 128-byte halves of 256 contiguous bytes of a row back to back (a single row tile
   // streams its weights from HBM, and lone 128-byte pieces 8 KB apart cost a DRAM row activation each: 50.5 -> 47.5 us
   // for 33..64 rows against 28672 x 8192 weights).  It needs the six-stage ring of the 64-row tile: with four stages
-  // the wait for the first tile of a pair leaves nothing in flight, and 65..128 rows measured slower paired.
+  // the wait for the first tile of a pair leaves nothing in flight, and 65..128 rows measured slower paired (with five
+  // stages as well).
   auto mma = [&](v8i(&fa)[WMB], v8i(&fb)[4], int dkt, bool two) {
 #pragma unroll
     for (int i = 0; i < 4 * WMB; ++i) {
@@ -424,8 +430,9 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tileN128(const uint8_t* __res
     // this wave's part of tile kt+1 has landed
     // (PAIR, even step: tile kt+1 is the first of its pair, so only the last instruction of that pair, which belongs to
     // the second tile, and the pairs issued since may be outstanding)
-    if (PAIR && even) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(PAIR ? (NS - 4) * IPW + 1 : 0));
-    else __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 2) * IPW));
+    if (!PAIR) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 2) * IPW));
+    else if (even) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(PAIR ? W_EVEN : 0));
+    else __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(PAIR ? W_ODD : 0));
     __syncthreads();             // ... everybody's has, and every wave holds tile kt in registers: its stage is free
     if (kt + 1 < nk) load_frags(na, nb, kt + 1);
     mma(ca, cb, kt + NS, even);
