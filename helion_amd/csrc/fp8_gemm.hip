@@ -327,11 +327,18 @@ __global__ __launch_bounds__(256) void hx_transpose_u8(const uint8_t* __restrict
 // re-read its last column (an L2 hit, no HBM traffic) and are not stored.
 // ------------------------------------------------------------------------------------------
 template <int OUT, int BM, bool PAIR = false>
-__global__ __launch_bounds__(256) void hx_fp8_gemm_tileN128(const uint8_t* __restrict__ A, const uint8_t* __restrict__ Bt,
-                                                           typename OutT<OUT>::T* __restrict__ C, int M, int N, int K, long lda,
+__global__ __launch_bounds__(256) void hx_fp8_gemm_tileN128(const uint8_t* __restrict__ A_, const uint8_t* __restrict__ Bt_,
+                                                           typename OutT<OUT>::T* __restrict__ C_, int M, int N, int K, long lda,
                                                            long ldb, long ldc, const float* __restrict__ scale_a,
-                                                           const float* __restrict__ scale_b, int tiles_m, int bn) {
+                                                           const float* __restrict__ scale_b, int tiles_m, int bn,
+                                                           int kt_per_split) {
   typedef typename OutT<OUT>::T out_t;
+  // split-K (kt_per_split != 0): workgroup row blockIdx.y multiplies k-tiles [kt0, kt0 + nk) into its own M x N slab of C_
+  const int kt0 = kt_per_split * (int)blockIdx.y;
+  const int nk = kt_per_split ? min(kt_per_split, K / T256_BK - kt0) : K / T256_BK;
+  const uint8_t* A = A_ + (long)kt0 * T256_BK;
+  const uint8_t* Bt = Bt_ + (long)kt0 * T256_BK;
+  out_t* C = C_ + (kt_per_split ? (long)blockIdx.y * M * ldc : 0);
   constexpr int NS = BM == 64 ? 6 : BM == 128 ? 4 : 3;   // 144, 128 or 144 KB of LDS
   constexpr int STAGE = (BM + 128) * 128;                // bytes of one stage: A tile, then B tile
   constexpr int WMB = BM / 32;                           // 16-row blocks per wave
@@ -355,7 +362,6 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tileN128(const uint8_t* __res
 #pragma unroll
   for (int jj = 0; jj < 4; ++jj) b_vo[jj] = (uint32_t)min((int)n0 + 8 * (w + 4 * jj) + lrow, nlast) * (uint32_t)ldb + chunk;
   const uint32_t lds0 = hx_lds_addr(&smem[0][0]);
-  const int nk = K / T256_BK;
   // instruction i (0 .. IPW-1) of this wave for k-tile kt; past the end: the last tile again, so that every step
   // issues IPW instructions and the counted waits stay exact
   auto issue_one = [&](int kt, int i) {
@@ -752,6 +758,40 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_general(const uint8_t* __rest
     }
 }
 
+// split-K: C = cast(alpha * sum over the splits' fp32 slabs [split][M][N]); one thread per four columns
+template <int OUT>
+__global__ __launch_bounds__(256) void hx_fp8_gemm_split_reduce(const float* __restrict__ part, typename OutT<OUT>::T* __restrict__ C,
+                                                                int M, int N, long ldc, int splits,
+                                                                const float* __restrict__ scale_a,
+                                                                const float* __restrict__ scale_b) {
+  typedef typename OutT<OUT>::T out_t;
+  const int n4 = (N + 3) >> 2;
+  const long id = (long)blockIdx.x * 256 + threadIdx.x;
+  if (id >= (long)M * n4) return;
+  const int m = (int)(id / n4), n = (int)(id % n4) * 4;
+  float alpha = 1.f;
+  if (scale_a) alpha = *scale_a;
+  if (scale_b) alpha = alpha * *scale_b;
+  const float* p = part + (long)m * N + n;
+  const long slab = (long)M * N;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  if ((N & 3) == 0) {
+    for (int sp = 0; sp < splits; ++sp) {
+      const v4f v = *(const v4f*)(p + sp * slab);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[r] += v[r];
+    }
+  } else {
+    for (int sp = 0; sp < splits; ++sp)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (n + r < N) acc[r] += p[sp * slab + r];
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+    if (n + r < N) C[(long)m * ldc + n + r] = (out_t)(acc[r] * alpha);
+}
+
 // ------------------------------------------------------------------------------------------
 // host dispatch
 // ------------------------------------------------------------------------------------------
@@ -768,6 +808,32 @@ static int tileN128_rows(int64_t M, int64_t N) {
   if (M <= 128) return 128;
   if (M <= 256) return 256;
   return 60 * rounds(128, 128) < 106 * rounds(256, 256) ? 128 : 0;
+}
+
+// column pitch of the 128-column tiles: 128, except that a single row tile of at most 128 rows (a decode batch) gets
+// about one column tile per CU (with a 256-row tile the MFMA work on the unused columns costs more than the idle CUs)
+static int tileN128_pitch(int64_t M, int64_t N) {
+  if (M > 128) return 128;
+  const int64_t blocks = (N + 15) / 16, per = (blocks + 255) / 256;  // 16-column blocks per tile for <= 256 tiles
+  return per <= 8 ? (int)(16 * (per < 4 ? 4 : per)) : 128;
+}
+
+// split-K for the 128-column tiles: when the tiles occupy less than half of the CUs and K is long, each tile's k range
+// is cut into `splits` pieces of *kt_per_split k-tiles (at least 8 each), one workgroup per piece, fp32 partial sums
+// in the workspace.  Returns 1 when it does not pay; the partial sums are capped at 32 MB.
+static int tileN128_splits(int64_t M, int64_t N, int64_t K, int* kt_per_split) {
+  *kt_per_split = 0;
+  const int bm = tileN128_rows(M, N);
+  if (bm == 0 || K % T256_BK != 0 || M <= 16 || (M <= 32 && K <= 8192)) return 1;  // other kernels take those
+  const int bn = tileN128_pitch(M, N);
+  const int64_t tiles = ((M + bm - 1) / bm) * ((N + bn - 1) / bn), nk = K / T256_BK;
+  int64_t s = 256 / tiles;
+  if (s > nk / 8) s = nk / 8;
+  while (s > 1 && s * M * N * 4 > (32LL << 20)) --s;
+  if (s < 2) return 1;
+  const int64_t per = (nk + s - 1) / s;
+  *kt_per_split = (int)per;
+  return (int)((nk + per - 1) / per);
 }
 
 // 0 general, 1 tile256, 2 skinny, 3 tile256 with edge tiles (M or N not a multiple of 256, K not of 128),
@@ -803,7 +869,7 @@ extern "C" int hx_fp8_gemm_path(int64_t M, int64_t N, int64_t K, int64_t lda, in
 
 template <int OUT>
 static void launch_kmajor(int path, const void* a, const void* bt, void* c, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
-                          int64_t ldc, const float* sa, const float* sb, hipStream_t stream) {
+                          int64_t ldc, const float* sa, const float* sb, void* ws, size_t ws_bytes, hipStream_t stream) {
   typedef typename OutT<OUT>::T out_t;
   if (path == 4) {  // row-major B; ldb is its row stride
     const int tiles_m = (int)((M + 255) / 256), tiles_n = (int)((N + 255) / 256);
@@ -817,24 +883,38 @@ static void launch_kmajor(int path, const void* a, const void* bt, void* c, int6
                          (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m,
                          tiles_n);
   } else if (path == 5) {
-    // column pitch of the tiles: 128, except that a single row tile (a decode batch) gets about one column tile per CU
-    int bn = 128;
-    if (M <= 128) {  // (with a 256-row tile the MFMA work on the unused columns costs more than the idle CUs)
-      const int64_t blocks = (N + 15) / 16, per = (blocks + 255) / 256;  // 16-column blocks per tile for <= 256 tiles
-      if (per <= 8) bn = (int)(16 * (per < 4 ? 4 : per));
+    const int bm = tileN128_rows(M, N), bn = tileN128_pitch(M, N);
+    const int tiles_m = (int)((M + bm - 1) / bm), tiles_n = (int)((N + bn - 1) / bn);
+    int ktps = 0;
+    const int splits = tileN128_splits(M, N, K, &ktps);
+    const bool split = splits > 1 && ws && aligned(ws, 16) && ws_bytes >= (size_t)splits * M * N * 4;
+    if (!split) ktps = 0;
+    const dim3 grid((unsigned)(tiles_m * tiles_n), split ? splits : 1);
+    // split-K launches write unscaled fp32 slabs into the workspace; hx_fp8_gemm_split_reduce sums, scales and casts them
+    if (split) {
+      float* part = (float*)ws;
+      if (bm == 64)
+        hipLaunchKernelGGL((hx_fp8_gemm_tileN128<HX_F32, 64, true>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
+                           part, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)N, nullptr, nullptr, tiles_m, bn, ktps);
+      else if (bm == 256)
+        hipLaunchKernelGGL((hx_fp8_gemm_tileN128<HX_F32, 256>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt, part,
+                           (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)N, nullptr, nullptr, tiles_m, bn, ktps);
+      else
+        hipLaunchKernelGGL((hx_fp8_gemm_tileN128<HX_F32, 128>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt, part,
+                           (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)N, nullptr, nullptr, tiles_m, bn, ktps);
+      const long quads = (long)M * ((N + 3) / 4);
+      hipLaunchKernelGGL((hx_fp8_gemm_split_reduce<OUT>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream,
+                         (const float*)part, (out_t*)c, (int)M, (int)N, (long)ldc, splits, sa, sb);
+    } else if (bm == 64) {
+      hipLaunchKernelGGL((hx_fp8_gemm_tileN128<OUT, 64, true>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
+                         (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m, bn, 0);
+    } else if (bm == 256) {
+      hipLaunchKernelGGL((hx_fp8_gemm_tileN128<OUT, 256>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
+                         (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m, bn, 0);
+    } else {
+      hipLaunchKernelGGL((hx_fp8_gemm_tileN128<OUT, 128>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
+                         (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m, bn, 0);
     }
-    const int tiles_n = (int)((N + bn - 1) / bn);
-    if (tileN128_rows(M, N) == 64)
-      hipLaunchKernelGGL((hx_fp8_gemm_tileN128<OUT, 64, true>), dim3((unsigned)tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
-                         (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, 1, bn);
-    else if (tileN128_rows(M, N) == 256)
-      hipLaunchKernelGGL((hx_fp8_gemm_tileN128<OUT, 256>), dim3((unsigned)((M + 255) / 256) * tiles_n), dim3(256), 0, stream,
-                         (const uint8_t*)a, (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa,
-                         sb, (int)((M + 255) / 256), bn);
-    else
-      hipLaunchKernelGGL((hx_fp8_gemm_tileN128<OUT, 128>), dim3((unsigned)((M + 127) / 128) * tiles_n), dim3(256), 0, stream,
-                         (const uint8_t*)a, (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa,
-                         sb, (int)((M + 127) / 128), bn);
   } else if (path == 1 || path == 3) {
     const int tiles_m = (int)((M + 255) / 256), tiles_n = (int)((N + 255) / 256);
     if (path == 1)
@@ -876,7 +956,7 @@ static int launch_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int
   typedef typename OutT<OUT>::T out_t;
   int path = hx_fp8_gemm_path(M, N, K, lda, ldb_k, ldb_n, ldc, a, b, c);
   if (path != 0) {
-    launch_kmajor<OUT>(path, a, b, c, M, N, K, lda, path == 4 ? ldb_k : ldb_n, ldc, sa, sb, stream);
+    launch_kmajor<OUT>(path, a, b, c, M, N, K, lda, path == 4 ? ldb_k : ldb_n, ldc, sa, sb, ws, ws_bytes, stream);
   } else {
     // row-major B with a workspace: transpose it once into K-contiguous form, then take a fast path
     int tpath = 0;
@@ -885,7 +965,7 @@ static int launch_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int
     if (tpath != 0) {
       dim3 tg((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64));
       hipLaunchKernelGGL(hx_transpose_u8, tg, dim3(256), 0, stream, (const uint8_t*)b, (uint8_t*)ws, (int)K, (int)N, (long)ldb_k);
-      launch_kmajor<OUT>(tpath, a, ws, c, M, N, K, lda, K, ldc, sa, sb, stream);
+      launch_kmajor<OUT>(tpath, a, ws, c, M, N, K, lda, K, ldc, sa, sb, nullptr, 0, stream);
     } else {
       dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
       hipLaunchKernelGGL(hx_fp8_gemm_general<OUT>, grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)b, (out_t*)c,
@@ -901,10 +981,16 @@ static int launch_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int
 }
 
 extern "C" size_t hx_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t ldb_k, int64_t ldb_n) {
-  // Only a row-major B (N contiguous) that the tile kernel cannot read in place (M <= 16: the skinny kernel wants K
+  // A row-major B (N contiguous) that the tile kernel cannot read in place (M <= 16: the skinny kernel wants K
   // contiguous; N or the row stride not a multiple of 16) but that could take a fast path after a transpose needs
-  // scratch: N*K bytes.
-  if (M <= 0 || N <= 0 || K <= 0 || ldb_k == 1 || ldb_n != 1 || K % 16 != 0) return 0;
+  // N*K bytes of scratch; a column-major B needs scratch only for split-K partial sums.
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  if (ldb_k == 1) {  // column-major B: fp32 partial sums when the 128-column tile kernel would split K
+    int ktps = 0;
+    const int splits = tileN128_splits(M, N, K, &ktps);
+    return splits > 1 ? (size_t)splits * M * N * 4 : 0;
+  }
+  if (ldb_n != 1 || K % 16 != 0) return 0;
   if (M > 16 && N % 16 == 0 && ldb_k % 16 == 0) return 0;
   return (size_t)(N * K);
 }

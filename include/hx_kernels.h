@@ -58,9 +58,11 @@ const char* hx_last_error(void);
 int hx_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int64_t lda,
                 int64_t ldb_k, int64_t ldb_n, int64_t ldc, const float* scale_a, const float* scale_b,
                 int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
-/* Scratch hx_fp8_gemm can use for these arguments: 0 unless B is row-major AND the tile kernel cannot read it in
- * place (M <= 16, or N / the row stride not a multiple of 16); then N*K bytes for a one-off transpose into the
- * K-contiguous layout, without which such a B runs on the slow general kernel. */
+/* Scratch hx_fp8_gemm can use for these arguments.  Row-major B that the tile kernel cannot read in place (M <= 16,
+ * or N / the row stride not a multiple of 16): N*K bytes for a one-off transpose into the K-contiguous layout,
+ * without which such a B runs on the slow general kernel.  Column-major B: splits*M*N*4 bytes when the 128-column
+ * tile kernel would cut K into `splits` pieces (its tiles occupy less than half of the CUs and K is at least 16
+ * k-tiles long; at most 32 MB), without which it runs unsplit.  0 otherwise. */
 size_t hx_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t ldb_k, int64_t ldb_n);
 
 /* Which kernel hx_fp8_gemm would launch for these arguments: 0 general (or, given a workspace, transpose + fast

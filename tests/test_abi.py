@@ -60,6 +60,14 @@ def test_gemm_path_selection():
     assert lib.hx_fp8_gemm_workspace_bytes(256, 512, 384, 512, 1) == 0          # row-major B the tile kernel reads in place
     assert lib.hx_fp8_gemm_workspace_bytes(8, 512, 384, 512, 1) == 512 * 384    # skinny shape: transpose scratch
     assert lib.hx_fp8_gemm_workspace_bytes(256, 512, 384, 1, 384) == 0
+    # column-major B: split-K partial sums only for few 128-column tiles and a long K, never for the skinny shapes
+    assert lib.hx_fp8_gemm_workspace_bytes(1024, 1280, 8192, 1, 8192) == 3 * 1024 * 1280 * 4
+    assert lib.hx_fp8_gemm_workspace_bytes(64, 2048, 8192, 1, 8192) == 8 * 64 * 2048 * 4
+    assert lib.hx_fp8_gemm_workspace_bytes(1024, 1024, 1024, 1, 1024) == 0
+    assert lib.hx_fp8_gemm_workspace_bytes(8192, 8192, 8192, 1, 8192) == 0
+    assert lib.hx_fp8_gemm_workspace_bytes(16, 2048, 8192, 1, 8192) == 0
+    assert lib.hx_fp8_gemm_workspace_bytes(64, 28672, 8192, 1, 8192) == 0
+    assert lib.hx_fp8_gemm_workspace_bytes(300, 520, 2048 + 16, 1, 2064) == 0   # K % 128 != 0: the edge kernel, no split
     assert lib.hx_fp8_gemm_path(256, 256, 256, 256, 1, 256, 256, A + 1, A, A) == 0  # misaligned
 
 

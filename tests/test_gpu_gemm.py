@@ -98,6 +98,35 @@ def test_reference_call_form_and_defaults():
         assert torch.equal(hx.fp8_gemm_tritonbench(x.to(DEV), y.to(DEV)), out)
 
 
+@pytest.mark.parametrize("m,n,k", [
+    (300, 520, 2048),      # 128-row tiles, two splits
+    (64, 2050, 2048),      # one 64-row tile, N % 4 != 0: scalar partial stores and reduce
+    (33, 256, 128 * 17),   # 17 k-tiles in pieces of 9 and 8
+    (200, 136, 4096),      # one 256-row tile
+    (1024, 1280, 8192),    # three splits of 22, 22, 20 k-tiles
+])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_split_k_few_tiles_long_k(m, n, k, out_dtype):
+    """Few 128-column tiles and a long K: the op hands over the workspace that hx_fp8_gemm_workspace_bytes asks for
+    and the kernel splits K (fp32 partial sums + reduce); without a workspace the same call runs unsplit."""
+    lib = _lib.load()
+    assert _path(m, n, k) == 5
+    ws_bytes = lib.hx_fp8_gemm_workspace_bytes(m, n, k, 1, k)
+    assert ws_bytes >= 2 * m * n * 4 and ws_bytes % (m * n * 4) == 0
+    a, b, sa, sb = inputs.gemm_scaled(m, n, k, seed=m + n + k)
+    ad, bd, sad, sbd = a.to(DEV), b.to(DEV), sa.to(DEV), sb.to(DEV)
+    ref = orc.fp8_gemm(a, b, sa, sb, out_dtype)
+    tol = 1e-2 if out_dtype != torch.float32 else 1e-4
+    out = hx.fp8_gemm(ad, bd, scale_a=sad, scale_b=sbd, out_dtype=out_dtype)
+    assert rel_err(out, ref) <= tol
+    unsplit = torch.empty_like(out)
+    rc = lib.hx_fp8_gemm(ad.data_ptr(), bd.data_ptr(), unsplit.data_ptr(), m, n, k, k, 1, k, n, sad.data_ptr(), sbd.data_ptr(),
+                         _lib.HX_BF16 if out_dtype == torch.bfloat16 else _lib.HX_F32, None, 0,
+                         torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, lib.hx_last_error()
+    assert rel_err(unsplit, ref) <= tol
+
+
 def test_golden_fixture():
     z = np.load(G / "fp8_gemm_small.npz")
     for name in ("ragged", "skinny"):
