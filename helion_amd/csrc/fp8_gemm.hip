@@ -345,7 +345,18 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tileN128(const uint8_t* __res
   constexpr int AJ = BM / 32, IPW = AJ + 4;              // DMA instructions per wave per k-tile: A, B
   __shared__ __attribute__((aligned(1024))) uint8_t smem[NS][STAGE];
 
-  const int tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m;
+  // Grouped raster, GM row tiles tall; every 256 consecutive tiles of that order are spread over the XCDs (workgroup i
+  // runs on XCD i % 8) in blocks of 32, so the tiles resident on one XCD share A and B panels in its L2.
+  int tm, tn;
+  {
+    const int nwg = gridDim.x, wg = blockIdx.x, chunk = wg >> 8, tiles_n = nwg / tiles_m;
+    const int tile = chunk < (nwg >> 8) ? (chunk << 8) + ((wg & 7) << 5) + ((wg >> 3) & 31) : wg;
+    constexpr int GM = 8;
+    const int group_size = GM * tiles_n, first_m = (tile / group_size) * GM;
+    const int gm = min(tiles_m - first_m, GM);
+    tm = first_m + (tile % group_size) % gm;
+    tn = (tile % group_size) / gm;
+  }
   const long m0 = (long)tm * BM, n0 = (long)tn * bn;
   const int nlast = (int)min(n0 + bn, (long)N) - 1;  // last column this tile owns
   const int tid = threadIdx.x, lane = tid & 63;
@@ -381,18 +392,17 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tileN128(const uint8_t* __res
   const int x16 = ((2 * kq) ^ ((r16 >> 1) & 7)) * 16;
   const int a_base = (wm * (BM / 2) + r16) * 128;
   const int b_base = BM * 128 + (wn * 64 + r16) * 128;
-  auto load_frags = [&](v8i(&fa)[WMB], v8i(&fb)[4], int kt) {
-    const uint8_t* st = &smem[kt % NS][0];
-#pragma unroll
-    for (int f = 0; f < WMB; ++f) {
-      const v4i lo = *(const v4i*)(st + a_base + f * 2048 + x16), hi = *(const v4i*)(st + a_base + f * 2048 + (x16 ^ 16));
-      fa[f] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-    }
-#pragma unroll
-    for (int f = 0; f < 4; ++f) {
-      const v4i lo = *(const v4i*)(st + b_base + f * 2048 + x16), hi = *(const v4i*)(st + b_base + f * 2048 + (x16 ^ 16));
-      fb[f] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-    }
+  // One set of fragments per wave, refilled in place: fragment f of A (of B) takes tile kt's rows a_base + 16 f ...
+  v8i fa[WMB], fb[4];
+  auto load_a = [&](int f, int kt) {
+    const uint8_t* st = &smem[kt % NS][0] + a_base + f * 2048;
+    const v4i lo = *(const v4i*)(st + x16), hi = *(const v4i*)(st + (x16 ^ 16));
+    fa[f] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+  };
+  auto load_b = [&](int f, int kt) {
+    const uint8_t* st = &smem[kt % NS][0] + b_base + f * 2048;
+    const v4i lo = *(const v4i*)(st + x16), hi = *(const v4i*)(st + (x16 ^ 16));
+    fb[f] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   };
   // acc[bj][bi][r] is C[m0 + wm*BM/2 + 16 bi + lane%16][n0 + wn*64 + 16 bj + 4*(lane/16) + r]
   v4f acc[4][WMB];
@@ -417,43 +427,45 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tileN128(const uint8_t* __res
   // for 33..64 rows against 28672 x 8192 weights).  It needs the six-stage ring of the 64-row tile: with four stages
   // the wait for the first tile of a pair leaves nothing in flight, and 65..128 rows measured slower paired (with five
   // stages as well).
-  auto mma = [&](v8i(&fa)[WMB], v8i(&fb)[4], int dkt, bool two) {
-#pragma unroll
-    for (int i = 0; i < 4 * WMB; ++i) {
-      acc[i & 3][i >> 2] = hx_mfma_16x16x128_e4m3(fb[i & 3], fa[i >> 2], acc[i & 3][i >> 2]);
-      if (!PAIR) {
-        if (i % EVERY == EVERY - 1 && i / EVERY < IPW) issue_one(dkt, i / EVERY);
-      } else if (two) {  // row piece by row piece: (dkt-1, 0), (dkt, 0), (dkt-1, 1), ...; the counted waits rely on that order
-#pragma unroll
-        for (int q = PER * i; q < PER * (i + 1) && q < 2 * IPW; ++q) issue_one((q & 1) ? dkt : dkt - 1, q >> 1);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  };
-  // step kt: tile kt is in `cur`; tiles kt+1 .. are landed or in flight.  Without PAIR every step issues tile kt+NS;
-  // with it the even steps issue tiles kt+NS-1 and kt+NS (the stages of tiles kt-1 and kt) and the odd steps none.
-  auto step = [&](v8i(&ca)[WMB], v8i(&cb)[4], v8i(&na)[WMB], v8i(&nb)[4], int kt, bool even) {
+  // step kt: the fragments hold tile kt; tiles kt+1 .. are landed or in flight.  The MFMAs run A row block by row
+  // block; a fragment is refilled with tile kt+1's as soon as its last MFMA of this tile has been issued (A fragment
+  // bi after the four MFMAs of its row block, the B fragments during the last row block), so there is no second
+  // register set and every step is the same code.  Past the last tile the refills read the ring's copy of the last
+  // tile again.  Without PAIR every step issues the DMA of tile kt+NS; with it the even steps issue tiles kt+NS-1 and
+  // kt+NS (the stages of tiles kt-1 and kt) and the odd steps none.
+  auto step = [&](int kt, bool even) {
     // this wave's part of tile kt+1 has landed
     // (PAIR, even step: tile kt+1 is the first of its pair, so only the last instruction of that pair, which belongs to
     // the second tile, and the pairs issued since may be outstanding)
     if (!PAIR) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 2) * IPW));
     else if (even) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(PAIR ? W_EVEN : 0));
     else __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(PAIR ? W_ODD : 0));
-    __syncthreads();             // ... everybody's has, and every wave holds tile kt in registers: its stage is free
-    if (kt + 1 < nk) load_frags(na, nb, kt + 1);
-    mma(ca, cb, kt + NS, even);
+    __syncthreads();  // ... everybody's has, and every wave has read tile kt out of its stage: that stage is free
+    const int dkt = kt + NS;
+#pragma unroll
+    for (int i = 0; i < 4 * WMB; ++i) {
+      const int bj = i & 3, bi = i >> 2;
+      acc[bj][bi] = hx_mfma_16x16x128_e4m3(fb[bj], fa[bi], acc[bj][bi]);
+      if (!PAIR) {
+        if (i % EVERY == EVERY - 1 && i / EVERY < IPW) issue_one(dkt, i / EVERY);
+      } else if (even) {  // row piece by row piece: (dkt-1, 0), (dkt, 0), (dkt-1, 1), ...; the counted waits rely on that order
+#pragma unroll
+        for (int q = PER * i; q < PER * (i + 1) && q < 2 * IPW; ++q) issue_one((q & 1) ? dkt : dkt - 1, q >> 1);
+      }
+      if (bj == 3) load_a(bi, kt + 1);
+      if (bi == WMB - 1) load_b(bj, kt + 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   };
   for (int t = 0; t < (PAIR ? NS - 1 : NS); ++t) issue(t);
   __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((PAIR ? NS - 2 : NS - 1) * IPW));
   __syncthreads();
-  v8i fa0[WMB], fb0[4], fa1[WMB], fb1[4];
-  load_frags(fa0, fb0, 0);
-  int kt = 0;
-  for (; kt + 1 < nk; kt += 2) {
-    step(fa0, fb0, fa1, fb1, kt, true);
-    step(fa1, fb1, fa0, fb0, kt + 1, false);
-  }
-  if (kt < nk) step(fa0, fb0, fa1, fb1, kt, true);
+#pragma unroll
+  for (int f = 0; f < WMB; ++f) load_a(f, 0);
+#pragma unroll
+  for (int f = 0; f < 4; ++f) load_b(f, 0);
+  // (one loop body for both kinds of step: with two copies of it the compiler shuffles the accumulators between them)
+  for (int kt = 0; kt < nk; ++kt) step(kt, (kt & 1) == 0);
   HX_WAIT_VM0();  // no DMA may still be writing this workgroup's LDS when it ends
 
   float alpha = 1.f;
@@ -798,16 +810,18 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_split_reduce(const float* __r
 static inline bool aligned(const void* p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
 // Which tile for a K-contiguous problem: 256x256 (returns 0) or 128 columns wide (returns the tile's rows: one row tile
-// of 128 or 256 rows for a decode batch that streams weights from HBM, 128 otherwise).  Both kernels run one workgroup
-// per CU, so a launch takes ceil(tiles / 256) rounds of K / 128 k-tile steps; per step the 128x128 tile costs about 0.6
-// of the 256x256 tile's when fed from L2 (measured: it is bound by what a CU can pull from L2, not by the MFMAs).  A
+// of 64, 128 or 256 rows for a decode batch that streams weights from HBM, 128 otherwise).  Both kernels run one
+// workgroup per CU, so a launch takes ceil(tiles / 256) rounds, each of K / 128 k-tile steps plus a prologue and an
+// epilogue.  Measured with every CU busy: a 256x256 step 1.37 us and about 6 us per round outside the loop, a 128x128
+// step 0.5 us (it is bound by what the CUs can pull out of the L2s, not by its MFMAs) and about 3 us per round.  A
 // 256x128 tile for more than 256 rows measured no better than either.
-static int tileN128_rows(int64_t M, int64_t N) {
+static int tileN128_rows(int64_t M, int64_t N, int64_t K) {
   auto rounds = [&](int64_t bm, int64_t bn) { return (((M + bm - 1) / bm) * ((N + bn - 1) / bn) + 255) / 256; };
   if (M <= 64) return 64;
   if (M <= 128) return 128;
   if (M <= 256) return 256;
-  return 60 * rounds(128, 128) < 106 * rounds(256, 256) ? 128 : 0;
+  const int64_t nk = (K + T256_BK - 1) / T256_BK;
+  return rounds(128, 128) * (50 * nk + 300) < rounds(256, 256) * (137 * nk + 600) ? 128 : 0;
 }
 
 // column pitch of the 128-column tiles: 128, except that a single row tile of at most 128 rows (a decode batch) gets
@@ -823,7 +837,7 @@ static int tileN128_pitch(int64_t M, int64_t N) {
 // in the workspace.  Returns 1 when it does not pay; the partial sums are capped at 32 MB.
 static int tileN128_splits(int64_t M, int64_t N, int64_t K, int* kt_per_split) {
   *kt_per_split = 0;
-  const int bm = tileN128_rows(M, N);
+  const int bm = tileN128_rows(M, N, K);
   if (bm == 0 || K % T256_BK != 0 || M <= 16 || (M <= 32 && K <= 8192)) return 1;  // other kernels take those
   const int bn = tileN128_pitch(M, N);
   const int64_t tiles = ((M + bm - 1) / bm) * ((N + bn - 1) / bn), nk = K / T256_BK;
@@ -845,10 +859,8 @@ static int gemm_path_kmajor(int64_t M, int64_t N, int64_t K, int64_t lda, int64_
   const bool ktail = K % 128 != 0;  // only the edge instantiation of the tile kernel pads a partial last k-tile
   if (!ktail && (M <= 16 || (M <= 32 && K <= 8192)) && lda >= K && ldb >= K) return 2;
   if (lda >= (1LL << 27) || ldb >= (1LL << 27)) return 0;
-  // 128-column tiles or 256x256 tiles?  Both run one workgroup per CU, so a launch takes ceil(tiles / 256) rounds of K / 128
-  // k-tile steps; a step of the small tile costs about 0.6 of a step of the large one when it is fed from L2 (measured),
-  // and far less when a single row tile streams weights from HBM.
-  if (!ktail && M * lda < (1LL << 32) && N * ldb < (1LL << 32) && tileN128_rows(M, N) != 0) return 5;
+  // 128-column tiles or 256x256 tiles: whichever tileN128_rows estimates to finish first
+  if (!ktail && M * lda < (1LL << 32) && N * ldb < (1LL << 32) && tileN128_rows(M, N, K) != 0) return 5;
   if (!ktail && (M % 256 == 0) && (N % 256 == 0) && (ldc % 8 == 0) && aligned(c, 16)) return 1;  // 16-byte row-aligned stores
   if (M * lda < (1LL << 32) && N * ldb < (1LL << 32)) return 3;
   return 0;
@@ -883,7 +895,7 @@ static void launch_kmajor(int path, const void* a, const void* bt, void* c, int6
                          (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m,
                          tiles_n);
   } else if (path == 5) {
-    const int bm = tileN128_rows(M, N), bn = tileN128_pitch(M, N);
+    const int bm = tileN128_rows(M, N, K), bn = tileN128_pitch(M, N);
     const int tiles_m = (int)((M + bm - 1) / bm), tiles_n = (int)((N + bn - 1) / bn);
     int ktps = 0;
     const int splits = tileN128_splits(M, N, K, &ktps);
