@@ -12,10 +12,10 @@
 //                                transposing read has 32 lanes fetch 4 consecutive k rows x 64 contiguous bytes, and
 //                                the xor puts the four rows into different 64-byte quarters of the bank window.
 //   W tile, column-major W     : [128 columns][128 B], exactly like the A tile.
-// The fragments of a whole k-tile (4 k-steps) are read into registers at once, one k-tile ahead of the MFMAs that use
-// them, so the LDS stage of a tile is free for the DMA of tile kt+NS as soon as every wave has passed the barrier of
-// tile kt; two register sets alternate.  Past the last k-tile the DMA fetches the last tile again, so every step
-// issues the same number of instructions and the counted waits stay exact.
+// The fragments of a whole k-tile (4 k-steps) live in registers and are refilled in place with the next tile's, k-step
+// by k-step, right behind the MFMAs that used them, so the LDS stage of a tile is free for the DMA of tile kt+NS as soon
+// as every wave has passed the barrier of tile kt.  Past the last k-tile the DMA fetches the last tile again, so every
+// step issues the same number of instructions and the counted waits stay exact.
 #pragma once
 #include "gemm16_tile256.h"
 
@@ -24,7 +24,7 @@
 #define G128_TILE_BYTES (128 * 128)
 
 template <bool BF, int MODE, bool BCOL = false, int NS = 2>
-__global__ __launch_bounds__(256, NS == 2 ? 2 : 1) void hx_gemm16_tile128(const uint8_t* __restrict__ A, const uint8_t* __restrict__ W,
+__global__ __launch_bounds__(256, 2) void hx_gemm16_tile128(const uint8_t* __restrict__ A, const uint8_t* __restrict__ W,
                                                            void* __restrict__ Cv, const int* __restrict__ num_tiles,
                                                            const MoeTile* __restrict__ table, const int32_t* __restrict__ idx, int T,
                                                            int K, int N, int max_tiles, int tiles_n, int a_div, G16Dense d) {
@@ -135,56 +135,51 @@ __global__ __launch_bounds__(256, NS == 2 ? 2 : 1) void hx_gemm16_tile128(const 
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  auto load_frags = [&](V8(&af)[4][2], V8(&wf)[4][2], int stage) {
+  // One set of fragments per wave (4 k-steps x (2 A + 2 W)), refilled in place: the four fragments of k-step ks take
+  // tile kt+1's as soon as the four MFMAs of k-step ks of tile kt have been issued, twelve MFMAs before their next use.
+  V8 af[4][2], wf[4][2];
+  auto load_ks = [&](int ks, int stage) {
     const uint8_t* sa = &smem[stage][0][0];
     const uint8_t* sw = &smem[stage][1][0];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
+    for (int bi = 0; bi < 2; ++bi) af[ks][bi] = *(const V8*)(sa + a_base + bi * 4096 + (ax ^ (ks * 32)));
 #pragma unroll
-      for (int bi = 0; bi < 2; ++bi) af[ks][bi] = *(const V8*)(sa + a_base + bi * 4096 + (ax ^ (ks * 32)));
+    for (int bj = 0; bj < 2; ++bj) {
+      if (BCOL) {
+        wf[ks][bj] = *(const V8*)(sw + (wn * 64 + r31) * 128 + bj * 4096 + (ax ^ (ks * 32)));
+      } else {
+        v4s part[2];
 #pragma unroll
-      for (int bj = 0; bj < 2; ++bj) {
-        if (BCOL) {
-          wf[ks][bj] = *(const V8*)(sw + (wn * 64 + r31) * 128 + bj * 4096 + (ax ^ (ks * 32)));
-        } else {
-          v4s part[2];
-#pragma unroll
-          for (int half = 0; half < 2; ++half)
-            part[half] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (v4s __attribute__((address_space(3)))*)(sw + ((w_off[half] ^ (bj * 64)) + ks * 4096)));
-          v8s both = (v8s){part[0][0], part[0][1], part[0][2], part[0][3], part[1][0], part[1][1], part[1][2], part[1][3]};
-          wf[ks][bj] = __builtin_bit_cast(V8, both);
-        }
+        for (int half = 0; half < 2; ++half)
+          part[half] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (v4s __attribute__((address_space(3)))*)(sw + ((w_off[half] ^ (bj * 64)) + ks * 4096)));
+        v8s both = (v8s){part[0][0], part[0][1], part[0][2], part[0][3], part[1][0], part[1][1], part[1][2], part[1][3]};
+        wf[ks][bj] = __builtin_bit_cast(V8, both);
       }
     }
   };
-  auto mma = [&](V8(&af)[4][2], V8(&wf)[4][2]) {
+  // one k-tile: the fragments hold tile kt; tile kt+1 has landed (the refills read it), later ones are in flight.  Every
+  // step is the same code (a second register set, alternating, had the compiler shuffle the accumulators between
+  // the two copies of the loop body).  Past the last k-tile the refills read the ring's copy of the last tile again.
+  auto ktile = [&](int kt) {
+    __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 2) * 8));  // this wave's part of tile kt+1 has landed
+    __syncthreads();  // ... everybody's has, and every wave has read tile kt out of its stage: that stage is free
+    issue(kt + NS);
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks)
+    for (int ks = 0; ks < 4; ++ks) {
 #pragma unroll
       for (int bj = 0; bj < 2; ++bj)
 #pragma unroll
         for (int bi = 0; bi < 2; ++bi) acc[bj][bi] = Mfma16<BF>::run(wf[ks][bj], af[ks][bi], acc[bj][bi]);
+      load_ks(ks, (kt + 1) % NS);
+    }
   };
-  // one k-tile: `cur` holds tile kt; tile kt+1 is in flight into the other stage
-  auto ktile = [&](V8(&ca)[4][2], V8(&cw)[4][2], V8(&na)[4][2], V8(&nw)[4][2], int kt) {
-    __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 2) * 8));  // this wave's part of tile kt+1 has landed
-    __syncthreads();  // ... everybody's has, and every wave holds tile kt in registers: its stage is free
-    issue(kt + NS);
-    if (kt + 1 < nk) load_frags(na, nw, (kt + 1) % NS);
-    mma(ca, cw);
-  };
-  V8 fa0[4][2], fw0[4][2], fa1[4][2], fw1[4][2];
   for (int t = 0; t < NS; ++t) issue(t);
   __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 1) * 8));
   __syncthreads();
-  load_frags(fa0, fw0, 0);
-  int kt = 0;
-  for (; kt + 1 < nk; kt += 2) {
-    ktile(fa0, fw0, fa1, fw1, kt);
-    ktile(fa1, fw1, fa0, fw0, kt + 1);
-  }
-  if (kt < nk) ktile(fa0, fw0, fa1, fw1, kt);
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) load_ks(ks, 0);
+  for (int kt = 0; kt < nk; ++kt) ktile(kt);
   HX_WAIT_VM0();  // no DMA may still be writing this workgroup's LDS when it ends
 
   // ---- epilogue: acc[bj][bi][4a+b] is C[row_of(wm*64 + bi*32 + lane%32)][n0 + wn*64 + bj*32 + 8a + 4g + b].
