@@ -186,7 +186,7 @@ def bench_next_rows(steps, warmup):
         return hx.fp8_gemm(xa, bufs[turn[0]], out_dtype=torch.bfloat16)
 
     ms, _ = _time_launches(decode64, n_it, n_w)
-    out["decode_gemm_m64"] = hbm(28672 * 8192 + 64 * 8192 + 2 * 64 * 28672, ms, "hx_fp8_gemm_tileN128<bf16, 128>",
+    out["decode_gemm_m64"] = hbm(28672 * 8192 + 64 * 8192 + 2 * 64 * 28672, ms, "hx_fp8_gemm_tileN128<bf16, 64 rows, paired DMA>",
                                  "fp8_gemm M64 N28672 K8192 bf16 out, 4 rotating weight buffers (HBM-cold)")
     del bufs, xa
     # routing tables at the C5 row count and at 1M rows
