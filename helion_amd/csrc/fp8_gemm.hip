@@ -207,7 +207,9 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
       __builtin_amdgcn_sched_barrier(0);
     }
     HX_WAIT_VM0();
-    if (has_tail && kt == nk - 2) zero_tail(stage ^ 1);  // the last tile has just landed in the other stage
+    // the last tile has just landed in the other stage.  (Only in the copy of the loop that runs the last two tiles:
+    // with this branch in the main loop the compiler moves the accumulators around it, one move per MFMA.)
+    if (!dma && has_tail && kt == nk - 2) zero_tail(stage ^ 1);
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
