@@ -237,7 +237,6 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restri
   HX_WAIT_VM0();  // trailing re-fetches must land before the workgroup's LDS is released
 
   // ---- epilogue: acc[bj][bi][4a+b] is C[row_of(wm*128 + bi*32 + lane%32)][n0 + wn*128 + bj*32 + 8a + 4g + b].
-  // N % 8 == 0 and a piece starts at a multiple of 4: it is either wholly inside the row or wholly outside.
   const long ncol = n0 + wn * 128 + 4 * g;
   if (MODE == 2) {
     float* Cp = (float*)Cv + (long)blockIdx.y * T * d.ldc;
@@ -255,36 +254,47 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restri
     }
     return;
   }
+  // A lane holds 4 consecutive columns of a row, so direct stores would hit every 128-byte line of C with sixteen
+  // separate 8-byte writes, and the write burst at the end of a round of tiles becomes L2-transaction-bound.  Each wave
+  // instead passes 32 rows x 128 columns at a time through its own quarter of the (now idle) LDS and writes whole
+  // 256-byte row pieces: 16 bytes per lane, consecutive lanes on consecutive bytes.  The matrix rows of the wave's
+  // 128 tile rows (gathered in the grouped mode) go through the LDS as well.
   out_t* C = (out_t*)Cv;
   typedef out_t ov4 __attribute__((ext_vector_type(4)));
-  int rr[4];  // matrix row of each of this lane's four tile rows, -1: not stored
+  __syncthreads();  // every wave is past its last fragment read: the LDS can be reused
+  constexpr int RSTR = 256 + 16;   // padded row stride of a staging block
+  constexpr int BLK = 32 * RSTR;
+  uint8_t* st = &smem[0][0][0] + w * MOE_TILE_BYTES;  // this wave's 32 KB: two staging blocks, then the row table
+  int* srow = (int*)(st + 2 * BLK);
+  if (g == 0) {
 #pragma unroll
-  for (int bi = 0; bi < 4; ++bi) {
-    const int lr = wm * 128 + bi * 32 + r31;
-    rr[bi] = lr < mt.rows ? row_of(lr) : -1;
+    for (int bi = 0; bi < 4; ++bi) {
+      const int lr = wm * 128 + bi * 32 + r31;
+      srow[bi * 32 + r31] = lr < mt.rows ? row_of(lr) : -1;  // -1: not stored
+    }
   }
+  v4f bv[4][4];  // MODE 1: bias of this lane's columns n0 + wn*128 + 32 bj + 8 a + 4 g ..+3
+  if (MODE == 1) {
 #pragma unroll
-  for (int bj = 0; bj < 4; ++bj) {
-    v4f bv[4];
-    if (MODE == 1) {
+    for (int bj = 0; bj < 4; ++bj)
 #pragma unroll
       for (int a = 0; a < 4; ++a) {
-        bv[a] = (v4f){0.f, 0.f, 0.f, 0.f};
+        bv[bj][a] = (v4f){0.f, 0.f, 0.f, 0.f};
         const long n = ncol + bj * 32 + 8 * a;
         if (d.bias && n < N) {
           if (d.bias_f32) {
-            bv[a] = *(const v4f*)((const float*)d.bias + n);
+            bv[bj][a] = *(const v4f*)((const float*)d.bias + n);
           } else {
             const ov4 b16 = *(const ov4*)((const out_t*)d.bias + n);
-            bv[a] = (v4f){(float)b16[0], (float)b16[1], (float)b16[2], (float)b16[3]};
+            bv[bj][a] = (v4f){(float)b16[0], (float)b16[1], (float)b16[2], (float)b16[3]};
           }
         }
       }
-    }
+  }
+  auto stage_rows = [&](int bi) {  // accumulators of tile rows 32 bi .. +31 of this wave -> staging block bi % 2
+    uint8_t* sb = st + (bi & 1) * BLK + r31 * RSTR + 8 * g;
 #pragma unroll
-    for (int bi = 0; bi < 4; ++bi) {
-      if (rr[bi] < 0) continue;
-      out_t* crow = C + (long)rr[bi] * d.ldc + ncol + bj * 32;
+    for (int bj = 0; bj < 4; ++bj)
 #pragma unroll
       for (int a = 0; a < 4; ++a) {
         ov4 o;
@@ -292,14 +302,34 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restri
         for (int b = 0; b < 4; ++b) {
           float v = acc[bj][bi][4 * a + b];
           if (MODE == 1) {
-            v += bv[a][b];
+            v += bv[bj][a][b];
             if (d.relu) v = fmaxf(v, 0.f);
           }
           o[b] = (out_t)v;
         }
-        if (ncol + bj * 32 + 8 * a < N) *(ov4*)(crow + 8 * a) = o;
+        *(ov4*)(sb + (bj * 32 + 8 * a) * 2) = o;
       }
+  };
+  const int rb_row = lane >> 4, rb_ch = lane & 15;  // on the way out: 16 lanes per row, 4 rows per store instruction
+  const long ncol8 = n0 + wn * 128 + rb_ch * 8;    // N % 8 == 0: an 8-column piece is wholly inside the row or outside
+  auto drain = [&](int bi) {
+    const uint8_t* sb = st + (bi & 1) * BLK;
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+      const int row = p * 4 + rb_row;
+      const int r = srow[bi * 32 + row];
+      const v4i v = *(const v4i*)(sb + row * RSTR + rb_ch * 16);
+      if (r >= 0 && ncol8 < N) *(v4i*)(C + (long)r * d.ldc + ncol8) = v;
     }
+  };
+  // The LDS executes one wave's operations in order, so a block may be refilled as soon as the reads that drain it
+  // have been issued; the fences only pin that program order.  With two blocks the conversion of the next row block
+  // runs under the LDS and store latency of the previous one.
+#pragma unroll
+  for (int bi = 0; bi < 5; ++bi) {
+    if (bi < 4) stage_rows(bi);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    if (bi >= 1) drain(bi - 1);
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
 }
-

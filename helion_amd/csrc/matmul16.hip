@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256) void hx_matmul16_reduce(const float* __restric
 static bool mm_fast_ok(const void* a, const void* b, const void* c, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k,
                        int64_t ldb_n, int64_t ldc, const void* bias, int in_dtype) {
   if (in_dtype != HX_BF16 && in_dtype != HX_F16) return false;
-  if (K < MOE_BK || K % MOE_BK || N % 8 || lda % 8 || ldc % 4) return false;
+  if (K < MOE_BK || K % MOE_BK || N % 8 || lda % 8 || ldc % 8) return false;  // 16-byte row pieces in and out
   if ((((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)bias) & 15) != 0) return false;
   if (M * lda * 2 >= (1LL << 32)) return false;
   if (ldb_n == 1) return ldb_k % 8 == 0 && ldb_k * 4 < (1LL << 31);               // row-major B
