@@ -198,7 +198,7 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restri
                    int dstage, int d0) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      if (load_next && i < 8) load_frag(na, nw, nstage, nks, i);
+      if (load_next && !(i & 1)) load_frag(na, nw, nstage, nks, i >> 1);
       acc[i >> 2][i & 3] = Mfma16<BF>::run(cw[i >> 2], ca[i & 3], acc[i >> 2][i & 3]);
       if (dma && (i & 1)) issue_one(dkt, dstage, d0 + (i >> 1));
       __builtin_amdgcn_sched_barrier(0);
