@@ -7,7 +7,8 @@
 // Launch sequence (all on the caller's stream, no host synchronisation):
 //   1. hx_moe_prep       : builds the tile table (tile -> expert, first sorted row, row count) from
 //                          counts/offsets on the device and clears the row-covered flags;
-//   2. hx_moe_mark       : flags every row some expert covers;
+//   2. hx_moe_mark       : flags every row some expert covers (1 and 2 are one launch, hx_moe_prep_mark_small, for
+//                          small problems);
 //   3. hx_gemm16_tile256 / _tile128 / _rows32 or hx_moe_general : the grouped GEMM over (row tile, column tile) pairs;
 //   4. hx_moe_zero_rows  : zero-fills rows whose flag is still clear.
 // Padded rows of a tile are never stored, so there is no read-modify-write and no write race.
@@ -60,12 +61,84 @@ __global__ void hx_moe_mark(const int* __restrict__ num_tiles, const MoeTile* __
   }
 }
 
+// one workgroup per 256 rows: uncovered rows are rare, so most workgroups read 256 flags and leave
 template <typename T16>
-__global__ void hx_moe_zero_rows(T16* __restrict__ C, long ldc, int T, int N, const uint8_t* __restrict__ flags) {
-  const int row = blockIdx.x;
-  if (row >= T || flags[row]) return;
-  T16* c = C + (long)row * ldc;
-  for (int n = threadIdx.x; n < N; n += blockDim.x) c[n] = (T16)0.f;
+__global__ __launch_bounds__(256) void hx_moe_zero_rows(T16* __restrict__ C, long ldc, int T, int N, const uint8_t* __restrict__ flags) {
+  __shared__ uint8_t s_flag[256];
+  const int row0 = blockIdx.x * 256, tid = threadIdx.x;
+  const bool uncovered = row0 + tid < T && !flags[row0 + tid];
+  s_flag[tid] = uncovered;
+  if (!__syncthreads_or(uncovered)) return;
+  for (int r = 0; r < 256; ++r) {
+    if (!s_flag[r]) continue;  // workgroup-uniform
+    T16* c = C + (long)(row0 + r) * ldc;
+    for (int n = tid; n < N; n += 256) c[n] = (T16)0.f;
+  }
+}
+
+// Small problems (a decode step, a few thousand rows): one workgroup does what hx_moe_prep and hx_moe_mark do, so the
+// grouped GEMM is preceded by one short launch instead of two.  E <= 1024, T <= 4096.
+__global__ __launch_bounds__(1024) void hx_moe_prep_mark_small(const int32_t* __restrict__ counts, const int32_t* __restrict__ offsets,
+                                                               const int32_t* __restrict__ idx, int E, int T, int bm, int max_tiles,
+                                                               int* __restrict__ num_tiles, MoeTile* __restrict__ table,
+                                                               uint8_t* __restrict__ flags) {
+  __shared__ int s_first[1025];  // tiles before expert e (exclusive prefix), s_first[E] = total
+  __shared__ int s_start[1024], s_cnt[1024];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int i = tid; i < T; i += 1024) flags[i] = 0;
+  int nt = 0;
+  if (tid < E) {
+    int c = counts[tid];
+    c = c < 0 ? 0 : c;
+    const int start = offsets[tid];
+    // clamp malformed tables so the GEMM never indexes outside idx[0..T)
+    if (start < 0 || start > T) c = 0;
+    if (c > T - start) c = T - start;
+    s_start[tid] = start;
+    s_cnt[tid] = c;
+    nt = (c + bm - 1) / bm;
+  }
+  // inclusive scan of the tile counts over the 1024 threads (Hillis-Steele in LDS), shifted into s_first[1..]
+  if (tid == 0) s_first[0] = 0;
+  s_first[tid + 1] = nt;
+  __syncthreads();
+  for (int d = 1; d < 1024; d <<= 1) {
+    const int v = tid >= d ? s_first[tid + 1 - d] : 0;
+    __syncthreads();
+    s_first[tid + 1] += v;
+    __syncthreads();
+  }
+  const int total = min(s_first[E], max_tiles);
+  if (tid == 0) *num_tiles = total;
+  // tile t belongs to the expert e with s_first[e] <= t < s_first[e+1]
+  auto tile_of = [&](int t, int& e, int& rs, int& rows) {
+    int lo = 0, hi = E;  // invariant: s_first[lo] <= t < s_first[hi]
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (s_first[mid] <= t) lo = mid; else hi = mid;
+    }
+    e = lo;
+    const int i = t - s_first[lo];
+    rs = s_start[lo] + i * bm;
+    rows = min(bm, s_cnt[lo] - i * bm);
+  };
+  for (int t = tid; t < total; t += 1024) {
+    int e, rs, rows;
+    tile_of(t, e, rs, rows);
+    table[t].expert = e;
+    table[t].row_start = rs;
+    table[t].rows = rows;
+    table[t].pad = 0;
+  }
+  __syncthreads();  // (includes the wait for the flag stores above: they are cleared before any is set)
+  for (int t = wave; t < total; t += 16) {
+    int e, rs, rows;
+    tile_of(t, e, rs, rows);
+    for (int i = lane; i < rows; i += 64) {
+      const int r = idx[rs + i];
+      if (r >= 0 && r < T) flags[r] = 1;
+    }
+  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -155,11 +228,16 @@ static int launch_moe(const void* A, const void* W, void* C, const int32_t* coun
   tb = (tb + 255) & ~(size_t)255;
   uint8_t* flags = (uint8_t*)ws + tb;
 
-  const int prep_blocks = (int)((T + 256 * 64 - 1) / (256 * 64)) + 1;
-  hipLaunchKernelGGL(hx_moe_prep, dim3(prep_blocks), dim3(256), 0, s, counts, offsets, (int)E, (int)T, bm, max_tiles, num_tiles, table,
-                     flags);
-  hipLaunchKernelGGL(hx_moe_mark, dim3(max_tiles < 1024 ? max_tiles : 1024), dim3(256), 0, s, (const int*)num_tiles,
-                     (const MoeTile*)table, idx, (int)T, flags);
+  if (E <= 1024 && T <= 4096) {
+    hipLaunchKernelGGL(hx_moe_prep_mark_small, dim3(1), dim3(1024), 0, s, counts, offsets, idx, (int)E, (int)T, bm, max_tiles, num_tiles,
+                       table, flags);
+  } else {
+    const int prep_blocks = (int)((T + 256 * 64 - 1) / (256 * 64)) + 1;
+    hipLaunchKernelGGL(hx_moe_prep, dim3(prep_blocks), dim3(256), 0, s, counts, offsets, (int)E, (int)T, bm, max_tiles, num_tiles, table,
+                       flags);
+    hipLaunchKernelGGL(hx_moe_mark, dim3(max_tiles < 1024 ? max_tiles : 1024), dim3(256), 0, s, (const int*)num_tiles,
+                       (const MoeTile*)table, idx, (int)T, flags);
+  }
   if (fast) {
     G16Dense d = {};
     d.lda = K; d.ldb = N; d.ldc = N;
@@ -184,7 +262,8 @@ static int launch_moe(const void* A, const void* W, void* C, const int32_t* coun
     hipLaunchKernelGGL(hx_moe_general<T16>, grid, dim3(256), 0, s, (const T16*)A, (const T16*)W, (T16*)C, (const int*)num_tiles,
                        (const MoeTile*)table, idx, (int)T, (int)K, (int)N, (int)a_div);
   }
-  hipLaunchKernelGGL(hx_moe_zero_rows<T16>, dim3((unsigned)T), dim3(256), 0, s, (T16*)C, (long)N, (int)T, (int)N, (const uint8_t*)flags);
+  hipLaunchKernelGGL(hx_moe_zero_rows<T16>, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, s, (T16*)C, (long)N, (int)T, (int)N,
+                     (const uint8_t*)flags);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     hx_set_error("hx_moe_grouped_gemm: launch failed: %s", hipGetErrorString(e));
