@@ -192,47 +192,49 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restri
       wf[f - 4] = __builtin_bit_cast(V8, both);
     }
   };
-  // One k-step: 16 MFMAs on the current fragments; pinned between them the 8 fragment loads of the next k-step and,
-  // when DMA is set, NDMA DMA instructions starting at number D0 (one per MFMA), as in the fp8 GEMM.
-  auto kstep = [&](V8(&ca)[4], V8(&cw)[4], V8(&na)[4], V8(&nw)[4], int nstage, int nks, bool load_next, bool dma, int dkt,
-                   int dstage, int d0) {
+  // The fragments of a whole k-tile live in registers (4 k-steps x (4 A + 4 W) = 128 VGPRs) and are refilled in place
+  // with the next tile's as they die, always a good part of a tile before their next use, so that an LDS read slowed
+  // down by the DMA writing the same LDS never holds up an MFMA.  One k-tile:
+  //   first half  (k-steps 0, 1): 32 MFMAs and nothing else;
+  //   barrier: tile kt+1 has landed in the other stage, and the last reads of this stage (issued at the end of the
+  //            previous tile) are complete: it is free;
+  //   second half (k-steps 2, 3): 32 MFMAs, behind them the refills - k-steps 0 and 1 under k-step 2, k-step 2 under
+  //            k-step 3, k-step 3's own fragments each behind its last MFMA - and the 16 DMA instructions of tile kt+2
+  //            into the free stage, one every other MFMA.  Past the last tile the last one is fetched again and the
+  //            refills read whatever the other stage holds: every tile runs the same code.
+  V8 fa[4][4], fw[4][4];  // [k-step][row block], [k-step][column block]
+  auto mfma_ks = [&](int ks, auto after) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      if (load_next && !(i & 1)) load_frag(na, nw, nstage, nks, i >> 1);
-      acc[i >> 2][i & 3] = Mfma16<BF>::run(cw[i >> 2], ca[i & 3], acc[i >> 2][i & 3]);
-      if (dma && (i & 1)) issue_one(dkt, dstage, d0 + (i >> 1));
+      acc[i >> 2][i & 3] = Mfma16<BF>::run(fw[ks][i >> 2], fa[ks][i & 3], acc[i >> 2][i & 3]);
+      after(i);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-
-  // software pipeline, as in the fp8 GEMM: k-tile kt in stage kt&1, four k-steps per tile, fragments double
-  // buffered; the one barrier per tile sits before the last k-step's MFMAs; the 16 DMA instructions of tile kt+2 go
-  // out under the MFMAs of (kt, ks=3) and (kt+1, ks=0), one every other MFMA.
-  V8 fa0[4], fw0[4], fa1[4], fw1[4];
   issue(0, 0);
   if (nk > 1) issue(1, 1);
   if (nk > 1) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(16)); else HX_WAIT_VM0();
   __syncthreads();
 #pragma unroll
-  for (int f = 0; f < 8; ++f) load_frag(fa0, fw0, 0, 0, f);
-  for (int kt = 0; kt < nk - 1; ++kt) {
-    const int stage = kt & 1;
-    // (kt, ks=0): second half of tile kt+1's DMA (its first half went out under (kt-1, ks=3)); stage^1 is free
-    // since the last barrier, and both halves are complete at this iteration's barrier
-    kstep(fa0, fw0, fa1, fw1, stage, 1, true, kt > 0, min(kt + 1, nk - 1), stage ^ 1, 8);
-    kstep(fa1, fw1, fa0, fw0, stage, 2, true, false, 0, 0, 0);
-    kstep(fa0, fw0, fa1, fw1, stage, 3, true, false, 0, 0, 0);
+  for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+    for (int f = 0; f < 8; ++f) load_frag(fa[ks], fw[ks], 0, ks, f);
+  for (int kt = 0; kt < nk; ++kt) {
+    const int stage = kt & 1, dkt = min(kt + 2, nk - 1);
+    mfma_ks(0, [](int) {});
+    mfma_ks(1, [](int) {});
     HX_WAIT_VM0();
     __syncthreads();
-    // (kt, ks=3): first half of tile kt+2's DMA into the stage just freed
-    kstep(fa1, fw1, fa0, fw0, stage ^ 1, 0, true, true, min(kt + 2, nk - 1), stage, 0);
-  }
-  {
-    const int stage = (nk - 1) & 1;
-    kstep(fa0, fw0, fa1, fw1, stage, 1, true, nk > 1, nk - 1, stage ^ 1, 8);
-    kstep(fa1, fw1, fa0, fw0, stage, 2, true, false, 0, 0, 0);
-    kstep(fa0, fw0, fa1, fw1, stage, 3, true, false, 0, 0, 0);
-    kstep(fa1, fw1, fa0, fw0, 0, 0, false, false, 0, 0, 0);
+    mfma_ks(2, [&](int i) {
+      load_frag(fa[i >> 3], fw[i >> 3], stage ^ 1, i >> 3, i & 7);
+      if (i & 1) issue_one(dkt, stage, i >> 1);
+    });
+    mfma_ks(3, [&](int i) {
+      if (i < 8) load_frag(fa[2], fw[2], stage ^ 1, 2, i);
+      if (i & 1) issue_one(dkt, stage, 8 + (i >> 1));
+      if ((i & 3) == 3) load_frag(fa[3], fw[3], stage ^ 1, 3, 4 + (i >> 2));  // W fragment i>>2: its four MFMAs are out
+      if (i >= 12) load_frag(fa[3], fw[3], stage ^ 1, 3, i - 12);             // A fragment i-12: last used by MFMA i
+    });
   }
   HX_WAIT_VM0();  // trailing re-fetches must land before the workgroup's LDS is released
 
