@@ -203,7 +203,6 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
       if (j + 2 < ntiles) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(KPW));  // tile j+1 landed, tile j+2 may be in flight
       else HX_WAIT_VM0();
       __syncthreads();  // tile j+1 visible to every wave; every wave is done with tile j-1
-      if (j + ATT_LEAD < ntiles) issue_k(j + ATT_LEAD, (j + ATT_LEAD) % ATT_NS);
       if (active) {
         if (j + 1 < ntiles) scores(&smem[(j + 1) % ATT_NS][0][0], next);
 #pragma unroll
@@ -212,6 +211,7 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
           smax1 = fmaxf(fmaxf(smax1, cur[1][r]), cur[1][r + 1]);
         }
       }
+      if (j + ATT_LEAD < ntiles) issue_k(j + ATT_LEAD, (j + ATT_LEAD) % ATT_NS);  // (at the end of the step: see pass 2)
     };
     v16f sa[2], sb[2];
     if (active) scores(&smem[0][0][0], sa);
@@ -290,13 +290,15 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
       if (j + 2 < ntiles) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(KPW + VPW));
       else HX_WAIT_VM0();
       __syncthreads();
-      if (j + ATT_LEAD < ntiles) {
-        issue_k(j + ATT_LEAD, (j + ATT_LEAD) % ATT_NS);
-        issue_v(j + ATT_LEAD, (j + ATT_LEAD) % ATT_NS);
-      }
       if (active) {
         if (j + 1 < ntiles) scores(&smem[(j + 1) % ATT_NS][0][0], next);
         softmax_pv(cur, &smem[j % ATT_NS][1][0]);
+      }
+      // the slot freed by this step's barrier is refilled at the end of the step: four DMA instructions in a row hold
+      // the issuing wave up, and here nothing of this step is left to wait behind them (2 % against the top of the step)
+      if (j + ATT_LEAD < ntiles) {
+        issue_k(j + ATT_LEAD, (j + ATT_LEAD) % ATT_NS);
+        issue_v(j + ATT_LEAD, (j + ATT_LEAD) % ATT_NS);
       }
     };
     v16f sa[2], sb[2];
