@@ -51,6 +51,13 @@ def test_gemm_path_selection():
     assert lib.hx_fp8_gemm_path(33, 28672, 8192, 8192, 1, 8192, 28672, A, A, A) == 5   # a decode batch: 128-column tiles
     assert lib.hx_fp8_gemm_path(2048, 2048, 2048, 2048, 1, 2048, 2048, A, A, A) == 5   # 64 tiles of 256x256 would idle the chip
     assert lib.hx_fp8_gemm_path(4096, 4096, 4096, 4096, 1, 4096, 4096, A, A, A) == 1
+    # tile choice by estimated rounds: two rounds of 128x128 tiles beat one half-empty round of 256x256 tiles when K is
+    # long, but not five rounds against two when K is two k-tiles
+    assert lib.hx_fp8_gemm_path(1024, 7168, 8192, 8192, 1, 8192, 7168, A, A, A) == 5
+    assert lib.hx_fp8_gemm_path(2048, 4096, 4096, 4096, 1, 4096, 4096, A, A, A) == 5
+    assert lib.hx_fp8_gemm_path(8192, 1280, 8192, 8192, 1, 8192, 1280, A, A, A) == 1
+    assert lib.hx_fp8_gemm_path(4096, 8192, 7168, 7168, 1, 7168, 8192, A, A, A) == 1
+    assert lib.hx_fp8_gemm_path(4000, 4100, 256, 256, 1, 256, 4100, A, A, A) == 3
     assert lib.hx_fp8_gemm_path(256, 256, 256, 256, 256, 1, 256, A, A, A) == 4  # row-major B, read in place
     assert lib.hx_fp8_gemm_path(16, 256, 256, 256, 256, 1, 256, A, A, A) == 0   # row-major B for the skinny shape: via workspace
     assert lib.hx_fp8_gemm_path(100, 72, 128, 128, 72, 1, 72, A, A, A) == 0     # row-major B, N % 16 != 0
