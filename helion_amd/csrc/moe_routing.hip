@@ -75,8 +75,38 @@ __global__ __launch_bounds__(64 * RT_WAVES) void hx_moe_routing_kernel(const IdT
   const int chunk = block_rows / RT_WAVES;
   const int begin = (int)min((long long)T, b0 + (long long)w * chunk), end = (int)min((long long)T, (long long)begin + chunk);
 
+  // Up to 2048 rows per wave (the one-workgroup form up to 32768 rows) the ids are read once, all loads in flight
+  // together, and both passes walk the registers.
+  constexpr int RT_CACHE = 32;
+  const bool cached = MODE == 0 && chunk <= 64 * RT_CACHE;  // workgroup-uniform
+  int ec[RT_CACHE];
+  if (cached) {
+#pragma unroll
+    for (int u = 0; u < RT_CACHE; ++u) {
+      const int r = begin + 64 * u + lane;
+      ec[u] = -1;
+      if (r < end) {
+        const IdT v = ids[r];
+        ec[u] = (v >= 0 && v < (IdT)E) ? (int)v : -1;
+      }
+    }
+  }
+  auto for_rows = [&](auto f) {
+    if (cached) {
+#pragma unroll
+      for (int u = 0; u < RT_CACHE; ++u) {
+        if (begin + 64 * u >= end) break;  // wave-uniform
+        const bool ok = ec[u] >= 0;
+        const uint64_t m = rt_match(ec[u], ok, nbits);
+        if (ok) f(begin + 64 * u + lane, ec[u], m);
+      }
+    } else {
+      rt_for_rows(ids, begin, end, E, nbits, lane, f);
+    }
+  };
+
   // ---- count pass: the first lane of every group of equal experts adds the group's size
-  rt_for_rows(ids, begin, end, E, nbits, lane, [&](int, int e, uint64_t m) {
+  for_rows([&](int, int e, uint64_t m) {
     if ((m & lt_mask) == 0) hist[w][e] += __builtin_popcountll(m);
   });
   __syncthreads();
@@ -129,7 +159,7 @@ __global__ __launch_bounds__(64 * RT_WAVES) void hx_moe_routing_kernel(const IdT
   __syncthreads();
 
   // ---- scatter pass
-  rt_for_rows(ids, begin, end, E, nbits, lane, [&](int r, int e, uint64_t m) {
+  for_rows([&](int r, int e, uint64_t m) {
     const int slot = hist[w][e];  // every lane of the group reads before its first lane advances the slot
     const int rank = __builtin_popcountll(m & lt_mask);
     if (rank == 0) hist[w][e] = slot + __builtin_popcountll(m);
