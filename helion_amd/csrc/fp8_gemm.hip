@@ -1,10 +1,12 @@
 // FP8 (OCP e4m3fn) GEMM for gfx950: C[M,N] = cast((A[M,K] @ B[K,N]) * scale_a*scale_b), fp32 accumulate.
 // Drop-in device side of examples/fp8_gemm.py:29-57 of the reference.
 //
-// Three kernels:
-//   hx_fp8_gemm_tile256 : 256x256x128 workgroup tile, 4 waves (2x2) of 128x128, 32x32x64 fp8 MFMA,
+// The kernels:
+//   hx_fp8_gemm_tile256 : 256x256x128 workgroup tile, 4 waves (2x2) of 128x128, 16x16x128 fp8 MFMA,
 //                         A/B k-tiles DMA'd global->LDS (double buffered, XOR-swizzled 16B chunks).
-//   hx_fp8_gemm_tileN128 : 128x128 / 256x128 tiles with a deeper LDS ring, for problems with too few 256x256 tiles.
+//   hx_fp8_gemm_tileN128 : 64/128/256 x 128 tiles with a deeper LDS ring, for problems with too few 256x256 tiles
+//                         (decode batches, mid-size products), with split-K (+ hx_fp8_gemm_split_reduce) when even
+//                         those tiles are few and K is long.
 //   hx_fp8_gemm_skinny_direct : M <= 32, K <= 8192; HBM-bound streaming of B^T through registers into
 //                         16x16x128 MFMA, K split across the 8 waves of a workgroup, partials summed in LDS.
 //   hx_fp8_gemm_skinny  : M <= 16, larger K; same split, A panel staged through LDS in 8 KB chunks of K.
@@ -317,12 +319,12 @@ __global__ __launch_bounds__(256) void hx_transpose_u8(const uint8_t* __restrict
 }
 
 // ------------------------------------------------------------------------------------------
-// tileN128: BM x 128 x 128 workgroup tile (BM = 128 or 256), for problems that 256x256 tiles cut into too few pieces
+// tileN128: BM x 128 x 128 workgroup tile (BM = 64, 128 or 256), for problems that 256x256 tiles cut into too few pieces
 // to occupy the chip: a decode batch of 33..256 rows against a wide weight matrix (one row tile: the kernel is then a
 // weight-streaming loop and wants every CU busy and several k-tiles in flight per CU), or a mid-size square product.
 // Column-major B (B^T rows of K).  4 waves (2x2) of (BM/2) x 64, 16x16x128 MFMAs, same LDS tile layout and k-block
-// assignment as tile256.  LDS ring of NS stages of (A BM x 128 B + B 128 x 128 B): NS - 1 k-tiles in flight; the
-// fragments of k-tile kt+1 are read into a second register set before the MFMAs of tile kt.  Rows and columns past
+// assignment as tile256.  LDS ring of NS stages of (A BM x 128 B + B 128 x 128 B): NS - 1 k-tiles in flight; one set
+// of fragments per wave, refilled in place with k-tile kt+1's behind the MFMAs of tile kt.  Rows and columns past
 // M / N re-read the last valid one and are never stored, so ragged M and N need no second instantiation.
 // bn (a multiple of 16, 64..128) is the column pitch of the tiles: with a single row tile the host picks it so that
 // the column tiles come to about one per CU (N = 28672: 112 columns, 256 tiles); the columns of a tile past bn
