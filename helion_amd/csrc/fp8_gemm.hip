@@ -354,7 +354,11 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tileN128(const uint8_t* __res
   int tm, tn;
   {
     const int nwg = gridDim.x, wg = blockIdx.x, chunk = wg >> 8, tiles_n = nwg / tiles_m;
-    const int tile = chunk < (nwg >> 8) ? (chunk << 8) + ((wg & 7) << 5) + ((wg >> 3) & 31) : wg;
+    // (the last, partial run of R tiles likewise in 8 blocks of R / 8 when R is a multiple of 8)
+    const int rem = nwg & 255, l = wg & 255;
+    const int tile = chunk < (nwg >> 8) ? (chunk << 8) + ((wg & 7) << 5) + ((wg >> 3) & 31)
+                     : (rem & 7) == 0   ? (chunk << 8) + (l & 7) * (rem >> 3) + (l >> 3)
+                                        : wg;
     constexpr int GM = 8;
     const int group_size = GM * tiles_n, first_m = (tile / group_size) * GM;
     const int gm = min(tiles_m - first_m, GM);
@@ -813,19 +817,23 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_split_reduce(const float* __r
 // ------------------------------------------------------------------------------------------
 static inline bool aligned(const void* p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
-// Which tile for a K-contiguous problem: 256x256 (returns 0) or 128 columns wide (returns the tile's rows: one row tile
-// of 64, 128 or 256 rows for a decode batch that streams weights from HBM, 128 otherwise).  Both kernels run one
-// workgroup per CU, so a launch takes ceil(tiles / 256) rounds, each of K / 128 k-tile steps plus a prologue and an
-// epilogue.  Measured with every CU busy: a 256x256 step 1.37 us and about 6 us per round outside the loop, a 128x128
-// step 0.5 us (it is bound by what the CUs can pull out of the L2s, not by its MFMAs) and about 3 us per round.  A
-// 256x128 tile for more than 256 rows measured no better than either.
+// Which tile for a K-contiguous problem: 256x256 (returns 0) or 128 columns wide (returns the tile's rows: 64, 128 or
+// 256).  Up to 256 rows it is one row tile, a decode batch that streams weights from HBM.  Beyond that all kernels run
+// one workgroup per CU, so a launch takes ceil(tiles / 256) rounds, each of K / 128 k-tile steps plus a prologue and an
+// epilogue, and the cheapest estimate wins.  Measured with every CU busy, per step and per round outside the loop:
+// 256x256 1.37 us and 6 us; 128x128 0.43 us and 4.6 us (it is bound by what the CUs can pull out of the L2s, not by
+// its MFMAs); 256x128 0.8 us and 9 us, and only with at least three row tiles (with two, an XCD's tiles share too few
+// operand panels: 512 x 14336 x 4096 measured 40 us against 36 for 128x128).
 static int tileN128_rows(int64_t M, int64_t N, int64_t K) {
   auto rounds = [&](int64_t bm, int64_t bn) { return (((M + bm - 1) / bm) * ((N + bn - 1) / bn) + 255) / 256; };
   if (M <= 64) return 64;
   if (M <= 128) return 128;
   if (M <= 256) return 256;
   const int64_t nk = (K + T256_BK - 1) / T256_BK;
-  return rounds(128, 128) * (50 * nk + 300) < rounds(256, 256) * (137 * nk + 600) ? 128 : 0;
+  const int64_t c256 = rounds(256, 256) * (137 * nk + 600), c128 = rounds(128, 128) * (43 * nk + 460);
+  const int64_t c21 = M > 512 ? rounds(256, 128) * (80 * nk + 900) : INT64_MAX;
+  if (c256 <= c128 && c256 <= c21) return 0;
+  return c21 < c128 ? 256 : 128;
 }
 
 // column pitch of the 128-column tiles: 128, except that a single row tile of at most 128 rows (a decode batch) gets

@@ -64,7 +64,11 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restri
   int tile;
   {
     const int nwg = gridDim.x, wg = blockIdx.x, chunk = wg >> 8;
-    tile = chunk < (nwg >> 8) ? (chunk << 8) + ((wg & 7) << 5) + ((wg >> 3) & 31) : wg;
+    // (the last, partial run of R tiles likewise in 8 blocks of R / 8 when R is a multiple of 8)
+    const int rem = nwg & 255, l = wg & 255;
+    tile = chunk < (nwg >> 8) ? (chunk << 8) + ((wg & 7) << 5) + ((wg >> 3) & 31)
+           : (rem & 7) == 0   ? (chunk << 8) + (l & 7) * (rem >> 3) + (l >> 3)
+                              : wg;
   }
   const int GM = 4;
   const int group_size = GM * tiles_n;
