@@ -12,19 +12,23 @@ struct MoeTile {
 
 
 // ------------------------------------------------------------------------------------------
-// tile256: 256 gathered rows x 256 columns x 64 k per step; 4 waves (2x2) of 128x128; 32x32x16 MFMA.
+// tile256: 256 gathered rows x 256 columns x 64 k per step; 4 waves (2x2) of 128x128; 16x16x32 MFMA (under the power
+//   limit a stream of them sustains about a fifth more than one of 32x32x16: a quarter of the accumulator registers
+//   move per instruction).
 //   A tile  [256 rows][128 B]  : same chunk-swizzled layout as the fp8 GEMM; the DMA gathers rows
 //                                through idx, so the gather costs nothing extra.
 //   W tile  [64 k][512 B]      : row = k, 32 chunks of 8 columns; chunk stored at pos = chunk ^ (moe_wswz(k)<<1).
 //                                The MFMA wants 8 consecutive k per lane for one column, W has the
 //                                columns contiguous: ds_read_b64_tr_b16 transposes 4(k) x 16(n) blocks
 //                                on the way out of LDS (two reads per operand).
+//   One MFMA multiplies 32 k; lane (r = lane%16, g = lane/16) supplies k = 8g .. 8g+7 of row / column r: chunk
+//   4*ks + g of an A row, k rows 32*ks + 8g .. +7 of a W column.
 // ------------------------------------------------------------------------------------------
 // Swizzle of a W-tile row, in units of 32 bytes (a pair of chunks).  One transposing read has the 32 lanes
-// that the LDS serves together fetch 4 consecutive k rows x two adjacent 32-byte column groups; rows are 512 B
-// apart (the same banks), so the 8 (row, group) combinations must land in 8 different 32-byte bank groups:
-// k&3 goes to bits 2:1 and bit 2 of k to bit 0, which the column-group bit then flips.
-__device__ __forceinline__ int moe_wswz(int k) { return ((k & 3) << 1) | ((k >> 2) & 1); }
+// that the LDS serves together (two groups of 16) fetch 4 consecutive k rows each, 8 rows apart, of the same 32-byte
+// column group; rows are 512 B apart (the same banks), so the 8 rows must land in 8 different 32-byte bank groups:
+// k&3 goes to bits 2:1 and bit 3 of k to bit 0.
+__device__ __forceinline__ int moe_wswz(int k) { return ((k & 3) << 1) | ((k >> 3) & 1); }
 
 #define MOE_BM 256
 #define MOE_BN 256
@@ -116,15 +120,15 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restri
     a_vo[j] = (uint32_t)(r / a_div) * (uint32_t)(d.lda * 2) + (uint32_t)((lpos ^ swz) * 16);
   }
   // ---- W DMA: wave w owns k rows [16w, 16w+16), 8 instructions of 2 rows x 512 B.
-  // row k = 16w + 2j + (lane>>5); chunk = (lane&31) ^ (moe_wswz(k)<<1); k&7 = (2j + (lane>>5)) & 7
+  // row k = 16w + 2j + (lane>>5); chunk = (lane&31) ^ (moe_wswz(k)<<1); k&15 = 2j + (lane>>5)
   const uint8_t* We = W + (long)mt.expert * K * N * 2 + n0 * 2 + ((long)kt0 * MOE_BK + w * 16) * d.ldb * 2;  // wave-uniform
   const int wk_l = lane >> 5, wpos = lane & 31;
-  uint32_t w_vo[4];
+  uint32_t w_vo[8];
   // The last column tile may be ragged (N % 256 != 0, N % 8 == 0): chunks past the end re-read the last valid chunk of
   // the row; the columns they feed are never stored.
   const int cmax = (int)((min((long)N - n0, (long)MOE_BN) >> 3) - 1);
 #pragma unroll
-  for (int j = 0; j < 4; ++j) w_vo[j] = (uint32_t)(wk_l * d.ldb * 2 + min(wpos ^ (moe_wswz(2 * j + wk_l) << 1), cmax) * 16);
+  for (int j = 0; j < 8; ++j) w_vo[j] = (uint32_t)(wk_l * d.ldb * 2 + min(wpos ^ (moe_wswz(2 * j + wk_l) << 1), cmax) * 16);
   // column-major W: wave w owns tile columns [64w, 64w+64) = rows of W^T, 8 instructions of 8 rows, exactly like A;
   // columns past N re-read column N-1 and are never stored (W^T is below 4 GB, checked by the host)
   uint32_t wc_vo[BCOL ? 8 : 1];
@@ -144,7 +148,7 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restri
     const uint32_t lw = lds0 + (uint32_t)stage * 2 * MOE_TILE_BYTES + MOE_TILE_BYTES + (uint32_t)w * 16 * 512;
     if (i < 8) hx_g2l16_s(A + (long)kt * 128, a_vo[i], la + i * 1024);
     else if (BCOL) hx_g2l16_s(W + ((long)kt0 + kt) * 128, wc_vo[BCOL ? i - 8 : 0], lds0 + (uint32_t)stage * 2 * MOE_TILE_BYTES + MOE_TILE_BYTES + (uint32_t)w * 64 * 128 + (i - 8) * 1024);
-    else hx_g2l16_s(We + ((long)kt * MOE_BK + 2 * (i - 8)) * d.ldb * 2, w_vo[(i - 8) & 3], lw + (i - 8) * 1024);
+    else hx_g2l16_s(We + ((long)kt * MOE_BK + 2 * (i - 8)) * d.ldb * 2, w_vo[i - 8], lw + (i - 8) * 1024);
   };
   auto issue = [&](int kt, int stage) {
 #pragma unroll
@@ -152,65 +156,63 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restri
   };
 
   // ---- operand addressing
-  const int r31 = lane & 31, g = lane >> 5;
-  const int ax = (g ^ ((r31 >> 1) & 7)) * 16;  // chunk (2*ks + g) ^ swz -> ax ^ (ks*32)
-  const int a_base = (wm * 128 + r31) * 128;
-  // transposing read: lane -> (block b = lane>>4, e = (lane>>2)&3, q = lane&3)
-  //   k = 16*ks + 8*(b>>1) + 4*half + e ; n = wn*128 + 32*bj + 16*(b&1) + 4q
-  const int tb = lane >> 4, te = (lane >> 2) & 3, tq = lane & 3;
-  const int tk = 8 * (tb >> 1) + te;                  // + 16*ks + 4*half
-  const int tn_ = wn * 128 + 16 * (tb & 1) + 4 * tq;  // + 32*bj
-  // byte offset of (k = tk + 4*half, n = tn_) in the W tile.  Column block bj adds 4 to the chunk index in bits
-  // the swizzle mask and tn_>>3 leave alone, so it is an xor with 64*bj; k-step ks adds 16 rows = 8192 bytes.
+  const int r16 = lane & 15, g = lane >> 4;
+  const int ax = (g ^ ((r16 >> 1) & 7)) * 16;  // chunk (4*ks + g) ^ swz -> ax ^ (ks*64)
+  const int a_base = (wm * 128 + r16) * 128;
+  // transposing read: lane -> (group g = lane>>4, e = (lane>>2)&3, q = lane&3) supplies 8 bytes of
+  //   k = 32*ks + 8*g + 4*half + e ; n = wn*128 + 16*bj + 4q   and receives column lane%16 of block bj, 4 k
+  const int te = (lane >> 2) & 3, tq = lane & 3;
+  const int tn_ = wn * 128 + 4 * tq;  // + 16*bj
+  // byte offset of (k = 8g + e + 4*half, n = tn_) in the W tile.  Column block bj adds 2 to the chunk index in bits
+  // the swizzle mask covers and tn_>>3 leaves alone, so it is an xor with 32*bj; k-step ks adds 32 rows = 16384 bytes.
   int w_off[2];
 #pragma unroll
   for (int half = 0; half < 2; ++half) {
-    const int k = tk + 4 * half;
+    const int k = 8 * g + te + 4 * half;
     w_off[half] = k * 512 + (((tn_ >> 3) ^ (moe_wswz(k) << 1)) * 16) + (tn_ & 7) * 2;
   }
 
-  v16f acc[4][4];
+  // acc[bj][bi][r] is C[row_of(wm*128 + 16 bi + lane%16)][n0 + wn*128 + 16 bj + 4*(lane/16) + r]
+  v4f acc[8][8];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    for (int j = 0; j < 8; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
 
-  // fragment f (0..7) of k-step ks (16 k) of a stage: f < 4 -> A rows 32f.. (one b128), else W columns 32(f-4)..
-  // (two transposing b64 reads)
-  auto load_frag = [&](V8(&af)[4], V8(&wf)[4], int stage, int ks, int f) {
-    if (f < 4) {
-      af[f] = *(const V8*)(&smem[stage][0][0] + a_base + f * 4096 + (ax ^ (ks * 32)));
+  // fragment f (0..15) of k-step ks (32 k) of a stage: f < 8 -> A rows 16f.. (one b128), else W columns 16(f-8)..
+  // (two transposing b64 reads, or one b128 of a column-major W)
+  auto load_frag = [&](V8(&af)[8], V8(&wf)[8], int stage, int ks, int f) {
+    if (f < 8) {
+      af[f] = *(const V8*)(&smem[stage][0][0] + a_base + f * 2048 + (ax ^ (ks * 64)));
     } else if (BCOL) {
-      wf[f - 4] = *(const V8*)(&smem[stage][1][0] + (wn * 128 + r31) * 128 + (f - 4) * 4096 + (ax ^ (ks * 32)));
+      wf[f - 8] = *(const V8*)(&smem[stage][1][0] + (wn * 128 + r16) * 128 + (f - 8) * 2048 + (ax ^ (ks * 64)));
     } else {
       const uint8_t* sw = &smem[stage][1][0];
       v4s part[2];
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
-        const int off = (w_off[half] ^ ((f - 4) * 64)) + ks * 8192;
+        const int off = (w_off[half] ^ ((f - 8) * 32)) + ks * 16384;
         part[half] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3)))*)(sw + off));
       }
       v8s both = (v8s){part[0][0], part[0][1], part[0][2], part[0][3], part[1][0], part[1][1], part[1][2], part[1][3]};
-      wf[f - 4] = __builtin_bit_cast(V8, both);
+      wf[f - 8] = __builtin_bit_cast(V8, both);
     }
   };
-  // The fragments of a whole k-tile live in registers (4 k-steps x (4 A + 4 W) = 128 VGPRs) and are refilled in place
+  // The fragments of a whole k-tile live in registers (2 k-steps x (8 A + 8 W) = 128 VGPRs) and are refilled in place
   // with the next tile's as they die, always a good part of a tile before their next use, so that an LDS read slowed
   // down by the DMA writing the same LDS never holds up an MFMA.  One k-tile:
-  //   first half  (k-steps 0, 1): 32 MFMAs and nothing else;
+  //   first half  (k-step 0): 64 MFMAs and nothing else;
   //   barrier: tile kt+1 has landed in the other stage, and the last reads of this stage (issued at the end of the
   //            previous tile) are complete: it is free;
-  //   second half (k-steps 2, 3): 32 MFMAs, behind them the refills - k-steps 0 and 1 under k-step 2, k-step 2 under
-  //            k-step 3, k-step 3's own fragments each behind its last MFMA - and the 16 DMA instructions of tile kt+2
-  //            into the free stage, one every other MFMA.  Past the last tile the last one is fetched again and the
-  //            refills read whatever the other stage holds: every tile runs the same code.
-  V8 fa[4][4], fw[4][4];  // [k-step][row block], [k-step][column block]
+  //   second half (k-step 1): 64 MFMAs, behind them the refills - k-step 0's fragments under the first 32, k-step 1's
+  //            own each behind its last MFMA - and the 16 DMA instructions of tile kt+2 into the free stage, one every
+  //            fourth MFMA.  Past the last tile the last one is fetched again and the refills read whatever the other
+  //            stage holds: every tile runs the same code.
+  V8 fa[2][8], fw[2][8];  // [k-step][row block], [k-step][column block]
   auto mfma_ks = [&](int ks, auto after) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      acc[i >> 2][i & 3] = Mfma16<BF>::run(fw[ks][i >> 2], fa[ks][i & 3], acc[i >> 2][i & 3]);
+    for (int i = 0; i < 64; ++i) {
+      acc[i >> 3][i & 7] = Mfma16<BF>::run16(fw[ks][i >> 3], fa[ks][i & 7], acc[i >> 3][i & 7]);
       after(i);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -220,46 +222,25 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restri
   if (nk > 1) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(16)); else HX_WAIT_VM0();
   __syncthreads();
 #pragma unroll
-  for (int ks = 0; ks < 4; ++ks)
+  for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-    for (int f = 0; f < 8; ++f) load_frag(fa[ks], fw[ks], 0, ks, f);
+    for (int f = 0; f < 16; ++f) load_frag(fa[ks], fw[ks], 0, ks, f);
   for (int kt = 0; kt < nk; ++kt) {
     const int stage = kt & 1, dkt = min(kt + 2, nk - 1);
     mfma_ks(0, [](int) {});
-    mfma_ks(1, [](int) {});
     HX_WAIT_VM0();
     __syncthreads();
-    mfma_ks(2, [&](int i) {
-      load_frag(fa[i >> 3], fw[i >> 3], stage ^ 1, i >> 3, i & 7);
-      if (i & 1) issue_one(dkt, stage, i >> 1);
-    });
-    mfma_ks(3, [&](int i) {
-      if (i < 8) load_frag(fa[2], fw[2], stage ^ 1, 2, i);
-      if (i & 1) issue_one(dkt, stage, 8 + (i >> 1));
-      if ((i & 3) == 3) load_frag(fa[3], fw[3], stage ^ 1, 3, 4 + (i >> 2));  // W fragment i>>2: its four MFMAs are out
-      if (i >= 12) load_frag(fa[3], fw[3], stage ^ 1, 3, i - 12);             // A fragment i-12: last used by MFMA i
+    mfma_ks(1, [&](int i) {
+      if (i < 32 && !(i & 1)) load_frag(fa[0], fw[0], stage ^ 1, 0, i >> 1);
+      if ((i & 3) == 3) issue_one(dkt, stage, i >> 2);
+      if ((i & 7) == 7) load_frag(fa[1], fw[1], stage ^ 1, 1, 8 + (i >> 3));  // W fragment i>>3: its eight MFMAs are out
+      if (i >= 56) load_frag(fa[1], fw[1], stage ^ 1, 1, i - 56);              // A fragment i-56: last used by MFMA i
     });
   }
   HX_WAIT_VM0();  // trailing re-fetches must land before the workgroup's LDS is released
 
-  // ---- epilogue: acc[bj][bi][4a+b] is C[row_of(wm*128 + bi*32 + lane%32)][n0 + wn*128 + bj*32 + 8a + 4g + b].
+  // ---- epilogue: acc[bj][bi][r] is C[row_of(wm*128 + 16 bi + lane%16)][n0 + wn*128 + 16 bj + 4g + r].
   const long ncol = n0 + wn * 128 + 4 * g;
-  if (MODE == 2) {
-    float* Cp = (float*)Cv + (long)blockIdx.y * T * d.ldc;
-#pragma unroll
-    for (int bi = 0; bi < 4; ++bi) {
-      const int lr = wm * 128 + bi * 32 + r31;
-      if (lr >= mt.rows) continue;
-      float* crow = Cp + (long)(mt.row_start + lr) * d.ldc + ncol;
-#pragma unroll
-      for (int bj = 0; bj < 4; ++bj)
-#pragma unroll
-        for (int a = 0; a < 4; ++a)
-          if (ncol + bj * 32 + 8 * a < N)
-            *(v4f*)(crow + bj * 32 + 8 * a) = (v4f){acc[bj][bi][4 * a], acc[bj][bi][4 * a + 1], acc[bj][bi][4 * a + 2], acc[bj][bi][4 * a + 3]};
-    }
-    return;
-  }
   // A lane holds 4 consecutive columns of a row, so direct stores would hit every 128-byte line of C with sixteen
   // separate 8-byte writes, and the write burst at the end of a round of tiles becomes L2-transaction-bound.  Each wave
   // instead passes 32 rows x 128 columns at a time through its own quarter of the (now idle) LDS and writes whole
@@ -272,58 +253,86 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restri
   constexpr int BLK = 32 * RSTR;
   uint8_t* st = &smem[0][0][0] + w * MOE_TILE_BYTES;  // this wave's 32 KB: two staging blocks, then the row table
   int* srow = (int*)(st + 2 * BLK);
-  if (g == 0) {
 #pragma unroll
-    for (int bi = 0; bi < 4; ++bi) {
-      const int lr = wm * 128 + bi * 32 + r31;
-      srow[bi * 32 + r31] = lr < mt.rows ? row_of(lr) : -1;  // -1: not stored
-    }
+  for (int p = 0; p < 2; ++p) {
+    const int lr = wm * 128 + p * 64 + lane;
+    srow[p * 64 + lane] = lr < mt.rows ? row_of(lr) : -1;  // -1: not stored
   }
-  v4f bv[4][4];  // MODE 1: bias of this lane's columns n0 + wn*128 + 32 bj + 8 a + 4 g ..+3
-  if (MODE == 1) {
+  if (MODE == 2) {  // fp32 accumulators as they are: 16 rows x 128 columns per staging block, two rows per store instruction
+    float* Cp = (float*)Cv + (long)blockIdx.y * T * d.ldc;
+    constexpr int RS2 = 512 + 16, BLK2 = 16 * RS2;
+    const int q_row = lane >> 5, q_ch = lane & 31;
+    const long ncol4 = n0 + wn * 128 + q_ch * 4;
 #pragma unroll
-    for (int bj = 0; bj < 4; ++bj)
+    for (int bb = 0; bb < 9; ++bb) {
+      if (bb < 8) {
+        uint8_t* sb = st + (bb & 1) * BLK2 + r16 * RS2 + 16 * g;
 #pragma unroll
-      for (int a = 0; a < 4; ++a) {
-        bv[bj][a] = (v4f){0.f, 0.f, 0.f, 0.f};
-        const long n = ncol + bj * 32 + 8 * a;
-        if (d.bias && n < N) {
-          if (d.bias_f32) {
-            bv[bj][a] = *(const v4f*)((const float*)d.bias + n);
-          } else {
-            const ov4 b16 = *(const ov4*)((const out_t*)d.bias + n);
-            bv[bj][a] = (v4f){(float)b16[0], (float)b16[1], (float)b16[2], (float)b16[3]};
-          }
+        for (int bj = 0; bj < 8; ++bj) {
+          v4f t = acc[bj][bb];
+          asm volatile("" : "+v"(t));  // a copy the compiler cannot fold into the accumulator's own register
+          *(v4f*)(sb + bj * 64) = t;
         }
       }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      if (bb >= 1) {
+        const uint8_t* sb = st + ((bb - 1) & 1) * BLK2;
+#pragma unroll
+        for (int p = 0; p < 8; ++p) {
+          const int row = p * 2 + q_row;
+          const int r = srow[(bb - 1) * 16 + row];
+          const v4i v = *(const v4i*)(sb + row * RS2 + q_ch * 16);
+          if (r >= 0 && ncol4 < N) *(v4i*)(Cp + (long)r * d.ldc + ncol4) = v;
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    return;
   }
-  auto stage_rows = [&](int bi) {  // accumulators of tile rows 32 bi .. +31 of this wave -> staging block bi % 2
-    uint8_t* sb = st + (bi & 1) * BLK + r31 * RSTR + 8 * g;
+  v4f bv[8];  // MODE 1: bias of this lane's columns n0 + wn*128 + 16 bj + 4 g ..+3
+  if (MODE == 1) {
 #pragma unroll
-    for (int bj = 0; bj < 4; ++bj)
+    for (int bj = 0; bj < 8; ++bj) {
+      bv[bj] = (v4f){0.f, 0.f, 0.f, 0.f};
+      const long n = ncol + bj * 16;
+      if (d.bias && n < N) {
+        if (d.bias_f32) {
+          bv[bj] = *(const v4f*)((const float*)d.bias + n);
+        } else {
+          const ov4 b16 = *(const ov4*)((const out_t*)d.bias + n);
+          bv[bj] = (v4f){(float)b16[0], (float)b16[1], (float)b16[2], (float)b16[3]};
+        }
+      }
+    }
+  }
+  auto stage_rows = [&](int bb) {  // accumulators of tile rows 32 bb .. +31 of this wave -> staging block bb % 2
 #pragma unroll
-      for (int a = 0; a < 4; ++a) {
+    for (int h = 0; h < 2; ++h) {
+      uint8_t* sb = st + (bb & 1) * BLK + (16 * h + r16) * RSTR + 8 * g;
+#pragma unroll
+      for (int bj = 0; bj < 8; ++bj) {
         ov4 o;
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
-          float v = acc[bj][bi][4 * a + b];
+          float v = acc[bj][2 * bb + h][b];
           if (MODE == 1) {
-            v += bv[bj][a][b];
+            v += bv[bj][b];
             if (d.relu) v = fmaxf(v, 0.f);
           }
           o[b] = (out_t)v;
         }
-        *(ov4*)(sb + (bj * 32 + 8 * a) * 2) = o;
+        *(ov4*)(sb + bj * 32) = o;
       }
+    }
   };
   const int rb_row = lane >> 4, rb_ch = lane & 15;  // on the way out: 16 lanes per row, 4 rows per store instruction
   const long ncol8 = n0 + wn * 128 + rb_ch * 8;    // N % 8 == 0: an 8-column piece is wholly inside the row or outside
-  auto drain = [&](int bi) {
-    const uint8_t* sb = st + (bi & 1) * BLK;
+  auto drain = [&](int bb) {
+    const uint8_t* sb = st + (bb & 1) * BLK;
 #pragma unroll
     for (int p = 0; p < 8; ++p) {
       const int row = p * 4 + rb_row;
-      const int r = srow[bi * 32 + row];
+      const int r = srow[bb * 32 + row];
       const v4i v = *(const v4i*)(sb + row * RSTR + rb_ch * 16);
       if (r >= 0 && ncol8 < N) *(v4i*)(C + (long)r * d.ldc + ncol8) = v;
     }
@@ -332,10 +341,10 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restri
   // have been issued; the fences only pin that program order.  With two blocks the conversion of the next row block
   // runs under the LDS and store latency of the previous one.
 #pragma unroll
-  for (int bi = 0; bi < 5; ++bi) {
-    if (bi < 4) stage_rows(bi);
+  for (int bb = 0; bb < 5; ++bb) {
+    if (bb < 4) stage_rows(bb);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    if (bi >= 1) drain(bi - 1);
+    if (bb >= 1) drain(bb - 1);
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
 }

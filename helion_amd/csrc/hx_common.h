@@ -64,7 +64,8 @@ __device__ __forceinline__ v4f hx_mfma_16x16x128_e4m3(v8i a, v8i b, v4f c) {
 }
 
 // 16-bit MFMA (32x32x16, fp32 accumulate): lane l supplies 8 elements of row/col l%32, k = 8*(l/32) .. +7; the result
-// layout is that of the 32x32 fp8 MFMA above.
+// layout is that of the 32x32 fp8 MFMA above.  run16 is the 16x16x32 shape: lane l supplies row/col l%16, k = 8*(l/16)
+// .. +7, and receives D[4*(l/16) + r][l%16], r = 0..3.
 template <bool BF>
 struct Mfma16;
 template <>
@@ -72,12 +73,14 @@ struct Mfma16<true> {
   typedef __bf16 T;
   typedef v8bf V8;
   static __device__ __forceinline__ v16f run(v8bf a, v8bf b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ v4f run16(v8bf a, v8bf b, v4f c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
 };
 template <>
 struct Mfma16<false> {
   typedef _Float16 T;
   typedef v8h V8;
   static __device__ __forceinline__ v16f run(v8h a, v8h b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ v4f run16(v8h a, v8h b, v4f c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
 };
 
 template <int OUT>
