@@ -225,17 +225,26 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restri
   for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
     for (int f = 0; f < 16; ++f) load_frag(fa[ks], fw[ks], 0, ks, f);
+  constexpr bool EARLY = MODE == 0;
+  if (EARLY) __syncthreads();  // ... of stage 0
   for (int kt = 0; kt < nk; ++kt) {
     const int stage = kt & 1, dkt = min(kt + 2, nk - 1);
-    mfma_ks(0, [](int) {});
-    HX_WAIT_VM0();
+    // EARLY (grouped mode): a second barrier at the end of the tile frees the stage a half tile sooner, so the DMA of
+    // tile kt+2 goes out under the first half and has a whole tile to land (C5 -1 %; given the same structure the
+    // dense instantiations compile with accumulator copies inside the loop and run slower).
+    mfma_ks(0, [&](int i) {
+      if (EARLY && (i & 3) == 3) issue_one(dkt, stage, i >> 2);
+    });
+    if (EARLY) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(16));  // tile kt+1, issued a tile ago, has landed; tile kt+2 stays in flight
+    else HX_WAIT_VM0();
     __syncthreads();
     mfma_ks(1, [&](int i) {
       if (i < 32 && !(i & 1)) load_frag(fa[0], fw[0], stage ^ 1, 0, i >> 1);
-      if ((i & 3) == 3) issue_one(dkt, stage, i >> 2);
+      if (!EARLY && (i & 3) == 3) issue_one(dkt, stage, i >> 2);
       if ((i & 7) == 7) load_frag(fa[1], fw[1], stage ^ 1, 1, 8 + (i >> 3));  // W fragment i>>3: its eight MFMAs are out
       if (i >= 56) load_frag(fa[1], fw[1], stage ^ 1, 1, i - 56);              // A fragment i-56: last used by MFMA i
     });
+    if (EARLY) __syncthreads();  // every wave has read tile kt+1's fragments out of the other stage: it is free
   }
   HX_WAIT_VM0();  // trailing re-fetches must land before the workgroup's LDS is released
 
