@@ -197,6 +197,10 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
         if (r >= ktail) *(v4i*)(&smem[stage][1][0] + r * 256 + (lane & 15) * 16) = z;
   };
   const bool has_tail = EDGE && ktail != T256_BK;
+  // EARLY (full tiles of a K-contiguous B): all sixteen fragments of the next tile are fetched in the second half, a
+  // second barrier at the end of the tile frees this tile's stage a half tile sooner, and the DMA of tile kt+2 goes out
+  // under the first half: it has a whole tile to land instead of half of one.
+  constexpr bool EARLY = !EDGE && !BROW;
   v8i fa[8], fb[8];
   auto ktile = [&](int kt, auto with_dma) {
     constexpr bool dma = decltype(with_dma)::value;
@@ -204,11 +208,13 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
       const int bi = i >> 2, bj = i & 3;
-      if ((i & 7) == 0) load_b(fb[4 + (i >> 3)], stage, 4 + (i >> 3));
+      if (!EARLY && (i & 7) == 0) load_b(fb[4 + (i >> 3)], stage, 4 + (i >> 3));
       acc[bj][bi] = hx_mfma_16x16x128_e4m3(fb[bj], fa[bi], acc[bj][bi]);
+      if (EARLY && (i & 1) && dma) issue_one(kt + 2, stage, i >> 1);
       __builtin_amdgcn_sched_barrier(0);
     }
-    HX_WAIT_VM0();
+    if (EARLY && dma) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(16));  // tile kt+1 has landed; tile kt+2 stays in flight
+    else HX_WAIT_VM0();
     // the last tile has just landed in the other stage.  (Only in the copy of the loop that runs the last two tiles:
     // with this branch in the main loop the compiler moves the accumulators around it, one move per MFMA.)
     if (!dma && has_tail && kt == nk - 2) zero_tail(stage ^ 1);
@@ -219,9 +225,11 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
       acc[bj][bi] = hx_mfma_16x16x128_e4m3(fb[bj], fa[bi], acc[bj][bi]);
       if ((i & 3) == 3) load_a(fa[bi], stage ^ 1, bi);
       if ((i & 7) == 1) load_b(fb[i >> 3], stage ^ 1, i >> 3);
-      if ((i & 1) && dma) issue_one(kt + 2, stage, i >> 1);
+      if (EARLY && i >= 28) load_b(fb[4 + (i - 28)], stage ^ 1, 4 + (i - 28));  // its last MFMA of this tile is out
+      if (!EARLY && (i & 1) && dma) issue_one(kt + 2, stage, i >> 1);
       __builtin_amdgcn_sched_barrier(0);
     }
+    if (EARLY) __syncthreads();  // every wave has read tile kt+1's fragments out of the other stage: it is free
   };
   issue(0, 0);
   if (nk > 1) issue(1, 1);
@@ -231,7 +239,8 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
 #pragma unroll
   for (int f = 0; f < 8; ++f) load_a(fa[f], 0, f);
 #pragma unroll
-  for (int f = 0; f < 4; ++f) load_b(fb[f], 0, f);
+  for (int f = 0; f < (EARLY ? 8 : 4); ++f) load_b(fb[f], 0, f);
+  if (EARLY) __syncthreads();  // ... of stage 0
   int kt = 0;
   for (; kt + 2 < nk; ++kt) ktile(kt, std::true_type{});
   for (; kt < nk; ++kt) ktile(kt, std::false_type{});  // the last two k-tiles have nothing left to fetch
