@@ -230,8 +230,8 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restri
   for (int kt = 0; kt < nk; ++kt) {
     const int stage = kt & 1, dkt = min(kt + 2, nk - 1);
     // EARLY (grouped mode): a second barrier at the end of the tile frees the stage a half tile sooner, so the DMA of
-    // tile kt+2 goes out under the first half and has a whole tile to land (C5 -1 %; given the same structure the
-    // dense instantiations compile with accumulator copies inside the loop and run slower).
+    // tile kt+2 goes out under the first half and has a whole tile to land (C5 -1 %; the dense instantiations
+    // measured 1-2 % slower with it, and those with an epilogue then compile with accumulator copies inside the loop).
     mfma_ks(0, [&](int i) {
       if (EARLY && (i & 3) == 3) issue_one(dkt, stage, i >> 2);
     });
