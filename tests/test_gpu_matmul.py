@@ -111,6 +111,22 @@ def test_split_k_vs_oracle(m, k, n, dtype):
     assert rel_err(lam, orc.matmul(x, y, bias)) <= 1e-2
 
 
+@pytest.mark.parametrize("m,k,n", [(3072, 256, 3072), (3000, 192, 3080)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_split_k_on_the_256_tile_kernel(m, k, n, dtype):
+    """More than 128 tiles of 256 x 256: an explicit split_k then runs the 256 x 256 kernel's fp32 partial-sum mode
+    (full and ragged edge tiles, row-major and column-major W), the reduction adds the epilogue."""
+    x, y, bias = _mk(m, k, n, dtype, m + k + n)
+    xd, yd, bd = x.to(DEV), y.to(DEV), bias.to(DEV)
+    ref = orc.matmul(x, y)
+    refb = orc.matmul(x, y, bias, relu=True)
+    for yy in (yd, yd.t().contiguous().t()):
+        out = hx.matmul_split_k(xd, yy, split_k=2)
+        assert out.dtype == dtype and rel_err(out, ref) <= 1e-2
+        assert rel_err(hx.matmul_split_k(xd, yy, bias_relu(bd), split_k=3), refb) <= 1e-2
+        assert torch.equal(out, hx.matmul_split_k(xd, yy, split_k=2))
+
+
 def test_strided_operands_and_tritonbench_wrappers():
     x, y, bias = _mk(300, 256, 264, torch.bfloat16, 11)
     xd, yd, bd = x.to(DEV), y.to(DEV), bias.to(DEV)
