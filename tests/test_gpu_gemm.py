@@ -23,7 +23,7 @@ def _path(m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k,path", [
-    (4096, 4096, 128, 1), (2048, 6144, 256, 1),                                                      # enough full 256x256 tiles
+    (4096, 4096, 128, 1), (2048, 6144, 256, 1), (4096, 2048, 384, 1), (2048, 4096, 640, 1),          # enough full 256x256 tiles; 1, 2, 3, 5 k-tiles
     (256, 256, 256, 5), (512, 512, 512, 5), (1024, 1024, 1024, 5), (256, 768, 128, 5), (768, 256, 1152, 5),   # too few: 128-column tiles
     (64, 28672, 256, 5), (128, 40000, 128, 5), (90, 20000, 128, 5),      # one row tile: column pitch 112 / 128 / 80
     (48, 1024, 512, 5), (100, 3000, 256, 5), (129, 520, 384, 5), (256, 1000, 128, 5), (200, 136, 1280, 5), (33, 256, 256, 5),
