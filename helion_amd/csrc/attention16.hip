@@ -391,10 +391,10 @@ static void launch_att16(const void* q, const void* k, const void* v, void* out,
   const int qtiles = (int)((M + A16_BM - 1) / A16_BM);
   const int hpx = (int)((BH + 7) / 8);
   if (N % A16_BN)
-    hipLaunchKernelGGL((hx_attention16_kernel<D, BF, true>), dim3(8 * hpx * qtiles), dim3(64 * A16_WAVES), 0, s, (const uint8_t*)q,
+    hx_launch((hx_attention16_kernel<D, BF, true>), dim3(8 * hpx * qtiles), dim3(64 * A16_WAVES), 0, s, (const uint8_t*)q,
                        (const uint8_t*)k, (const uint8_t*)v, out, (int)M, (int)N, (int)BH, qtiles, c);
   else
-    hipLaunchKernelGGL((hx_attention16_kernel<D, BF, false>), dim3(8 * hpx * qtiles), dim3(64 * A16_WAVES), 0, s, (const uint8_t*)q,
+    hx_launch((hx_attention16_kernel<D, BF, false>), dim3(8 * hpx * qtiles), dim3(64 * A16_WAVES), 0, s, (const uint8_t*)q,
                        (const uint8_t*)k, (const uint8_t*)v, out, (int)M, (int)N, (int)BH, qtiles, c);
 }
 
@@ -444,16 +444,16 @@ extern "C" int hx_attention(const void* q, const void* k, const void* v, void* o
     }
     const dim3 grid((unsigned)M, (unsigned)BH);
     if (dtype == HX_BF16)
-      hipLaunchKernelGGL(hx_attention_general<__bf16>, grid, dim3(256), 0, s, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
+      hx_launch(hx_attention_general<__bf16>, grid, dim3(256), 0, s, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
                          (__bf16*)out, (int)M, (int)N, (int)D, c);
     else if (dtype == HX_F16)
-      hipLaunchKernelGGL(hx_attention_general<_Float16>, grid, dim3(256), 0, s, (const _Float16*)q, (const _Float16*)k,
+      hx_launch(hx_attention_general<_Float16>, grid, dim3(256), 0, s, (const _Float16*)q, (const _Float16*)k,
                          (const _Float16*)v, (_Float16*)out, (int)M, (int)N, (int)D, c);
     else
-      hipLaunchKernelGGL(hx_attention_general<float>, grid, dim3(256), 0, s, (const float*)q, (const float*)k, (const float*)v,
+      hx_launch(hx_attention_general<float>, grid, dim3(256), 0, s, (const float*)q, (const float*)k, (const float*)v,
                          (float*)out, (int)M, (int)N, (int)D, c);
   }
-  hipError_t e = hipGetLastError();
+  hipError_t e = hx_launch_status();
   if (e != hipSuccess) {
     hx_set_error("hx_attention: launch failed: %s", hipGetErrorString(e));
     return (int)e;

@@ -425,7 +425,7 @@ static void launch_att_kernel(const void* q, const void* k, const void* v, void*
   const int qtiles = (int)((S + ATT_BM - 1) / ATT_BM);
   const int hpx = (int)((BH + 7) / 8);
   const int grid = 8 * hpx * qtiles;
-  hipLaunchKernelGGL((hx_fp8_attention_kernel<D, OUT, EXACT, VSD>), dim3(grid), dim3(256), 0, s, (const uint8_t*)q, (const uint8_t*)k,
+  hx_launch((hx_fp8_attention_kernel<D, OUT, EXACT, VSD>), dim3(grid), dim3(256), 0, s, (const uint8_t*)q, (const uint8_t*)k,
                      (const uint8_t*)v, out, (int)S, (int)BH, qtiles, c);
 }
 
@@ -438,7 +438,7 @@ static int launch_att(const void* q, const void* k, const void* v, void* out, in
     if (vsd) launch_att_kernel<D, OUT, false, true>(q, k, v, out, BH, S, c, s);
     else launch_att_kernel<D, OUT, false, false>(q, k, v, out, BH, S, c, s);
   }
-  hipError_t e = hipGetLastError();
+  hipError_t e = hx_launch_status();
   if (e != hipSuccess) {
     hx_set_error("hx_fp8_attention: launch failed: %s", hipGetErrorString(e));
     return (int)e;
@@ -481,12 +481,12 @@ extern "C" int hx_fp8_attention(const void* q, const void* k, const void* v, voi
     }
     const dim3 grid((unsigned)S, (unsigned)BH);
     if (out_dtype == HX_F32)
-      hipLaunchKernelGGL(hx_fp8_attention_general<HX_F32>, grid, dim3(256), 0, s, (const uint8_t*)q, (const uint8_t*)k, (const uint8_t*)v,
+      hx_launch(hx_fp8_attention_general<HX_F32>, grid, dim3(256), 0, s, (const uint8_t*)q, (const uint8_t*)k, (const uint8_t*)v,
                          out, (int)S, (int)D, (long)v_stride_d, (long)v_stride_s, c);
     else
-      hipLaunchKernelGGL(hx_fp8_attention_general<HX_E4M3>, grid, dim3(256), 0, s, (const uint8_t*)q, (const uint8_t*)k,
+      hx_launch(hx_fp8_attention_general<HX_E4M3>, grid, dim3(256), 0, s, (const uint8_t*)q, (const uint8_t*)k,
                          (const uint8_t*)v, out, (int)S, (int)D, (long)v_stride_d, (long)v_stride_s, c);
-    hipError_t e = hipGetLastError();
+    hipError_t e = hx_launch_status();
     if (e != hipSuccess) {
       hx_set_error("hx_fp8_attention: launch failed: %s", hipGetErrorString(e));
       return (int)e;

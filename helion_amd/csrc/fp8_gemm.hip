@@ -908,11 +908,11 @@ static void launch_kmajor(int path, const void* a, const void* bt, void* c, int6
     const int tiles_m = (int)((M + 255) / 256), tiles_n = (int)((N + 255) / 256);
     const bool edge = (M % 256 != 0) || (N % 256 != 0) || (K % 128 != 0) || (ldc % 8 != 0) || !aligned(c, 16);
     if (!edge)
-      hipLaunchKernelGGL((hx_fp8_gemm_tile256<OUT, false, true>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
+      hx_launch((hx_fp8_gemm_tile256<OUT, false, true>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
                          (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m,
                          tiles_n);
     else
-      hipLaunchKernelGGL((hx_fp8_gemm_tile256<OUT, true, true>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
+      hx_launch((hx_fp8_gemm_tile256<OUT, true, true>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
                          (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m,
                          tiles_n);
   } else if (path == 5) {
@@ -927,35 +927,35 @@ static void launch_kmajor(int path, const void* a, const void* bt, void* c, int6
     if (split) {
       float* part = (float*)ws;
       if (bm == 64)
-        hipLaunchKernelGGL((hx_fp8_gemm_tileN128<HX_F32, 64, true>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
+        hx_launch((hx_fp8_gemm_tileN128<HX_F32, 64, true>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
                            part, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)N, nullptr, nullptr, tiles_m, bn, ktps);
       else if (bm == 256)
-        hipLaunchKernelGGL((hx_fp8_gemm_tileN128<HX_F32, 256>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt, part,
+        hx_launch((hx_fp8_gemm_tileN128<HX_F32, 256>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt, part,
                            (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)N, nullptr, nullptr, tiles_m, bn, ktps);
       else
-        hipLaunchKernelGGL((hx_fp8_gemm_tileN128<HX_F32, 128>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt, part,
+        hx_launch((hx_fp8_gemm_tileN128<HX_F32, 128>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt, part,
                            (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)N, nullptr, nullptr, tiles_m, bn, ktps);
       const long quads = (long)M * ((N + 3) / 4);
-      hipLaunchKernelGGL((hx_fp8_gemm_split_reduce<OUT>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream,
+      hx_launch((hx_fp8_gemm_split_reduce<OUT>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream,
                          (const float*)part, (out_t*)c, (int)M, (int)N, (long)ldc, splits, sa, sb);
     } else if (bm == 64) {
-      hipLaunchKernelGGL((hx_fp8_gemm_tileN128<OUT, 64, true>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
+      hx_launch((hx_fp8_gemm_tileN128<OUT, 64, true>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
                          (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m, bn, 0);
     } else if (bm == 256) {
-      hipLaunchKernelGGL((hx_fp8_gemm_tileN128<OUT, 256>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
+      hx_launch((hx_fp8_gemm_tileN128<OUT, 256>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
                          (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m, bn, 0);
     } else {
-      hipLaunchKernelGGL((hx_fp8_gemm_tileN128<OUT, 128>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
+      hx_launch((hx_fp8_gemm_tileN128<OUT, 128>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
                          (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m, bn, 0);
     }
   } else if (path == 1 || path == 3) {
     const int tiles_m = (int)((M + 255) / 256), tiles_n = (int)((N + 255) / 256);
     if (path == 1)
-      hipLaunchKernelGGL((hx_fp8_gemm_tile256<OUT, false, false>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
+      hx_launch((hx_fp8_gemm_tile256<OUT, false, false>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
                          (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m,
                          tiles_n);
     else
-      hipLaunchKernelGGL((hx_fp8_gemm_tile256<OUT, true, false>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
+      hx_launch((hx_fp8_gemm_tile256<OUT, true, false>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
                          (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m,
                          tiles_n);
   } else {  // path == 2
@@ -965,19 +965,19 @@ static void launch_kmajor(int path, const void* a, const void* bt, void* c, int6
     const int ncg = (int)((N + 15) / 16);
     const int grid = ncg < cus ? ncg : cus;
     if (K == 8192 && M <= 16)
-      hipLaunchKernelGGL((hx_fp8_gemm_skinny_direct<OUT, true, 1>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
+      hx_launch((hx_fp8_gemm_skinny_direct<OUT, true, 1>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
                          (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb);
     else if (K == 8192)
-      hipLaunchKernelGGL((hx_fp8_gemm_skinny_direct<OUT, true, 2>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
+      hx_launch((hx_fp8_gemm_skinny_direct<OUT, true, 2>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
                          (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb);
     else if (K < 8192 && M <= 16)
-      hipLaunchKernelGGL((hx_fp8_gemm_skinny_direct<OUT, false, 1>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
+      hx_launch((hx_fp8_gemm_skinny_direct<OUT, false, 1>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
                          (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb);
     else if (K < 8192)
-      hipLaunchKernelGGL((hx_fp8_gemm_skinny_direct<OUT, false, 2>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
+      hx_launch((hx_fp8_gemm_skinny_direct<OUT, false, 2>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
                          (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb);
     else
-      hipLaunchKernelGGL(hx_fp8_gemm_skinny<OUT>, dim3(grid), dim3(512), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
+      hx_launch(hx_fp8_gemm_skinny<OUT>, dim3(grid), dim3(512), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
                          (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb);
   }
 }
@@ -997,15 +997,15 @@ static int launch_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int
       tpath = gemm_path_kmajor(M, N, K, lda, K, ldc, a, ws, c);
     if (tpath != 0) {
       dim3 tg((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64));
-      hipLaunchKernelGGL(hx_transpose_u8, tg, dim3(256), 0, stream, (const uint8_t*)b, (uint8_t*)ws, (int)K, (int)N, (long)ldb_k);
+      hx_launch(hx_transpose_u8, tg, dim3(256), 0, stream, (const uint8_t*)b, (uint8_t*)ws, (int)K, (int)N, (long)ldb_k);
       launch_kmajor<OUT>(tpath, a, ws, c, M, N, K, lda, K, ldc, sa, sb, nullptr, 0, stream);
     } else {
       dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
-      hipLaunchKernelGGL(hx_fp8_gemm_general<OUT>, grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)b, (out_t*)c,
+      hx_launch(hx_fp8_gemm_general<OUT>, grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)b, (out_t*)c,
                          (int)M, (int)N, (int)K, (long)lda, (long)ldb_k, (long)ldb_n, (long)ldc, sa, sb);
     }
   }
-  hipError_t e = hipGetLastError();
+  hipError_t e = hx_launch_status();
   if (e != hipSuccess) {
     hx_set_error("hx_fp8_gemm: launch failed: %s", hipGetErrorString(e));
     return (int)e;

@@ -152,10 +152,10 @@ static int qz_grid(long long n) {
 
 static int qz_launch_cast(const QzJobs& jobs, int njobs, long long nmax_, int dt, const float* mul, hipStream_t s) {
   dim3 grid((unsigned)qz_grid(nmax_), (unsigned)njobs);
-  if (dt == HX_F16) hipLaunchKernelGGL(hx_cast_e4m3_kernel<HX_F16>, grid, dim3(QZ_THREADS), 0, s, jobs, mul);
-  else if (dt == HX_BF16) hipLaunchKernelGGL(hx_cast_e4m3_kernel<HX_BF16>, grid, dim3(QZ_THREADS), 0, s, jobs, mul);
-  else hipLaunchKernelGGL(hx_cast_e4m3_kernel<HX_F32>, grid, dim3(QZ_THREADS), 0, s, jobs, mul);
-  hipError_t e = hipGetLastError();
+  if (dt == HX_F16) hx_launch(hx_cast_e4m3_kernel<HX_F16>, grid, dim3(QZ_THREADS), 0, s, jobs, mul);
+  else if (dt == HX_BF16) hx_launch(hx_cast_e4m3_kernel<HX_BF16>, grid, dim3(QZ_THREADS), 0, s, jobs, mul);
+  else hx_launch(hx_cast_e4m3_kernel<HX_F32>, grid, dim3(QZ_THREADS), 0, s, jobs, mul);
+  hipError_t e = hx_launch_status();
   if (e != hipSuccess) {
     hx_set_error("fp8 cast: launch failed: %s", hipGetErrorString(e));
     return (int)e;
@@ -223,11 +223,11 @@ extern "C" int hx_fp8_quantize(const void* src, void* dst, int64_t n, int src_dt
   float* triple = (float*)workspace;
   float* partial = triple + 4;
   const int blocks = qz_grid(n);
-  if (src_dtype == HX_F16) hipLaunchKernelGGL(hx_amax_partial_kernel<HX_F16>, dim3(blocks), dim3(QZ_THREADS), 0, s, src, (long long)n, partial);
-  else if (src_dtype == HX_BF16) hipLaunchKernelGGL(hx_amax_partial_kernel<HX_BF16>, dim3(blocks), dim3(QZ_THREADS), 0, s, src, (long long)n, partial);
-  else hipLaunchKernelGGL(hx_amax_partial_kernel<HX_F32>, dim3(blocks), dim3(QZ_THREADS), 0, s, src, (long long)n, partial);
-  hipLaunchKernelGGL(hx_amax_final_kernel, dim3(1), dim3(QZ_THREADS), 0, s, (const float*)partial, blocks, triple, scale_out);
-  hipError_t e = hipGetLastError();
+  if (src_dtype == HX_F16) hx_launch(hx_amax_partial_kernel<HX_F16>, dim3(blocks), dim3(QZ_THREADS), 0, s, src, (long long)n, partial);
+  else if (src_dtype == HX_BF16) hx_launch(hx_amax_partial_kernel<HX_BF16>, dim3(blocks), dim3(QZ_THREADS), 0, s, src, (long long)n, partial);
+  else hx_launch(hx_amax_partial_kernel<HX_F32>, dim3(blocks), dim3(QZ_THREADS), 0, s, src, (long long)n, partial);
+  hx_launch(hx_amax_final_kernel, dim3(1), dim3(QZ_THREADS), 0, s, (const float*)partial, blocks, triple, scale_out);
+  hipError_t e = hx_launch_status();
   if (e != hipSuccess) {
     hx_set_error("hx_fp8_quantize: launch failed: %s", hipGetErrorString(e));
     return (int)e;

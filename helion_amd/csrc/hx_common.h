@@ -4,6 +4,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <tuple>
+#include <utility>
+
 #include "../../include/hx_kernels.h"
 
 typedef int v8i __attribute__((ext_vector_type(8)));
@@ -106,3 +109,27 @@ __device__ __forceinline__ float hx_e4m3_to_f32(uint8_t code) {
 }
 
 void hx_set_error(const char* fmt, ...);
+
+// Kernel launches go through hipLaunchKernel, whose own return code is the launch's status: the library never
+// reads (and so never clears) the caller's sticky HIP error state, and a foreign earlier error is never
+// attributed to one of its calls.  hx_launch records the first failure of the calling thread's current entry
+// point; hx_launch_status() returns it and resets the record (every entry point ends with it).
+inline thread_local hipError_t hx_tls_launch_err = hipSuccess;
+template <typename... KArgs, typename... Args, size_t... I>
+static inline hipError_t hx_launch_impl(void (*kernel)(KArgs...), dim3 grid, dim3 block, unsigned shmem, hipStream_t s,
+                                        std::index_sequence<I...>, Args&&... args) {
+  std::tuple<KArgs...> vals{static_cast<KArgs>(args)...};
+  void* ptrs[] = {(void*)&std::get<I>(vals)..., nullptr};
+  return hipLaunchKernel((const void*)kernel, grid, block, ptrs, shmem, s);
+}
+template <typename... KArgs, typename... Args>
+static inline void hx_launch(void (*kernel)(KArgs...), dim3 grid, dim3 block, unsigned shmem, hipStream_t s, Args&&... args) {
+  static_assert(sizeof...(KArgs) == sizeof...(Args), "hx_launch: argument count does not match the kernel's");
+  const hipError_t e = hx_launch_impl(kernel, grid, block, shmem, s, std::index_sequence_for<KArgs...>{}, std::forward<Args>(args)...);
+  if (e != hipSuccess && hx_tls_launch_err == hipSuccess) hx_tls_launch_err = e;
+}
+static inline hipError_t hx_launch_status() {
+  const hipError_t e = hx_tls_launch_err;
+  hx_tls_launch_err = hipSuccess;
+  return e;
+}

@@ -159,7 +159,7 @@ template <typename TI, typename TO>
 static void mm_launch_general(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k,
                               int64_t ldb_n, int64_t ldc, const void* bias, int bias_f32, int relu, hipStream_t s) {
   dim3 grid((unsigned)((M + 63) / 64), (unsigned)((N + 63) / 64));
-  hipLaunchKernelGGL((hx_matmul_general<TI, TO>), grid, dim3(256), 0, s, (const TI*)a, (const TI*)b, (TO*)c, (int)M, (int)N, (int)K,
+  hx_launch((hx_matmul_general<TI, TO>), grid, dim3(256), 0, s, (const TI*)a, (const TI*)b, (TO*)c, (int)M, (int)N, (int)K,
                      (long)lda, (long)ldb_k, (long)ldb_n, (long)ldc, bias, bias_f32, relu);
 }
 
@@ -175,14 +175,14 @@ static void mm_launch_fast(const void* a, const void* b, void* c, int64_t M, int
   if (!partial && out_dtype != HX_F32) {
     d.ldc = ldc;
     if (tile == 256)
-      hipLaunchKernelGGL((hx_gemm16_tile256<BF, 1, BCOL>), dim3(tiles_m * tiles_n), dim3(256), 0, s, (const uint8_t*)a, (const uint8_t*)b, c,
+      hx_launch((hx_gemm16_tile256<BF, 1, BCOL>), dim3(tiles_m * tiles_n), dim3(256), 0, s, (const uint8_t*)a, (const uint8_t*)b, c,
                          (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M, (int)K, (int)N, tiles_m, tiles_n, 1, d);
     else if (tiles_m * tiles_n <= 256)
-      hipLaunchKernelGGL((hx_gemm16_tile128<BF, 1, BCOL, 4>), dim3(tiles_m * tiles_n), dim3(256), 0, s, (const uint8_t*)a, (const uint8_t*)b,
+      hx_launch((hx_gemm16_tile128<BF, 1, BCOL, 4>), dim3(tiles_m * tiles_n), dim3(256), 0, s, (const uint8_t*)a, (const uint8_t*)b,
                          c, (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M, (int)K, (int)N, tiles_m, tiles_n, 1,
                          d);
     else
-      hipLaunchKernelGGL((hx_gemm16_tile128<BF, 1, BCOL, 2>), dim3(tiles_m * tiles_n), dim3(256), 0, s, (const uint8_t*)a, (const uint8_t*)b,
+      hx_launch((hx_gemm16_tile128<BF, 1, BCOL, 2>), dim3(tiles_m * tiles_n), dim3(256), 0, s, (const uint8_t*)a, (const uint8_t*)b,
                          c, (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M, (int)K, (int)N, tiles_m, tiles_n, 1,
                          d);
     return;
@@ -191,25 +191,25 @@ static void mm_launch_fast(const void* a, const void* b, void* c, int64_t M, int
   d.kt_per_split = (nkt + splits - 1) / splits;
   d.ldc = partial ? N : ldc;
   if (tile == 256)
-    hipLaunchKernelGGL((hx_gemm16_tile256<BF, 2, BCOL>), dim3(tiles_m * tiles_n, splits), dim3(256), 0, s, (const uint8_t*)a,
+    hx_launch((hx_gemm16_tile256<BF, 2, BCOL>), dim3(tiles_m * tiles_n, splits), dim3(256), 0, s, (const uint8_t*)a,
                        (const uint8_t*)b, partial ? ws : c, (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M,
                        (int)K, (int)N, tiles_m, tiles_n, 1, d);
   else if ((long)tiles_m * tiles_n * splits <= 256)
-    hipLaunchKernelGGL((hx_gemm16_tile128<BF, 2, BCOL, 4>), dim3(tiles_m * tiles_n, splits), dim3(256), 0, s, (const uint8_t*)a,
+    hx_launch((hx_gemm16_tile128<BF, 2, BCOL, 4>), dim3(tiles_m * tiles_n, splits), dim3(256), 0, s, (const uint8_t*)a,
                        (const uint8_t*)b, partial ? ws : c, (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M,
                        (int)K, (int)N, tiles_m, tiles_n, 1, d);
   else
-    hipLaunchKernelGGL((hx_gemm16_tile128<BF, 2, BCOL, 2>), dim3(tiles_m * tiles_n, splits), dim3(256), 0, s, (const uint8_t*)a,
+    hx_launch((hx_gemm16_tile128<BF, 2, BCOL, 2>), dim3(tiles_m * tiles_n, splits), dim3(256), 0, s, (const uint8_t*)a,
                        (const uint8_t*)b, partial ? ws : c, (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M,
                        (int)K, (int)N, tiles_m, tiles_n, 1, d);
   if (!partial) return;
   const long groups = M * (N / 4);
   const dim3 grid((unsigned)((groups + 15) / 16));
   if (out_dtype == HX_F32)
-    hipLaunchKernelGGL((hx_matmul16_reduce<T16, float>), grid, dim3(256), 0, s, (const float*)ws, splits, (int)M, (int)N, (float*)c, (long)ldc,
+    hx_launch((hx_matmul16_reduce<T16, float>), grid, dim3(256), 0, s, (const float*)ws, splits, (int)M, (int)N, (float*)c, (long)ldc,
                        bias, bias_f32, relu);
   else
-    hipLaunchKernelGGL((hx_matmul16_reduce<T16, T16>), grid, dim3(256), 0, s, (const float*)ws, splits, (int)M, (int)N, (T16*)c, (long)ldc,
+    hx_launch((hx_matmul16_reduce<T16, T16>), grid, dim3(256), 0, s, (const float*)ws, splits, (int)M, (int)N, (T16*)c, (long)ldc,
                        bias, bias_f32, relu);
 }
 
@@ -284,7 +284,7 @@ extern "C" int hx_matmul(const void* a, const void* b, void* c, int64_t M, int64
     if (out_dtype == HX_F32) mm_launch_general<_Float16, float>(a, b, c, M, N, K, lda, ldb_k, ldb_n, ldc, bias, bias_f32, relu, s);
     else mm_launch_general<_Float16, _Float16>(a, b, c, M, N, K, lda, ldb_k, ldb_n, ldc, bias, bias_f32, relu, s);
   }
-  hipError_t e = hipGetLastError();
+  hipError_t e = hx_launch_status();
   if (e != hipSuccess) {
     hx_set_error("hx_matmul: launch failed: %s", hipGetErrorString(e));
     return (int)e;

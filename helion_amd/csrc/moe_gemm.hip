@@ -229,13 +229,13 @@ static int launch_moe(const void* A, const void* W, void* C, const int32_t* coun
   uint8_t* flags = (uint8_t*)ws + tb;
 
   if (E <= 1024 && T <= 4096) {
-    hipLaunchKernelGGL(hx_moe_prep_mark_small, dim3(1), dim3(1024), 0, s, counts, offsets, idx, (int)E, (int)T, bm, max_tiles, num_tiles,
+    hx_launch(hx_moe_prep_mark_small, dim3(1), dim3(1024), 0, s, counts, offsets, idx, (int)E, (int)T, bm, max_tiles, num_tiles,
                        table, flags);
   } else {
     const int prep_blocks = (int)((T + 256 * 64 - 1) / (256 * 64)) + 1;
-    hipLaunchKernelGGL(hx_moe_prep, dim3(prep_blocks), dim3(256), 0, s, counts, offsets, (int)E, (int)T, bm, max_tiles, num_tiles, table,
+    hx_launch(hx_moe_prep, dim3(prep_blocks), dim3(256), 0, s, counts, offsets, (int)E, (int)T, bm, max_tiles, num_tiles, table,
                        flags);
-    hipLaunchKernelGGL(hx_moe_mark, dim3(max_tiles < 1024 ? max_tiles : 1024), dim3(256), 0, s, (const int*)num_tiles,
+    hx_launch(hx_moe_mark, dim3(max_tiles < 1024 ? max_tiles : 1024), dim3(256), 0, s, (const int*)num_tiles,
                        (const MoeTile*)table, idx, (int)T, flags);
   }
   if (fast) {
@@ -243,28 +243,28 @@ static int launch_moe(const void* A, const void* W, void* C, const int32_t* coun
     d.lda = K; d.ldb = N; d.ldc = N;
     if (bm == R32_BM) {
       const int tiles_n = (int)((N + R32_BN - 1) / R32_BN);
-      hipLaunchKernelGGL((hx_gemm16_rows32<BF, 3>), dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W,
+      hx_launch((hx_gemm16_rows32<BF, 3>), dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W,
                          (void*)C, (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, max_tiles, tiles_n,
                          (int)a_div, d);
     } else if (bm == MOE_BM) {
       const int tiles_n = (int)tn256;
-      hipLaunchKernelGGL((hx_gemm16_tile256<BF, 0>), dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W,
+      hx_launch((hx_gemm16_tile256<BF, 0>), dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W,
                          (void*)C, (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, max_tiles, tiles_n,
                          (int)a_div, d);
     } else {
       const int tiles_n = (int)((N + G128_BN - 1) / G128_BN);
-      hipLaunchKernelGGL((hx_gemm16_tile128<BF, 0>), dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W,
+      hx_launch((hx_gemm16_tile128<BF, 0>), dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W,
                          (void*)C, (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, max_tiles, tiles_n,
                          (int)a_div, d);
     }
   } else {
     dim3 grid((unsigned)max_tiles, (unsigned)((N + 63) / 64));
-    hipLaunchKernelGGL(hx_moe_general<T16>, grid, dim3(256), 0, s, (const T16*)A, (const T16*)W, (T16*)C, (const int*)num_tiles,
+    hx_launch(hx_moe_general<T16>, grid, dim3(256), 0, s, (const T16*)A, (const T16*)W, (T16*)C, (const int*)num_tiles,
                        (const MoeTile*)table, idx, (int)T, (int)K, (int)N, (int)a_div);
   }
-  hipLaunchKernelGGL(hx_moe_zero_rows<T16>, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, s, (T16*)C, (long)N, (int)T, (int)N,
+  hx_launch(hx_moe_zero_rows<T16>, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, s, (T16*)C, (long)N, (int)T, (int)N,
                      (const uint8_t*)flags);
-  hipError_t e = hipGetLastError();
+  hipError_t e = hx_launch_status();
   if (e != hipSuccess) {
     hx_set_error("hx_moe_grouped_gemm: launch failed: %s", hipGetErrorString(e));
     return (int)e;

@@ -231,17 +231,17 @@ static void rt_launch(const IdT* ids, int64_t T, int64_t E, int nbits, int32_t* 
   const size_t need = hx_moe_routing_workspace_bytes(T, E);
   if (need == 0 || !ws || ws_bytes < need) {
     const int block_rows = (int)((((T + RT_WAVES - 1) / RT_WAVES + 63) & ~(int64_t)63) * RT_WAVES);
-    hipLaunchKernelGGL((hx_moe_routing_kernel<IdT, 0>), dim3(1), dim3(64 * RT_WAVES), 0, s, ids, (int)T, (int)E, nbits,
+    hx_launch((hx_moe_routing_kernel<IdT, 0>), dim3(1), dim3(64 * RT_WAVES), 0, s, ids, (int)T, (int)E, nbits,
                        block_rows > 0 ? block_rows : 64 * RT_WAVES, counts, offsets, idx, max_count, (int32_t*)nullptr);
     return;
   }
   int64_t br, nb;
   rt_blocks(T, &br, &nb);
   int32_t* tab = (int32_t*)ws;
-  hipLaunchKernelGGL((hx_moe_routing_kernel<IdT, 1>), dim3((unsigned)nb), dim3(64 * RT_WAVES), 0, s, ids, (int)T, (int)E, nbits, (int)br,
+  hx_launch((hx_moe_routing_kernel<IdT, 1>), dim3((unsigned)nb), dim3(64 * RT_WAVES), 0, s, ids, (int)T, (int)E, nbits, (int)br,
                      counts, offsets, idx, max_count, tab);
-  hipLaunchKernelGGL(hx_moe_routing_scan, dim3(1), dim3(RT_MAX_E), 0, s, tab, (int)nb, (int)E, counts, offsets, max_count);
-  hipLaunchKernelGGL((hx_moe_routing_kernel<IdT, 2>), dim3((unsigned)nb), dim3(64 * RT_WAVES), 0, s, ids, (int)T, (int)E, nbits, (int)br,
+  hx_launch(hx_moe_routing_scan, dim3(1), dim3(RT_MAX_E), 0, s, tab, (int)nb, (int)E, counts, offsets, max_count);
+  hx_launch((hx_moe_routing_kernel<IdT, 2>), dim3((unsigned)nb), dim3(64 * RT_WAVES), 0, s, ids, (int)T, (int)E, nbits, (int)br,
                      counts, offsets, idx, max_count, tab);
 }
 
@@ -268,7 +268,7 @@ extern "C" int hx_moe_routing(const void* expert_ids, int ids_are_int64, int64_t
   hipStream_t s = (hipStream_t)stream;
   if (ids_are_int64) rt_launch((const long long*)expert_ids, T, E, nbits, counts, offsets, idx, max_count, workspace, workspace_bytes, s);
   else rt_launch((const int*)expert_ids, T, E, nbits, counts, offsets, idx, max_count, workspace, workspace_bytes, s);
-  hipError_t err = hipGetLastError();
+  hipError_t err = hx_launch_status();
   if (err != hipSuccess) {
     hx_set_error("hx_moe_routing: launch failed: %s", hipGetErrorString(err));
     return (int)err;

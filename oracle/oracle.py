@@ -25,6 +25,9 @@ Pinning status (see tests/test_oracle_*.py):
 * fp8_attention             : float64 brute force (S<=32), closed-form special cases (S=1,
   uniform scores), permutation invariance, row-max-of-p == 1, a statement-by-statement walk of the
   reference kernel body with a single tile.
+* fp8_attention_tiled       : the same reference lines with the key loop in tiles (the compiled kernel's online
+  softmax); equals fp8_attention for one tile, float64 re-derivation with explicit loops, tile-size invariance
+  where p is exactly representable.
 * fp8_quantize_per_tensor   : the reference has no such function (it only ever passes unit scales,
   ``examples/fp8_gemm.py:74-78``), so there is nothing of the reference's to pin it against: it is the
   build's own definition (amax / 448 scaling), pinned by its algebraic properties (exact powers of two,
@@ -218,6 +221,40 @@ def fp8_attention_literal(q, k, v, batch, heads):
         acc = hl_dot_fp8(p_fp8, v_tile.t(), acc=acc)
         acc = acc / l_i[:, None]
         out[b, h] = acc.to(torch.float8_e4m3fn)
+    return out
+
+
+def fp8_attention_tiled(q, k, v, batch, heads, tile_n: int, out_dtype: torch.dtype = torch.float8_e4m3fn):
+    """examples/fp8_attention.py:54-105 with the key loop (``for tile_n in hl.tile(seq_len)``, :66) walked in tiles of
+    ``tile_n`` keys instead of one tile for the whole sequence: the online-softmax form the reference's compiled
+    kernel executes (its tile size is an autotuned config value; ref-eager mode is the ``tile_n >= seq_len`` case and
+    then this function equals :func:`fp8_attention` bit for bit).  Each statement of the loop body is restated in
+    order: scores of the tile, running max, p against the running max, l and acc rescaled by alpha, p cast to e4m3
+    for the second product.  The query tile spans the whole sequence (rows are independent of one another).
+    Pinned by: equality with :func:`fp8_attention` for one tile; an independent float64 re-derivation in
+    tests/test_oracle_attention.py (explicit per-row loops, own e4m3 rounding through the numpy encoder); invariance
+    of the result to tile_n when every p is exactly representable (uniform scores)."""
+    bh, s, d = q.shape
+    assert bh == batch * heads
+    c = attention_scale(d)
+    out = torch.empty(batch, heads, s, d, dtype=out_dtype)
+    for i in range(bh):
+        m_i = torch.full([s], float("-inf"), dtype=torch.float32)
+        l_i = torch.zeros([s], dtype=torch.float32)
+        acc = torch.zeros([s, d], dtype=torch.float32)
+        qf, kf, vf = dq(q[i]), dq(k[i]), dq(v[i])
+        for n0 in range(0, s, tile_n):
+            n1 = min(n0 + tile_n, s)
+            qk_scaled = (qf @ kf[n0:n1].T) * c
+            m_new = torch.maximum(m_i, torch.amax(qk_scaled, dim=-1))
+            p = torch.exp2(qk_scaled - m_new[:, None])
+            l_ij = torch.sum(p, dim=-1)
+            alpha = torch.exp2(m_i - m_new)
+            l_i = l_i * alpha + l_ij
+            acc = acc * alpha[:, None]
+            acc = acc + dq(to_e4m3(p)) @ vf[:, n0:n1].T
+            m_i = m_new
+        out[i // heads, i % heads] = (acc / l_i[:, None]).to(out_dtype)
     return out
 
 

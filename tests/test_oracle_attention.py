@@ -100,3 +100,58 @@ def test_output_layout_batch_heads():
     assert out.shape == (2, 3, 64, 16)
     one = orc.fp8_attention(q[4:5], k[4:5], v[4:5], 1, 1, torch.float32)
     assert torch.equal(out[1, 1], one[0, 0])  # bh = 4 -> b = 1, h = 1 (examples/fp8_attention.py:56-57)
+
+
+# ---- the key loop in tiles (the compiled kernel's online softmax) ------------------------------------------------
+@pytest.mark.parametrize("b,h,s,d", [(1, 2, 128, 64), (1, 1, 96, 32)])
+def test_tiled_with_one_tile_is_the_ref_eager_form(b, h, s, d):
+    q, k, v = _inputs(b, h, s, d, 7)
+    for tile in (s, s + 5, 4 * s):
+        a = orc.fp8_attention_tiled(q, k, v, b, h, tile)
+        assert torch.equal(a.view(torch.uint8), orc.fp8_attention(q, k, v, b, h).view(torch.uint8))
+
+
+def _tiled_f64(q, k, v, tile_n):
+    """Independent re-derivation for one head: explicit loops over rows and tiles in float64, p rounded to e4m3 by the
+    numpy encoder, exp2 arguments formed in fp32 exactly as the reference's fp32 tensors do."""
+    s, d = q.shape
+    qd, kd, vd = (orc.e4m3_decode(t.view(torch.uint8).numpy()).astype(np.float64) for t in (q, k, v))  # v: [d, s]
+    c = np.float32((1.0 / math.sqrt(float(d))) * 1.44269504)
+    out = np.zeros((s, d))
+    for r in range(s):
+        m, l, acc = -np.inf, 0.0, np.zeros(d)
+        for n0 in range(0, s, tile_n):
+            n1 = min(n0 + tile_n, s)
+            sc = (np.array([np.dot(qd[r], kd[j]) for j in range(n0, n1)]).astype(np.float32) * c).astype(np.float32)
+            m_new = max(m, float(sc.max()))
+            p = np.exp2((sc - np.float32(m_new)).astype(np.float32).astype(np.float64))
+            alpha = 0.0 if m == -np.inf else 2.0 ** float(np.float32(m) - np.float32(m_new))
+            l = l * alpha + p.sum()
+            p8 = orc.e4m3_decode(orc.e4m3_encode(p.astype(np.float32))).astype(np.float64)
+            acc = acc * alpha + np.array([np.dot(p8, vd[j, n0:n1]) for j in range(d)])
+            m = m_new
+        out[r] = acc / l
+    return out
+
+
+@pytest.mark.parametrize("s,d,tile", [(48, 16, 16), (64, 32, 16), (40, 16, 16)])
+def test_tiled_against_float64_rederivation(s, d, tile):
+    q, k, v = _inputs(1, 1, s, d, 11)
+    got = orc.fp8_attention_tiled(q, k, v, 1, 1, tile, torch.float32)[0, 0].numpy()
+    want = _tiled_f64(q[0], k[0], v[0], tile)
+    # same quantisation points; fp32 vs float64 sums (an exp2 ulp could flip an e4m3 tie; none does for this seed)
+    assert np.abs(got - want).max() <= 5e-6 * max(1.0, np.abs(want).max())
+    # and the tiling matters: it is not the single-tile result
+    one = orc.fp8_attention(q, k, v, 1, 1, torch.float32)[0, 0].numpy()
+    assert np.abs(got - one).max() > 1e-4
+
+
+def test_tiled_is_tile_invariant_when_p_is_exact():
+    s, d = 64, 32
+    q = torch.zeros(1, s, d).to(E4M3)  # uniform scores: p == 1 in every tile, whatever the running max
+    g = torch.Generator().manual_seed(6)
+    k = torch.randn(1, s, d, generator=g).to(E4M3)
+    v = torch.randn(1, d, s, generator=g).to(E4M3)
+    a = orc.fp8_attention_tiled(q, k, v, 1, 1, 16, torch.float32)
+    b = orc.fp8_attention(q, k, v, 1, 1, torch.float32)
+    assert torch.allclose(a, b, rtol=0, atol=1e-6)
