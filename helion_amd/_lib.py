@@ -38,6 +38,11 @@ _SIGNATURES = {
          _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int, _c.c_void_p, _c.c_size_t, _c.c_void_p],
     ),
     "hx_moe_workspace_bytes": (_c.c_size_t, [_c.c_int64, _c.c_int64]),
+    "hx_moe_grouped_gemm_static": (
+        _c.c_int,
+        [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int64,
+         _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int, _c.c_void_p],
+    ),
     "hx_moe_routing": (
         _c.c_int,
         [_c.c_void_p, _c.c_int, _c.c_int64, _c.c_int64, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,

@@ -12,6 +12,8 @@
 //   3. hx_gemm16_tile256 / _tile128 / _rows32 or hx_moe_general : the grouped GEMM over (row tile, column tile) pairs;
 //   4. hx_moe_zero_rows  : zero-fills rows whose flag is still clear.
 // Padded rows of a tile are never stored, so there is no read-modify-write and no write race.
+#include <mutex>
+
 #include "gemm16_tile128.h"
 #include "gemm16_rows32.h"
 
@@ -300,6 +302,60 @@ extern "C" int hx_moe_grouped_gemm(const void* A, const void* W, void* C, const 
   hipStream_t s = (hipStream_t)stream;
   if (dtype == HX_BF16) return launch_moe<true>(A, W, C, counts, offsets, idx, T, K, N, E, 1, workspace, s);
   return launch_moe<false>(A, W, C, counts, offsets, idx, T, K, N, E, 1, workspace, s);
+}
+
+// ------------------------------------------------------------------------------------------
+// hx_moe_grouped_gemm for callers that cannot allocate: the tile table and the row flags live in a file-scope
+// device array instead of a caller-provided workspace.  Every GPU holds its own copy of the array at its own
+// address; the address is looked up once per device (with that device current) and only that pointer is ever
+// handed to kernels -- the array's name is a host-side stand-in, not a device address.
+// ------------------------------------------------------------------------------------------
+#define HX_MOE_STATIC_SCRATCH_BYTES (256 * 1024)
+static __device__ __align__(256) uint8_t scratch[HX_MOE_STATIC_SCRATCH_BYTES];
+
+static std::mutex g_scratch_mu;
+static void* g_scratch_ptr[64];  // per device ordinal; nullptr = not looked up yet
+
+// Device address of this GPU's copy of `scratch` (cached after the first call on the device); nullptr + error set
+// on failure.
+static void* moe_static_scratch() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= 64) {
+    hx_set_error("hx_moe_grouped_gemm_static: hipGetDevice failed or device ordinal %d out of range: %s", dev, hipGetErrorString(e));
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      hx_set_error("hx_moe_grouped_gemm_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  return g_scratch_ptr[dev];
+}
+
+extern "C" int hx_moe_grouped_gemm_static(const void* A, const void* W, void* C, const int32_t* counts, const int32_t* offsets,
+                                          const int32_t* idx, int64_t T, int64_t K, int64_t N, int64_t E, int64_t max_T, int dtype,
+                                          void* stream) {
+  if (T < 0 || K < 0 || N < 0 || E < 0 || max_T < 0) {
+    hx_set_error("hx_moe_grouped_gemm_static: negative size");
+    return HX_ERR_BAD_ARG;
+  }
+  if (T > HX_MOE_STATIC_MAX_ROWS || E > HX_MOE_STATIC_MAX_EXPERTS || hx_moe_workspace_bytes(T, E) > HX_MOE_STATIC_SCRATCH_BYTES) {
+    hx_set_error("hx_moe_grouped_gemm_static: T = %lld rows / E = %lld experts exceed the built-in scratch (at most %d rows and %d "
+                 "experts); use hx_moe_grouped_gemm with a workspace", (long long)T, (long long)E, HX_MOE_STATIC_MAX_ROWS,
+                 HX_MOE_STATIC_MAX_EXPERTS);
+    return HX_ERR_UNSUPPORTED;
+  }
+  if (T == 0 || N == 0) return 0;
+  void* ptr = moe_static_scratch();
+  if (!ptr) return HX_ERR_WORKSPACE;
+  // same checks, same kernels: the workspace is this device's copy of the static array
+  return hx_moe_grouped_gemm(A, W, C, counts, offsets, idx, T, K, N, E, max_T, dtype, ptr, HX_MOE_STATIC_SCRATCH_BYTES, stream);
 }
 
 // ------------------------------------------------------------------------------------------

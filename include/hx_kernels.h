@@ -111,6 +111,20 @@ int hx_moe_grouped_gemm(const void* A, const void* W, void* C, const int32_t* co
                         void* stream);
 size_t hx_moe_workspace_bytes(int64_t T, int64_t E);
 
+/* hx_moe_grouped_gemm for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, checks, kernels and
+ * results as hx_moe_grouped_gemm, minus the workspace: the tile table and the row-covered flags live in a 256 KiB
+ * device array built into the library (one copy per GPU, held until the process ends), whose address is looked up
+ * on the first call on each device.  Calls neither hipMalloc nor hipFree nor anything that allocates.
+ * Limits: T <= HX_MOE_STATIC_MAX_ROWS and E <= HX_MOE_STATIC_MAX_EXPERTS, otherwise HX_ERR_UNSUPPORTED and nothing
+ * is launched.  Every call on a GPU uses that GPU's one array (each call rewrites the part it reads, so nothing
+ * carries over from the previous call): two calls that overlap in time on one GPU -- different streams, or
+ * different host threads -- race on it; calls on one stream are ordered and safe. */
+enum { HX_MOE_STATIC_MAX_ROWS = 131072, HX_MOE_STATIC_MAX_EXPERTS = 1024 };
+int hx_moe_grouped_gemm_static(const void* A, const void* W, void* C, const int32_t* counts, const int32_t* offsets,
+                               const int32_t* idx, int64_t T, int64_t K, int64_t N, int64_t E, int64_t max_T, int dtype,
+                               void* stream);
+
 /* Replaces the tensor ops of `moe_matmul_ogs_helion_kernel_args_gen(A, W, top1_expert_per_token)` (reference:
  * examples/moe_matmul_ogs.py:84-121) with one kernel and no host synchronisation:
  *   idx = argsort(expert_ids, stable=True); counts = bincount(expert_ids, minlength=E);
