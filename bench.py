@@ -15,8 +15,12 @@ Timing protocol, the same for every kernel timed here:
   3. exactly K timed launches, every launch bracketed by its own pair of HIP events on the launch stream; the
      reported time per launch is the MEDIAN of the K event pairs (mean, min and max are printed next to it, and so
      is the mean over one event pair around all K launches).
-While the settle and timed launches run, a host thread samples the engine clock of the eight XCDs and the socket
-power through amdsmi; the mean is printed as "engine_clock_mhz" together with the MFMA peak recomputed at that clock.
+  4. clock phase, after the timed region and outside it: CLOCK_PHASE_LAUNCHES more launches of the same kernel,
+     back to back with the timed ones, while a one-wave probe kernel (hx_clock_probe) runs three times on a second
+     stream: it reads the shader-clock counter against the constant 100 MHz counter over 50 us, which gives the
+     engine clock the chip sustains under this kernel's load (it is power-limited well below its 2.4 GHz maximum).
+     Printed as "engine_clock_mhz" with the MFMA peak recomputed at that clock.  (amdsmi's clock readings are refreshed
+     about once a second, too slow for a timed region of a few milliseconds; its socket power is printed as a hint.)
 
 The JSON line also carries the other three configurations (decode-shape GEMM, FP8 attention, MoE grouped GEMM) under
 "other_workloads" together with the kernels either side of them (casts, quantisation, routing), each with its own
@@ -33,7 +37,6 @@ import pathlib
 import statistics
 import subprocess
 import sys
-import threading
 import time
 
 ROOT = pathlib.Path(__file__).resolve().parent
@@ -47,10 +50,12 @@ BF16_FLOP_PER_CU_CLK = 4096.0
 
 SETTLE_MIN_LAUNCHES = 40
 SETTLE_SECONDS = 0.4
+CLOCK_PHASE_LAUNCHES = 6
+CLOCK_PROBE_TICKS = 5000  # of the 100 MHz counter = 50 us
 
 
 # ----------------------------------------------------------------------------------------------------------------
-# device facts and the engine-clock sampler (amdsmi; both degrade to None when it is unavailable)
+# device facts (amdsmi and the amd-smi tool; every field degrades to None when they are unavailable)
 # ----------------------------------------------------------------------------------------------------------------
 class _Smi:
     def __init__(self):
@@ -90,68 +95,57 @@ class _Smi:
         return (sum(clks) / len(clks) if clks else None), (p if isinstance(p, int) else None)
 
 
-class ClockSampler:
-    """Samples the XCDs' engine clocks (their mean) and the socket power from a host thread between start() and stop()."""
-
-    def __init__(self, smi: _Smi, period_s=0.004):
-        self.smi, self.period = smi, period_s
-        self.samples, self._stop, self._t = [], False, None
-
-    def start(self):
-        if not self.smi.ok:
-            return
-        self._stop = False
-
-        def run():
-            while not self._stop:
-                try:
-                    self.samples.append(self.smi.sample())
-                except Exception:
-                    pass
-                time.sleep(self.period)
-
-        self._t = threading.Thread(target=run, daemon=True)
-        self._t.start()
-
-    def stop(self):
-        self._stop = True
-        if self._t is not None:
-            self._t.join()
-        clk = [c for c, _ in self.samples if c]
-        pw = [p for _, p in self.samples if p]
-        if not clk:
-            return None
-        return {"mean": sum(clk) / len(clk), "min": min(clk), "max": max(clk), "samples": len(clk),
-                "socket_power_w_mean": (sum(pw) / len(pw)) if pw else None,
-                "source": "amdsmi gpu_metrics current_gfxclks (mean over the 8 XCDs), sampled from a host thread during the "
-                          "second half of the settle launches and the warm-up and timed launches of this kernel"}
-
-
 _SMI = None
 _DEV = {}
+
+
+def _clock_phase(fn):
+    """Step 4 of the protocol: engine clock under this kernel's load, measured next to (not inside) the timed region."""
+    import torch
+    from helion_amd import _lib
+
+    lib = _lib.load()
+    side = torch.cuda.Stream()
+    bufs = torch.zeros(3, 2, dtype=torch.int64, device="cuda")
+    marks = []
+    for i in range(CLOCK_PHASE_LAUNCHES):
+        if i in (1, 3, 5):
+            ev = torch.cuda.Event()
+            ev.record()  # the probe starts once launch i-1 has finished, i.e. while launch i runs
+            marks.append(ev)
+        fn()
+        if i in (1, 3, 5):
+            side.wait_event(marks[-1])
+            _lib.check(lib.hx_clock_probe(bufs[len(marks) - 1].data_ptr(), CLOCK_PROBE_TICKS, side.cuda_stream), "hx_clock_probe")
+    torch.cuda.synchronize()
+    vals = [100.0 * c / r for c, r in bufs.cpu().tolist() if r > 0]
+    if not vals:
+        return None
+    out = {"mean": sum(vals) / len(vals), "probes": vals,
+           "source": f"hx_clock_probe: shader-clock counter / 100 MHz counter over {CLOCK_PROBE_TICKS // 100} us, one wave on a second "
+                     f"stream, three probes during {CLOCK_PHASE_LAUNCHES} extra launches issued right after the timed region"}
+    if _SMI is not None and _SMI.ok:
+        try:
+            out["socket_power_w_amdsmi"] = _SMI.sample()[1]
+        except Exception:
+            pass
+    return out
 
 
 def _time_launches(fn, steps, warmup, settle=True):
     """Times `fn` (one launch per call) as the module docstring describes.  Returns a dict: median / mean / min / max
     of the per-launch event pairs and the mean of one pair around the whole timed region (ms), the wall-clock time
-    per step of the same region bracketed by synchronisations, the settle launches done and the sampled clock."""
+    per step of the same region bracketed by synchronisations, the settle launches done and the measured clock."""
     import torch
 
-    sampler = ClockSampler(_SMI) if _SMI is not None else None
     n_settle = 0
     if settle:
         t_end = time.perf_counter() + SETTLE_SECONDS
-        started = False
         while n_settle < SETTLE_MIN_LAUNCHES or time.perf_counter() < t_end:
             for _ in range(8):
                 fn()
             n_settle += 8
             torch.cuda.synchronize()
-            if sampler is not None and not started and time.perf_counter() > t_end - SETTLE_SECONDS / 2:
-                sampler.start()
-                started = True
-        if sampler is not None and not started:
-            sampler.start()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -166,7 +160,9 @@ def _time_launches(fn, steps, warmup, settle=True):
     end.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    clock = sampler.stop() if (sampler is not None and settle) else None
+    for _ in range(2):  # keep the chip loaded between the synchronisation above and the clock phase
+        fn()
+    clock = _clock_phase(fn)
     per = [s.elapsed_time(e) for s, e in pairs]
     return {"median_ms": statistics.median(per), "mean_ms": sum(per) / len(per), "min_ms": min(per), "max_ms": max(per),
             "whole_region_mean_ms": start.elapsed_time(end) / steps, "wall_ms_per_step": wall_ms, "timed_launches": steps,

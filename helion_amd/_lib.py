@@ -74,6 +74,7 @@ _SIGNATURES = {
     "hx_matmul_splits": (_c.c_int, [_c.c_int64] * 7 + [_c.c_int, _c.c_int]),
     "hx_attention": (_c.c_int, [_c.c_void_p] * 4 + [_c.c_int64] * 5 + [_c.c_int, _c.c_void_p]),
     "hx_attention_path": (_c.c_int, [_c.c_int64] * 4 + [_c.c_int] + [_c.c_void_p] * 4),
+    "hx_clock_probe": (_c.c_int, [_c.c_void_p, _c.c_int64, _c.c_void_p]),
     "hx_matmul_path": (_c.c_int, [_c.c_int64] * 7 + [_c.c_int, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p]),
 }
 

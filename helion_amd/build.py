@@ -13,7 +13,7 @@ PKG = pathlib.Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 LIB = PKG / "libhx_kernels.so"
 SOURCES = ["hx_common.cpp", "fp8_gemm.hip", "fp8_attention.hip", "moe_gemm.hip", "moe_routing.hip", "fp8_quantize.hip",
-           "matmul16.hip", "attention16.hip"]
+           "matmul16.hip", "attention16.hip", "diag.hip"]
 FLAGS = [
     "--offload-arch=gfx950",
     "-O3",
