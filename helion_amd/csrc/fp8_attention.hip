@@ -23,6 +23,7 @@
 #include "hx_common.h"
 
 #include <cmath>
+#include <type_traits>
 
 #define ATT_BN 64      // keys per tile
 #define ATT_WAVES 4
@@ -45,47 +46,89 @@ __device__ __forceinline__ int att_vswz(int row) {
   return RB == 128 ? (((row >> 1) & 3) << 1) : (((row >> 2) & 1) << 1);
 }
 
-// wait until at most `newer` tiles' worth of this wave's DMA instructions (IPT per tile) are outstanding
+// ------------------------------------------------------------------------------------------
+// The MFMA kernel, software-pipelined three tiles deep.  MODE 1: exact row max (two passes); MODE 0: online softmax.
+//
+// What was measured on gfx950 and shapes this kernel:
+//   * a SIMD issues one VALU-class instruction at a time and an fp8 MFMA holds that port for most of its 64 cycles:
+//     on this kernel's instruction mix each 32x32x64 MFMA leaves room for about eight other VALU instructions of any
+//     kind in its shadow, and what does not fit is paid in full.  So no wave may ever wait on the LDS, and the VALU
+//     work has to be spread evenly between the MFMAs;
+//   * step j of the key loop therefore issues the score MFMAs of tile j+1, the softmax arithmetic of tile j and the
+//     P.V MFMAs of tile j-1: eight MFMAs that do not depend on the step's VALU work, one per micro-step, each followed
+//     by its share of the fma / exp2 / convert instructions; fragments are read from the LDS two MFMAs ahead;
+//   * the key loop is unrolled four times so that the LDS slot of every fragment read is an immediate offset, and every
+//     step issues the same DMA instructions (past the last tile it re-fetches the last tile into a slot nobody reads
+//     any more), so its body has no branch and one constant vmcnt wait;
+//   * pass 1 (MODE 1) streams K through all eight tile slots of the ring and synchronises once per two tiles.
+// LDS: K(t) lives in the K half of slot t % 4 from step t-4 to step t-1, V(t) in the V half of the same slot from
+// step t-2 to step t+1.
+// Any sequence length: the last key tile may be partial (keys past S are masked to -inf before the max and the
+// exponential; their K / V rows are re-reads of valid rows), and so may the last query rows of a wave.
+// ------------------------------------------------------------------------------------------
 template <int IPT>
-__device__ __forceinline__ void att_wait_tiles(int newer) {
-  if (newer >= 2) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(2 * IPT));
-  else if (newer == 1) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(IPT));
-  else __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(0));
+__device__ __forceinline__ void att_wait_outstanding(int n) {  // n tiles' worth of this wave's DMA may stay in flight
+  switch (n) {
+    case 0: __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(0)); break;
+    case 1: __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(IPT)); break;
+    case 2: __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(2 * IPT)); break;
+    case 3: __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(3 * IPT)); break;
+    case 4: __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(4 * IPT)); break;
+    default: __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(5 * IPT)); break;
+  }
 }
 
-template <int D, int OUT, bool EXACT, bool VSD>
-__global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t* __restrict__ Q, const uint8_t* __restrict__ Kt,
-                                                                  const uint8_t* __restrict__ Vt, void* __restrict__ Out, int S,
-                                                                  int BH, int qtiles, float c) {
-  constexpr int KSTEPS = D / 64;  // MFMA k-steps for S = K Q^T
-  constexpr int DB = D / 32;      // 32-row blocks of O^T
-  constexpr int KROWS_PER_DMA = 1024 / D;
-  constexpr int KPW = (ATT_BN / KROWS_PER_DMA) / ATT_WAVES;  // K DMA instructions per wave per tile
-  constexpr int VPW = VSD ? KPW : (D / 16) / ATT_WAVES;      // V DMA instructions per wave per tile ([D][S]: 16 rows x 64 B each)
-  constexpr int TILE = ATT_BN * D;                           // bytes of a K tile == bytes of a V tile
-  __shared__ __attribute__((aligned(1024))) uint8_t smem[ATT_NS][2][TILE];
+// v_max3_f32 as one instruction (fmaxf(fmaxf(a, b), c) first canonicalises every operand that comes out of an MFMA,
+// which doubles the instruction count of a max reduction)
+__device__ __forceinline__ float att_max3(float a, float b, float c) {
+  float d;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+  return d;
+}
 
-  // workgroup -> (head, query tile): XCD x (= id%8) takes heads x, x+8, ...; the query tiles of a head
-  // are consecutive on that XCD so its K/V stay in that XCD's L2.
+// max over the two halves of the wave: lane l and lane l ^ 32 both receive max(x[l], x[l ^ 32])
+__device__ __forceinline__ float att_max_across_halves(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
+template <int D, int OUT, int MODE, bool VSD>
+__global__ __launch_bounds__(256, 2) void hx_fp8_attention_pipe(const uint8_t* __restrict__ Q, const uint8_t* __restrict__ Kt,
+                                                                const uint8_t* __restrict__ Vt, void* __restrict__ Out, int S, int BH,
+                                                                int qtiles, float c) {
+  constexpr int KSTEPS = D / 64;  // MFMA k-steps for S = K Q^T
+  constexpr int DB = D / 32;      // 32-row blocks of O^T == score MFMAs per tile (2 key blocks x KSTEPS)
+  constexpr int KROWS_PER_DMA = 1024 / D;
+  constexpr int KPW = (ATT_BN / KROWS_PER_DMA) / ATT_WAVES;
+  constexpr int VPW = VSD ? KPW : (D / 16) / ATT_WAVES;
+  constexpr int TILE = ATT_BN * D;
+  constexpr int NM = 2 * DB;      // MFMA micro-steps per key tile in pass 2
+  constexpr int GPM = 8 / NM < 1 ? 1 : 8 / NM;  // softmax groups (4 scores each) per micro-step
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[ATT_NS][2][TILE];
+  __shared__ float xch[ATT_WAVES * 32];  // pass 1: the partial row maxima a wave pair exchanges
+  uint8_t* const sm = &smem[0][0][0];
+
   int bh, qt;
   {
     const int id = blockIdx.x, xcd = id & 7, loc = id >> 3;
     const int hl = loc / qtiles;
     qt = loc % qtiles;
     bh = xcd + 8 * hl;
-    if (bh >= BH) return;  // whole workgroup exits together
+    if (bh >= BH) return;
   }
   const int tid = threadIdx.x, lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int q31 = lane & 31, G = lane >> 5;
   const int q0 = qt * ATT_BM + w * 32;
-  const bool active = q0 < S;  // wave-uniform; inactive waves still help with DMA and barriers
+  const bool active = q0 < S;
+  const int ntiles = (S + ATT_BN - 1) / ATT_BN;
+  const int last = ntiles - 1;
+  const bool ragged = (S % ATT_BN) != 0;  // the last key tile is partial
 
   const uint8_t* Qh = Q + (long)bh * S * D;
   const uint8_t* Kh = Kt + (long)bh * S * D;
-  const uint8_t* Vh = Vt + (long)bh * D * S;  // either layout: D*S bytes per head
+  const uint8_t* Vh = Vt + (long)bh * D * S;
 
-  // ---- Q fragments (B operand of S^T): lane (q, G): Q[q][64t + 32G .. +31]
   v8i qf[KSTEPS];
   {
     const int qrow = min(q0 + q31, S - 1);
@@ -97,58 +140,88 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
     }
   }
 
-  // ---- DMA addressing: wave w issues K instructions j = w, w+4, ... (KROWS_PER_DMA rows of D bytes each) and
-  // V instructions j = w, w+4, ... (16 rows of 64 bytes each).  The swizzle of a lane's row does not depend on
-  // which of the wave's instructions it is, so one per-lane offset serves all of them.
-  constexpr int KCPR = D / 16;  // chunks per K row
+  // ---- DMA addressing (as in hx_fp8_attention_general's tiles: see att_swz); the destination is a byte offset into the ring
+  constexpr int KCPR = D / 16;
   const int k_lrow = lane / KCPR, k_lpos = lane % KCPR;
-  const uint32_t k_vo = (uint32_t)(k_lrow * D + ((k_lpos ^ att_swz<D>(w * KROWS_PER_DMA + k_lrow)) * 16));
+  const int k_chunk = (k_lpos ^ att_swz<D>(w * KROWS_PER_DMA + k_lrow)) * 16;
+  const uint32_t k_vo = (uint32_t)(k_lrow * D + k_chunk);
   const int v_lrow = lane >> 2, v_lpos = lane & 3;
-  const uint32_t v_vo = VSD ? (uint32_t)(k_lrow * D + ((k_lpos ^ att_vswz<D>(w * KROWS_PER_DMA + k_lrow)) * 16))
-                            : (uint32_t)(v_lrow * S + ((v_lpos ^ att_swz<64>(v_lrow)) * 16));
-  const uint32_t lds0 = hx_lds_addr(&smem[0][0][0]);
-  auto issue_k = [&](int tile, int stage) {
-#pragma unroll
-    for (int jj = 0; jj < KPW; ++jj) {
-      const int j = w + ATT_WAVES * jj;
-      hx_g2l16_s(Kh + ((long)tile * ATT_BN + j * KROWS_PER_DMA) * D, k_vo, lds0 + (uint32_t)stage * 2 * TILE + j * 1024);
+  const int v_chunk = VSD ? (k_lpos ^ att_vswz<D>(w * KROWS_PER_DMA + k_lrow)) * 16 : (v_lpos ^ att_swz<64>(v_lrow)) * 16;
+  const uint32_t v_vo = VSD ? (uint32_t)(k_lrow * D + v_chunk) : (uint32_t)(v_lrow * S + v_chunk);
+  const uint32_t lds0 = hx_lds_addr(sm);
+  // Two forms of every DMA instruction.  Plain: wave-uniform 64-bit base of the tile + a constant per-lane offset
+  // (scalar arithmetic only; for the branch-free steps, which never touch a partial tile).  Clamped: the head's base +
+  // a per-lane offset computed from the tile index (three vector instructions, no branch); rows (keys) past S re-read
+  // row S-1 and, in the [D][S] layout of V, 16-byte column chunks past S re-read the last chunk of the same row
+  // (S % 16 == 0 there), so a partial last tile is fetched by the same code as any other.
+  auto issue_k_one = [&](int tile, uint32_t dst, int jj, auto clamped) {
+    const int j = w + ATT_WAVES * jj;
+    if (decltype(clamped)::value) {
+      const int row = min(tile * ATT_BN + j * KROWS_PER_DMA + k_lrow, S - 1);
+      hx_g2l16_s(Kh, (uint32_t)(row * D + k_chunk), lds0 + dst + j * 1024);
+    } else {
+      hx_g2l16_s(Kh + ((long)tile * ATT_BN + j * KROWS_PER_DMA) * D, k_vo, lds0 + dst + j * 1024);
     }
   };
-  auto issue_v = [&](int tile, int stage) {
-#pragma unroll
-    for (int jj = 0; jj < VPW; ++jj) {
-      const int j = w + ATT_WAVES * jj;
-      if (VSD) hx_g2l16_s(Vh + ((long)tile * ATT_BN + j * KROWS_PER_DMA) * D, v_vo, lds0 + (uint32_t)stage * 2 * TILE + TILE + j * 1024);
-      else hx_g2l16_s(Vh + (long)(j * 16) * S + (long)tile * ATT_BN, v_vo, lds0 + (uint32_t)stage * 2 * TILE + TILE + j * 1024);
+  auto issue_v_one = [&](int tile, uint32_t dst, int jj, auto clamped) {
+    const int j = w + ATT_WAVES * jj;
+    if (decltype(clamped)::value) {
+      if (VSD) {
+        const int row = min(tile * ATT_BN + j * KROWS_PER_DMA + k_lrow, S - 1);
+        hx_g2l16_s(Vh, (uint32_t)(row * D + v_chunk), lds0 + dst + j * 1024);
+      } else {
+        const int col = min(tile * ATT_BN + v_chunk, S - 16);
+        hx_g2l16_s(Vh, (uint32_t)((j * 16 + v_lrow) * S + col), lds0 + dst + j * 1024);
+      }
+    } else if (VSD) {
+      hx_g2l16_s(Vh + ((long)tile * ATT_BN + j * KROWS_PER_DMA) * D, v_vo, lds0 + dst + j * 1024);
+    } else {
+      hx_g2l16_s(Vh + (long)(j * 16) * S + (long)tile * ATT_BN, v_vo, lds0 + dst + j * 1024);
     }
+  };
+  auto issue_k = [&](int tile, uint32_t dst) {
+#pragma unroll
+    for (int jj = 0; jj < KPW; ++jj) issue_k_one(tile, dst, jj, std::true_type{});
+  };
+  auto issue_v = [&](int tile, uint32_t dst) {
+#pragma unroll
+    for (int jj = 0; jj < VPW; ++jj) issue_v_one(tile, dst, jj, std::true_type{});
   };
 
-  // ---- MFMA operand addressing
-  // K operand (A of S^T): MFMA row i = lane%32 is key(i) within the 32-key block
+  // pass 2's first tiles, as "virtual steps" -4 .. -1: K(0) | K(1) | K(2), V(0) | K(3), V(1)   (tile indices clamped
+  // like in the steps).  Issued as early as the ring is free: at kernel start (MODE 0), or under pass 1's last round.
+  auto issue_pass2_prologue = [&]() {
+    issue_k(0, 0);
+    issue_k(min(1, last), 1 * 2 * TILE);
+    issue_k(min(2, last), 2 * 2 * TILE);
+    issue_v(0, TILE);
+    issue_k(min(3, last), 3 * 2 * TILE);
+    issue_v(min(1, last), 1 * 2 * TILE + TILE);
+  };
+
+  // ---- fragment addressing: per-lane parts in registers, slot / block parts as immediates
   const int krow = 16 * ((q31 >> 2) & 1) + 4 * (q31 >> 3) + (q31 & 3);
-  int k_off[2][KSTEPS][2];  // [block][t][half] byte offsets in the K tile
+  int k_off[KSTEPS][2];  // key block 0; block 1 is 32 rows further (its swizzle is the same)
 #pragma unroll
-  for (int kb = 0; kb < 2; ++kb)
+  for (int t = 0; t < KSTEPS; ++t)
 #pragma unroll
-    for (int t = 0; t < KSTEPS; ++t)
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const int row = kb * 32 + krow;
-        k_off[kb][t][h] = row * D + (((4 * t + 2 * G + h) ^ att_swz<D>(row)) * 16);
-      }
-  int v_off[2];  // [D][S] layout: [block] byte offsets in the V tile for d-row lane%32 (add db*32*64)
+    for (int h = 0; h < 2; ++h) k_off[t][h] = krow * D + (((4 * t + 2 * G + h) ^ att_swz<D>(krow)) * 16);
+  int v_off[2];
 #pragma unroll
   for (int kb = 0; kb < 2; ++kb) v_off[kb] = q31 * 64 + (((2 * kb + G) ^ att_swz<64>(q31)) * 16);
-  // [S][D] layout: transposing read j (0..3) of a 32-row block of V^T fetches keys kr0..kr0+7,
-  // kr0 = 32*(j>>1) + 16*G + 8*(j&1); this lane supplies 8 bytes of key row kr0 + (lane%16)/2, columns
-  // 16*((lane>>4)&1) + 8*(lane&1) .. +7 of the block, and receives column lane%32, keys kr0..kr0+7.
-  // Block db adds 2*db to the chunk index in bits the swizzle's xor commutes with: offset ^ (db*32).
   int vt_off[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int row = 32 * (j >> 1) + 16 * G + 8 * (j & 1) + ((lane & 15) >> 1);
     vt_off[j] = row * D + (((((lane >> 4) & 1)) ^ att_vswz<D>(row)) * 16) + (lane & 1) * 8;
   }
+  // n-th score MFMA of a tile: key block n % 2, k-step n / 2 (the two MFMAs of a block are never back to back)
+  auto load_kfrag = [&](const uint8_t* sk, int n) -> v8i {
+    const int kb = n & 1, t = n >> 1;
+    v4i lo = *(const v4i*)(sk + kb * 32 * D + k_off[t][0]);
+    v4i hi = *(const v4i*)(sk + kb * 32 * D + k_off[t][1]);
+    return (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+  };
   auto load_vfrag = [&](const uint8_t* sv, int d) -> v8i {
     if (VSD) {
       v8i f;
@@ -164,161 +237,304 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
     v4i hi = *(const v4i*)(sv + d * 32 * 64 + v_off[1]);
     return (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   };
-
-  const int ntiles = S / ATT_BN;
-
-  auto scores = [&](const uint8_t* sk, v16f(&s)[2]) {
+  const v16f zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  auto scores_plain = [&](const uint8_t* sk, v16f(&s)[2]) {
+    v8i kf[2 * KSTEPS];
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
+    for (int n = 0; n < 2 * KSTEPS; ++n) kf[n] = load_kfrag(sk, n);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) s[kb][r] = 0.f;
+    for (int n = 0; n < 2 * KSTEPS; ++n) s[n & 1] = hx_mfma_32x32x64_e4m3(kf[n], qf[n >> 1], (n >> 1) ? s[n & 1] : zero16);
+  };
+  // scores of the partial last tile: s[kb][r] belongs to key 64*last + 32*kb + 16*G + r; keys past S -> -inf
+  auto mask_last = [&](v16f(&s)[2]) {
+    int nv = S - last * ATT_BN - 16 * G;  // this lane's keys 32*kb + r of the tile are valid below nv
+    asm volatile("" : "+v"(nv));          // keep the 32 comparisons here, in the one step that needs them
 #pragma unroll
-      for (int t = 0; t < KSTEPS; ++t) {
-        v4i lo = *(const v4i*)(sk + k_off[kb][t][0]);
-        v4i hi = *(const v4i*)(sk + k_off[kb][t][1]);
-        v8i kf = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-        s[kb] = hx_mfma_32x32x64_e4m3(kf, qf[t], s[kb]);
-      }
-    }
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        if (32 * kb + r >= nv) s[kb][r] = -__builtin_inff();
   };
 
-  // The Q loads above are the only memory operations the compiler tracks; retire them here so that it has no
-  // reason to put a vmcnt wait (which would also wait for every DMA in flight) inside the key loops.
-  HX_WAIT_VM0();
+  HX_WAIT_VM0();  // the Q loads: the only memory operations the compiler tracks with vmcnt
 
-  float neg_m = __builtin_inff();  // minus the scaled-domain row max
-
-  // Both key loops are software pipelined by one tile: the score MFMAs of tile j+1 are issued before the
-  // VALU work on tile j's scores, so the matrix pipe runs under the softmax arithmetic.
-  // LDS slots: tile t lives in slot t % 4.  At iteration j the wave reads K of tile j+1 and V of tile j while
-  // tiles j+2 and j+3 are in flight; the barrier at the top of iteration j is what frees slot (j+3) % 4.
-  if (EXACT) {
-    // ---------------- pass 1: exact row max of the raw scores (K tiles only)
-    float smax0 = -__builtin_inff(), smax1 = -__builtin_inff();
-    for (int t = 0; t < ATT_LEAD && t < ntiles; ++t) issue_k(t, t % ATT_NS);
-    att_wait_tiles<KPW>(min(ATT_LEAD - 1, ntiles - 1));
-    __syncthreads();
-    // one tile: sync, prefetch, issue the score MFMAs of tile j+1 into `next`, then reduce tile j's scores (`cur`)
-    auto step1 = [&](v16f(&cur)[2], v16f(&next)[2], int j) {
-      if (j + 2 < ntiles) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(KPW));  // tile j+1 landed, tile j+2 may be in flight
-      else HX_WAIT_VM0();
-      __syncthreads();  // tile j+1 visible to every wave; every wave is done with tile j-1
-      if (active) {
-        if (j + 1 < ntiles) scores(&smem[(j + 1) % ATT_NS][0][0], next);
+  float neg_m = __builtin_inff();  // minus the row max in the scaled domain (MODE 0: of the keys seen so far)
+  // ================= pass 1 (MODE 1): exact row max of the raw scores.
+  // The waves work in pairs: waves 2p and 2p+1 together own 64 queries, and each of them multiplies every other key
+  // tile (parity = w & 1) by BOTH query blocks, so a K fragment read from the LDS feeds two MFMAs and the pass reads
+  // half the LDS bytes per MFMA of a wave-owns-its-queries scheme (it was bound by those reads, not by the matrix pipe).
+  // At the end the two waves of a pair exchange their partial maxima through the LDS.  A score is the same MFMA dot
+  // product, k-step order included, whichever wave computes it, so pass 2 reproduces the maximum bit for bit.
+  // Tile t sits in slot t % 8 of the ring viewed as eight K slots; one barrier per round of two tiles, with the four
+  // tiles of the next two rounds in flight.
+  if (MODE == 1) {
+    const int pair = w >> 1, par = w & 1;
+    const int qp0 = qt * ATT_BM + pair * 64;
+    const bool pair_active = qp0 < S;  // wave-uniform
+    v8i qp[2][KSTEPS];
 #pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-          smax0 = fmaxf(fmaxf(smax0, cur[0][r]), cur[0][r + 1]);
-          smax1 = fmaxf(fmaxf(smax1, cur[1][r]), cur[1][r + 1]);
-        }
+    for (int qb = 0; qb < 2; ++qb) {
+      const int qrow = min(qp0 + 32 * qb + q31, S - 1);
+#pragma unroll
+      for (int t = 0; t < KSTEPS; ++t) {
+        const v4i* pq = (const v4i*)(Qh + (long)qrow * D + 64 * t + 32 * G);
+        v4i lo = pq[0], hi = pq[1];
+        qp[qb][t] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
       }
-      if (j + ATT_LEAD < ntiles) issue_k(j + ATT_LEAD, (j + ATT_LEAD) % ATT_NS);  // (at the end of the step: see pass 2)
-    };
-    v16f sa[2], sb[2];
-    if (active) scores(&smem[0][0][0], sa);
-    int j = 0;
-    for (; j + 1 < ntiles; j += 2) {
-      step1(sa, sb, j);
-      step1(sb, sa, j + 1);
     }
-    if (j < ntiles) step1(sa, sb, j);
-    float smax = fmaxf(smax0, smax1);
-    smax = fmaxf(smax, __shfl_xor(smax, 32));
+    HX_WAIT_VM0();
+    float smx[2] = {-__builtin_inff(), -__builtin_inff()};  // per query block: max of this lane's scores so far
+    auto kslot = [&](int t) { return (uint32_t)((t & 7) * TILE); };
+    const int npro = min(6, ntiles);
+    for (int t = 0; t < npro; ++t) issue_k(t, kslot(t));
+    constexpr int NF = 2 * KSTEPS;     // K fragments (= MFMAs per query block) per tile
+    constexpr int RPF = 32 / NF;       // scores of each query block reduced per fragment step
+    // max reduction of part `part` (of NF) of a finished tile's scores, both query blocks
+    auto reduce_part = [&](v16f(&cur)[2][2], int part) {
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+        for (int e = part * RPF; e < (part + 1) * RPF; e += 2) smx[qb] = att_max3(smx[qb], cur[qb][e >> 4][e & 15], cur[qb][e >> 4][(e & 15) + 1]);
+    };
+    // One round: scores of tile `t` (if it exists) into `next` under the max reduction of `cur` (tile tc, if any).
+    // A fragment read takes several hundred cycles when the LDS is busy, more than a pair of MFMAs covers, so the
+    // four fragments of a tile live in registers and each is refilled with the NEXT round's fragment (tile t + 2) as
+    // soon as its two MFMAs are out: by then that tile has landed for every wave (the round's barrier waits for the
+    // tiles of two rounds), and the refill has the rest of the round and the barrier to arrive.
+    v8i kf[NF];
+    auto round = [&](v16f(&cur)[2][2], v16f(&next)[2][2], int t, int tc) {
+      if (!pair_active) return;
+      // (a partial last tile needs no masking here: its rows past S are re-reads of key S-1, whose score is a
+      // valid one, so they cannot change the maximum)
+      if (t < ntiles) {
+        const bool more = t + 2 < ntiles;
+        const uint8_t* sk2 = sm + kslot(more ? t + 2 : t);  // (no next tile: re-read this one, the values are not used)
+#pragma unroll
+        for (int n = 0; n < NF; ++n) {
+          const int kb = n & 1, ks = n >> 1;
+          next[0][kb] = hx_mfma_32x32x64_e4m3(kf[n], qp[0][ks], ks ? next[0][kb] : zero16);
+          next[1][kb] = hx_mfma_32x32x64_e4m3(kf[n], qp[1][ks], ks ? next[1][kb] : zero16);
+          kf[n] = load_kfrag(sk2, n);
+          if (tc >= 0) reduce_part(cur, n);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else if (tc >= 0) {
+#pragma unroll
+        for (int n = 0; n < NF; ++n) reduce_part(cur, n);
+      }
+    };
+    v16f ca[2][2], cb[2][2];
+    int tc = -1;  // the tile whose scores `cur` holds (-1: none)
+    // tiles 0 .. 3 (two rounds' worth) have landed before the first fragments are read
+    att_wait_outstanding<KPW>(max(npro - 4, 0));
+    __syncthreads();
+    if (pair_active) {
+#pragma unroll
+      for (int n = 0; n < NF; ++n) kf[n] = load_kfrag(sm + kslot(min(par, last)), n);
+    }
+    const int nrounds = (ntiles + 1) / 2;  // round r: tiles 2r and 2r+1
+    auto do_round = [&](v16f(&cur)[2][2], v16f(&next)[2][2], int r) {
+      const int jj = 2 * r;
+      // tiles jj .. jj+3 must have landed (this round's and the next round's, whose fragments this round
+      // prefetches); tiles jj+4, jj+5 may still be in flight
+      if (jj + 5 <= last) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(2 * KPW));
+      else HX_WAIT_VM0();
+      __syncthreads();  // ... for every wave; and every wave is done with tiles jj-2 and jj-1: their slots are free
+      if (jj + 6 < ntiles) issue_k(jj + 6, kslot(jj + 6));
+      if (jj + 7 < ntiles) issue_k(jj + 7, kslot(jj + 7));
+      // The last round multiplies out of registers (what its refills read is not used), and every wave has finished
+      // its real fragment reads before this round's barrier: the whole ring is free, and pass 2's first tiles go out
+      // now instead of after the pass.
+      if (r == nrounds - 1) issue_pass2_prologue();
+      const int t = jj + par;
+      round(cur, next, t, tc);
+      tc = t < ntiles ? t : -1;
+    };
+    for (int r = 0; r < nrounds; r += 2) {
+      do_round(ca, cb, r);
+      if (r + 1 < nrounds) do_round(cb, ca, r + 1);
+    }
+    if (pair_active && tc >= 0) {  // the last tile's scores: round r wrote cb when r is even, ca when it is odd
+      if ((nrounds - 1) & 1) {
+#pragma unroll
+        for (int n = 0; n < NF; ++n) reduce_part(ca, n);
+      } else {
+#pragma unroll
+        for (int n = 0; n < NF; ++n) reduce_part(cb, n);
+      }
+    }
+    const float m_own = att_max_across_halves(smx[par]);        // this wave's queries, its parity's tiles
+    const float m_give = att_max_across_halves(smx[par ^ 1]);   // the partner's queries, this wave's tiles
+    if (lane < 32) xch[w * 32 + lane] = m_give;
+    __syncthreads();
+    const float smax = fmaxf(m_own, xch[(w ^ 1) * 32 + q31]);
     neg_m = -(smax * c);  // max(s*c) == max(s)*c for c > 0 (rounding is monotone)
-    __syncthreads();      // all waves done with the last K tiles before pass 2 overwrites the slots
   }
 
-  // ---------------- pass 2 (or the only pass)
+  // ================= pass 2 (MODE 0: the only pass)
   v16f o[DB];
 #pragma unroll
-  for (int d = 0; d < DB; ++d)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) o[d][r] = 0.f;
-  float l4[4] = {0.f, 0.f, 0.f, 0.f};  // four independent partial row sums per lane
-  v8i pf = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int d = 0; d < DB; ++d) o[d] = zero16;
+  float l4[4] = {0.f, 0.f, 0.f, 0.f};  // four independent partial sums of the un-quantised p per lane
 
-  auto softmax_pv = [&](v16f(&s)[2], const uint8_t* sv) {
-    if (!EXACT) {
-      float t0 = s[0][0], t1 = s[1][0];
+  // softmax group g of a tile: scores cur[g / 4][4 * (g % 4) .. + 3] -> dword g of the P fragment
+  auto softmax_group = [&](v16f(&cur)[2], v8i& pf_new, int g) {
+    const int kb = g >> 2, r0 = 4 * (g & 3);
+    float p[4];
 #pragma unroll
-      for (int r = 0; r < 16; r += 2) {
-        t0 = fmaxf(fmaxf(t0, s[0][r]), s[0][r + 1]);
-        t1 = fmaxf(fmaxf(t1, s[1][r]), s[1][r + 1]);
+    for (int b = 0; b < 4; ++b) {
+      // s*c - m fused into one rounding: the score already carries the fp8 MFMA's accumulation rounding, three orders
+      // of magnitude above the difference between one and two roundings here
+      p[b] = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[kb][r0 + b], c, neg_m));
+      l4[b] += p[b];
+    }
+    const int dw = HX_CVT_PK_E4M3(p[0], p[1], pf_new[g], false);
+    pf_new[g] = HX_CVT_PK_E4M3(p[2], p[3], dw, true);
+  };
+
+  // step j: scores of tile j+1 -> next; softmax of tile j (cur) -> pf_new; P.V of tile j-1 (pf_prev)
+  auto step = [&](auto slot_c, auto full_c, v16f(&cur)[2], v16f(&next)[2], v8i& pf_prev, v8i& pf_new, int j) {
+    constexpr int SL = decltype(slot_c)::value;    // == j % 4
+    constexpr bool FULL = decltype(full_c)::value;  // all three parts present, no partial tile involved: no branches
+    const bool has_s = FULL || j + 1 < ntiles, has_sm = FULL || j < ntiles, has_pv = FULL || j >= 1;
+    // DMA issued in steps j-2 and j-1 may stay in flight; everything older (K(j+1), V(j-1) included) has landed.
+    __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(2 * (KPW + VPW)));
+    __syncthreads();
+    const int tk = min(j + 4, last), tv = min(j + 2, last);
+    const uint8_t* sk = sm + ((SL + 1) & 3) * 2 * TILE;         // K(j+1)
+    const uint8_t* sv = sm + ((SL + 3) & 3) * 2 * TILE + TILE;  // V(j-1)
+    constexpr uint32_t kdst = SL * 2 * TILE;                    // K(j+4) replaces K(j)
+    constexpr uint32_t vdst = ((SL + 2) & 3) * 2 * TILE + TILE;  // V(j+2) replaces V(j-2)
+    if (active) {
+      v8i kf[2], vf[2];
+      if (has_pv) {
+        vf[0] = load_vfrag(sv, 0);
+        vf[1] = load_vfrag(sv, 1);
       }
-      float tmax = fmaxf(t0, t1);
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-      const float neg_new = fminf(neg_m, -(tmax * c));
-      const float alpha = __builtin_amdgcn_exp2f(neg_new - neg_m);  // exp2(m_old - m_new); first tile: exp2(-inf) = 0
-      if (__builtin_amdgcn_ballot_w64(neg_new != neg_m)) {  // wave-uniform: most tiles leave every row max alone
+      if (has_s) {
+        kf[0] = load_kfrag(sk, 0);
+        kf[1] = load_kfrag(sk, 1);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      float alpha = 1.f;
+      bool rescale = false;
+      if (!FULL && ragged && j == last) mask_last(cur);
+      float t0 = -__builtin_inff(), t1 = -__builtin_inff();  // MODE 0: the tile's row max, one chain per key block
+      auto tile_max_half = [&](int kb) {
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          if (kb == 0) t0 = att_max3(t0, cur[0][r], cur[0][r + 1]);
+          else t1 = att_max3(t1, cur[1][r], cur[1][r + 1]);
+        }
+      };
+      // MODE 0: new reference point and the factor the older sums shrink by (first tile: exp2(-inf) = 0 on zeros)
+      auto new_reference = [&]() {
+        const float tmax = att_max_across_halves(fmaxf(t0, t1));
+        const float neg_new = fminf(neg_m, -(tmax * c));
+        alpha = __builtin_amdgcn_exp2f(neg_new - neg_m);
+        rescale = __builtin_amdgcn_ballot_w64(neg_new != neg_m) != 0;  // wave-uniform: most tiles leave every row max alone
+        neg_m = neg_new;
 #pragma unroll
         for (int i = 0; i < 4; ++i) l4[i] *= alpha;
+      };
+      // MODE 1: the first softmax groups cover the latency of the fragment reads above.  MODE 0: the first half of
+      // the max reduction does; the second half and the new reference follow the first MFMA, the groups start one
+      // micro-step later and the last micro-step takes what is left.
+      constexpr int GSH = MODE == 0 ? 1 : 0;  // micro-steps the groups are delayed by
+      if (has_sm) {
+        if (MODE == 0) {
+          tile_max_half(0);
+        } else {
+#pragma unroll
+          for (int g = 0; g < GPM; ++g) softmax_group(cur, pf_new, g);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < NM; ++i) {
+        const int h = i >> 1;
+        if ((i & 1) == 0) {
+          if (has_pv) {
+            o[h] = hx_mfma_32x32x64_e4m3(vf[h & 1], pf_prev, o[h]);
+            if (h + 2 < DB) vf[h & 1] = load_vfrag(sv, h + 2);
+          }
+        } else {
+          if (has_s) {
+            next[h & 1] = hx_mfma_32x32x64_e4m3(kf[h & 1], qf[h >> 1], (h >> 1) ? next[h & 1] : zero16);
+            if (h + 2 < DB) kf[h & 1] = load_kfrag(sk, h + 2);
+          }
+        }
+        if (has_sm) {
+          if (MODE == 0 && i == 0) {
+            tile_max_half(1);
+            new_reference();
+          } else {
+            const int g_lo = MODE == 0 ? (i - GSH) * GPM : (i + 1) * GPM;
+            const int g_hi = (MODE == 0 && i == NM - 1) ? 8 : g_lo + GPM;
+#pragma unroll
+            for (int g = g_lo; g < g_hi && g < 8; ++g) softmax_group(cur, pf_new, g);
+          }
+        }
+        // this step's DMA, one instruction per micro-step
+        if (i < KPW) issue_k_one(tk, kdst, i, std::bool_constant<!FULL>{});
+        else if (i < KPW + VPW) issue_v_one(tv, vdst, i - KPW, std::bool_constant<!FULL>{});
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // MODE 0: the sums of the older tiles (P.V of tile j-1 included: it was quantised against the old reference)
+      // shrink by alpha before tile j's P.V is added in the next step
+      if (MODE == 0 && rescale) {
 #pragma unroll
         for (int d = 0; d < DB; ++d)
 #pragma unroll
           for (int r = 0; r < 16; ++r) o[d][r] *= alpha;
       }
-      neg_m = neg_new;
+    } else {
+      issue_k(tk, kdst);
+      issue_v(tv, vdst);
     }
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      float p[16];
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        // s*c - m fused into one rounding: the score already carries the fp8 MFMA's accumulation rounding,
-        // three orders of magnitude above the difference between one and two roundings here
-        p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][r], c, neg_m));
-        l4[r & 3] += p[r];
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        // both halves of the dword are overwritten, so the previous tile's value serves as the tied operand
-        int dw = HX_CVT_PK_E4M3(p[4 * j], p[4 * j + 1], pf[kb * 4 + j], false);
-        pf[kb * 4 + j] = HX_CVT_PK_E4M3(p[4 * j + 2], p[4 * j + 3], dw, true);
-      }
-    }
-#pragma unroll
-    for (int d = 0; d < DB; ++d) o[d] = hx_mfma_32x32x64_e4m3(load_vfrag(sv, d), pf, o[d]);
   };
 
-  for (int t = 0; t < ATT_LEAD && t < ntiles; ++t) {
-    issue_k(t, t % ATT_NS);
-    issue_v(t, t % ATT_NS);
-  }
-  att_wait_tiles<KPW + VPW>(min(ATT_LEAD - 1, ntiles - 1));
+  if (MODE == 0) issue_pass2_prologue();  // (MODE 1: went out under pass 1's last round)
+  __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(3 * KPW + 2 * VPW));  // K(0) has landed
   __syncthreads();
+  v16f sa[2], sb[2];
+  v8i pfA = {0, 0, 0, 0, 0, 0, 0, 0}, pfB = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (active) scores_plain(sm, sa);
   {
-    auto step2 = [&](v16f(&cur)[2], v16f(&next)[2], int j) {
-      if (j + 2 < ntiles) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(KPW + VPW));
-      else HX_WAIT_VM0();
-      __syncthreads();
-      if (active) {
-        if (j + 1 < ntiles) scores(&smem[(j + 1) % ATT_NS][0][0], next);
-        softmax_pv(cur, &smem[j % ATT_NS][1][0]);
-      }
-      // the slot freed by this step's barrier is refilled at the end of the step: four DMA instructions in a row hold
-      // the issuing wave up, and here nothing of this step is left to wait behind them (2 % against the top of the step)
-      if (j + ATT_LEAD < ntiles) {
-        issue_k(j + ATT_LEAD, (j + ATT_LEAD) % ATT_NS);
-        issue_v(j + ATT_LEAD, (j + ATT_LEAD) % ATT_NS);
-      }
-    };
-    v16f sa[2], sb[2];
-    if (active) scores(&smem[0][0][0], sa);
-    int j = 0;
-    for (; j + 1 < ntiles; j += 2) {
-      step2(sa, sb, j);
-      step2(sb, sa, j + 1);
+    using std::integral_constant;
+    const integral_constant<int, 0> s0;
+    const integral_constant<int, 1> s1;
+    const integral_constant<int, 2> s2;
+    const integral_constant<int, 3> s3;
+    // Steps 0 .. ntiles.  Steps 1 .. ntiles-2 have all three parts and run the branch-free body, four at a time
+    // (slots 1, 2, 3, 0) -- with a partial last tile only up to step ntiles-6, so that neither its masking nor its
+    // DMA ever comes up there; the first step and whatever is left at the end run the guarded body.
+    const int full_to = ragged ? ntiles - 6 : ntiles - 2;
+    step(s0, std::false_type{}, sa, sb, pfA, pfB, 0);
+    int j = 1;
+    for (; j + 3 <= full_to; j += 4) {
+      step(s1, std::true_type{}, sb, sa, pfB, pfA, j);
+      step(s2, std::true_type{}, sa, sb, pfA, pfB, j + 1);
+      step(s3, std::true_type{}, sb, sa, pfB, pfA, j + 2);
+      step(s0, std::true_type{}, sa, sb, pfA, pfB, j + 3);
     }
-    if (j < ntiles) step2(sa, sb, j);
+    for (; j <= ntiles; j += 4) {  // j % 4 == 1 here
+      step(s1, std::false_type{}, sb, sa, pfB, pfA, j);
+      if (j + 1 <= ntiles) step(s2, std::false_type{}, sa, sb, pfA, pfB, j + 1);
+      if (j + 2 <= ntiles) step(s3, std::false_type{}, sb, sa, pfB, pfA, j + 2);
+      if (j + 3 <= ntiles) step(s0, std::false_type{}, sa, sb, pfA, pfB, j + 3);
+    }
   }
   const float l_lane = (l4[0] + l4[1]) + (l4[2] + l4[3]);
+  const float l = l_lane + __shfl_xor(l_lane, 32);
 
-  __syncthreads();  // every wave is past its last K/V fragment read: the LDS ring can be reused
+  HX_WAIT_VM0();     // the trailing re-fetches have landed ...
+  __syncthreads();  // ... and every wave is past its last fragment read: the ring can be reused
   if (!active) return;
   // ---------------- epilogue: o[db][4a+b] is O[q0 + lane%32][32 db + 8a + 4G + b]
   // A lane holds 4 consecutive columns of its row, so direct stores would write every output line in 16- or
   // 32-byte pieces.  Each wave instead passes its 32 rows through its own part of the LDS, PASS_COLS columns at a
   // time, and writes 16 bytes per lane with consecutive lanes on consecutive bytes of a row.
-  const float l = l_lane + __shfl_xor(l_lane, 32);
   constexpr int ESZ = OUT == HX_F32 ? 4 : 1;
   constexpr int PASS_COLS = OUT == HX_F32 ? D / 2 : D;  // 256 or 128 bytes of a row per pass (128 or 64 for D = 64)
   constexpr int PASS_BYTES = PASS_COLS * ESZ;
@@ -327,7 +543,7 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
   constexpr int RPI = 64 / LPR;                         // rows per store instruction
   constexpr int NDB = PASS_COLS / 32;                   // 32-column accumulator blocks per pass
   static_assert(ATT_WAVES * 32 * RSTR <= ATT_NS * 2 * TILE, "output staging fits the K/V ring");
-  uint8_t* st = &smem[0][0][0] + w * (32 * RSTR);
+  uint8_t* st = sm + w * (32 * RSTR);
   uint8_t* out_rows = (uint8_t*)Out + ((long)bh * S + q0) * D * ESZ;
   const int rb_row = lane / LPR, rb_ch = lane % LPR;
 #pragma unroll
@@ -353,7 +569,7 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_kernel(const uint8_t*
     for (int p = 0; p < 32 / RPI; ++p) {
       const int row = p * RPI + rb_row;
       const v4i v = *(const v4i*)(st + row * RSTR + rb_ch * 16);
-      *(v4i*)(out_rows + ((long)row * D + h * PASS_COLS) * ESZ + rb_ch * 16) = v;
+      if (q0 + row < S) *(v4i*)(out_rows + ((long)row * D + h * PASS_COLS) * ESZ + rb_ch * 16) = v;
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
@@ -420,23 +636,23 @@ __global__ __launch_bounds__(256) void hx_fp8_attention_general(const uint8_t* _
   }
 }
 
-template <int D, int OUT, bool EXACT, bool VSD>
-static void launch_att_kernel(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t S, float c, hipStream_t s) {
+template <int D, int OUT, int MODE, bool VSD>
+static void launch_att_pipe(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t S, float c, hipStream_t s) {
   const int qtiles = (int)((S + ATT_BM - 1) / ATT_BM);
   const int hpx = (int)((BH + 7) / 8);
   const int grid = 8 * hpx * qtiles;
-  hx_launch((hx_fp8_attention_kernel<D, OUT, EXACT, VSD>), dim3(grid), dim3(256), 0, s, (const uint8_t*)q, (const uint8_t*)k,
-                     (const uint8_t*)v, out, (int)S, (int)BH, qtiles, c);
+  hx_launch((hx_fp8_attention_pipe<D, OUT, MODE, VSD>), dim3(grid), dim3(256), 0, s, (const uint8_t*)q, (const uint8_t*)k,
+            (const uint8_t*)v, out, (int)S, (int)BH, qtiles, c);
 }
 
 template <int D, int OUT>
 static int launch_att(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t S, int exact, bool vsd, float c, hipStream_t s) {
   if (exact) {
-    if (vsd) launch_att_kernel<D, OUT, true, true>(q, k, v, out, BH, S, c, s);
-    else launch_att_kernel<D, OUT, true, false>(q, k, v, out, BH, S, c, s);
+    if (vsd) launch_att_pipe<D, OUT, 1, true>(q, k, v, out, BH, S, c, s);
+    else launch_att_pipe<D, OUT, 1, false>(q, k, v, out, BH, S, c, s);
   } else {
-    if (vsd) launch_att_kernel<D, OUT, false, true>(q, k, v, out, BH, S, c, s);
-    else launch_att_kernel<D, OUT, false, false>(q, k, v, out, BH, S, c, s);
+    if (vsd) launch_att_pipe<D, OUT, 0, true>(q, k, v, out, BH, S, c, s);
+    else launch_att_pipe<D, OUT, 0, false>(q, k, v, out, BH, S, c, s);
   }
   hipError_t e = hx_launch_status();
   if (e != hipSuccess) {
@@ -444,6 +660,29 @@ static int launch_att(const void* q, const void* k, const void* v, void* out, in
     return (int)e;
   }
   return 0;
+}
+
+// 1: the MFMA kernel takes these arguments; 0: the plain kernel does.  vsd: V is [S][D] per head.
+static bool att_fast_path(const void* q, const void* k, const void* v, const void* out, int64_t S, int64_t D, int64_t v_stride_d,
+                          int64_t v_stride_s, bool* vsd) {
+  bool fast = (D == 64 || D == 128) && S >= 1 && ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) == 0);
+  *vsd = false;
+  if (v_stride_s == 1 && (v_stride_d == S || D == 1)) {
+    *vsd = false;                                  // [D][S] per head: rows of S bytes, fetched in 16-byte pieces
+    if (S % 16 != 0) fast = false;
+  } else if (v_stride_d == 1 && (v_stride_s == D || S == 1)) {
+    *vsd = true;                                   // [S][D] per head
+  } else {
+    fast = false;
+  }
+  return fast;
+}
+
+extern "C" int hx_fp8_attention_path(int64_t BH, int64_t S, int64_t D, int64_t v_stride_d, int64_t v_stride_s, const void* q,
+                                     const void* k, const void* v, const void* out) {
+  bool vsd;
+  (void)BH;
+  return att_fast_path(q, k, v, out, S, D, v_stride_d, v_stride_s, &vsd) ? 1 : 0;
 }
 
 extern "C" int hx_fp8_attention(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t S, int64_t D,
@@ -469,10 +708,8 @@ extern "C" int hx_fp8_attention(const void* q, const void* k, const void* v, voi
   hipStream_t s = (hipStream_t)stream;
   // the softmax scale in base 2, evaluated the way the reference does: double arithmetic, rounded to fp32 once
   const float c = (float)((1.0 / sqrt((double)(scale_dim > 0 ? scale_dim : (D > 0 ? D : 1)))) * 1.44269504);
-  bool vsd = false, fast = (D == 64 || D == 128) && (S % ATT_BN) == 0 && ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) == 0);
-  if (v_stride_s == 1 && (v_stride_d == S || D == 1)) vsd = false;       // [D][S] per head
-  else if (v_stride_d == 1 && (v_stride_s == D || S == 1)) vsd = true;   // [S][D] per head
-  else fast = false;
+  bool vsd = false;
+  const bool fast = att_fast_path(q, k, v, out, S, D, v_stride_d, v_stride_s, &vsd);
   if (!fast) {  // any other shape, alignment or V striding within a head (heads are D*S elements apart)
     if (D > 256 || D < 1 || BH >= 65536) {
       hx_set_error("hx_fp8_attention: unsupported shape S=%lld D=%lld BH=%lld (MFMA kernel: D in {64,128}, S %% 64 == 0; plain kernel: D <= 256, BH < 65536)",

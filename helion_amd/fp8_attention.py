@@ -16,7 +16,7 @@ def fp8_attention_kernel(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batc
     [batch, heads, seq, dim] float8_e4m3fn.  ``exact_max=True`` (default) quantises the un-normalised
     probabilities against the exact row max, which is what the reference computes when its kernel body
     is executed with one tile per loop; ``exact_max=False`` is the single-pass online softmax."""
-    return fp8_attention_call(q, k, v, batch, heads, out_dtype, exact_max)
+    return fp8_attention_call(q, k, v, batch, heads, out_dtype, int(exact_max))
 
 
 def preprocess_fp8_attention_inputs(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):

@@ -85,7 +85,7 @@ def _(x, y, scale_a, scale_b, out_dtype):
 
 # ------------------------------------------------------------------------------ fp8 attention
 def _fp8_attention_impl(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batch: int, heads: int,
-                     out_dtype: torch.dtype, exact_max: bool) -> torch.Tensor:
+                     out_dtype: torch.dtype, exact_max: int) -> torch.Tensor:
     _require_cuda(q, k, v)
     for t in (q, k, v):
         if t.dtype != torch.float8_e4m3fn:
@@ -100,7 +100,7 @@ def _fp8_attention_impl(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batch
     if out_dtype not in (torch.float8_e4m3fn, torch.float32):
         raise TypeError(f"unsupported out_dtype {out_dtype}")
     d_true = d
-    if d not in (64, 128) and 0 < d < 128 and s % 64 == 0:
+    if d not in (64, 128) and 0 < d < 128:
         # zero-pad the head dimension to what the MFMA kernel takes: q.k and the other output columns are unchanged,
         # the softmax scale still comes from the true head dimension
         dp = 64 if d < 64 else 128
@@ -113,12 +113,16 @@ def _fp8_attention_impl(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batch
     # memory (strides (S*D, 1, D)); the kernel reads that layout directly, so only other stridings are copied.
     if bh > 1 and v.stride(0) != s * d or v.stride()[1:] not in ((s, 1), (1, d)):
         v = v.contiguous()
+    if v.stride()[1:] == (s, 1) and s % 16 != 0 and d in (64, 128) and s > 1:
+        # [D][S] rows that are not a multiple of 16 bytes cannot be fetched in 16-byte pieces: hand the MFMA kernel the
+        # [S][D] layout instead (one copy) rather than fall to the plain kernel
+        v = v.transpose(1, 2).contiguous().transpose(1, 2)
     out = torch.empty((batch, heads, s, d), dtype=out_dtype, device=q.device)
     if bh == 0 or s == 0:
         return out
     lib = _lib.load()
     rc = lib.hx_fp8_attention(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), bh, s, d, d_true, v.stride(1),
-                              v.stride(2), _DT[out_dtype], 1 if exact_max else 0, _stream_ptr(q.device))
+                              v.stride(2), _DT[out_dtype], int(exact_max), _stream_ptr(q.device))
     _lib.check(rc, "hx_fp8_attention")
     return out if d == d_true else out[..., :d_true].contiguous()
 

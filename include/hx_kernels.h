@@ -89,11 +89,14 @@ int hx_fp8_gemm_path(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k
  * scale_dim: the head dimension the softmax scale 1/sqrt(.) is taken from; 0 = D.  (A caller whose head dimension is
  *   not 64 or 128 can zero-pad q, k and v to one of them, pass the true one here and drop the padded output columns:
  *   zero columns change neither q.k nor the other output columns.  The Python op does this.)
- * MFMA kernel: D == 128 or 64, S % 64 == 0, 16-byte aligned pointers, v in one of the two layouts above.  Every other
- * shape with D <= 256 and BH < 65536 (and any v strides within a head) runs a plain kernel that always computes the
- * exact-max form. */
+ * MFMA kernel: D == 128 or 64, any S (a partial last key tile is masked), 16-byte aligned pointers, v in one of the
+ * two layouts above (the [D][S] layout needs S % 16 == 0: its rows are fetched in 16-byte pieces).  Every other shape
+ * with D <= 256 and BH < 65536 (and any v strides within a head) runs a plain kernel that always computes the
+ * exact-max form.  hx_fp8_attention_path: 1 = the MFMA kernel would run, 0 = the plain one. */
 int hx_fp8_attention(const void* q, const void* k, const void* v, void* out, int64_t BH, int64_t S, int64_t D,
                      int64_t scale_dim, int64_t v_stride_d, int64_t v_stride_s, int out_dtype, int exact_max, void* stream);
+int hx_fp8_attention_path(int64_t BH, int64_t S, int64_t D, int64_t v_stride_d, int64_t v_stride_s, const void* q,
+                          const void* k, const void* v, const void* out);
 
 /* Replaces the device side of `moe_matmul_ogs(A, W, expert_token_counts, expert_token_offsets,
  * sorted_to_orig_token_idx, max_T_per_expert_tensor)` (reference: examples/moe_matmul_ogs.py:25-80;

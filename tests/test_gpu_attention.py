@@ -7,12 +7,17 @@ import pytest
 import torch
 
 import helion_amd as hx
-from helion_amd import inputs
+from helion_amd import _lib, inputs
 from oracle import oracle as orc
 from tests._util import TOL, rel_err
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
+# The online mode (exact_max=False) is NOT the parity mode: it restates the reference body with 64-key tiles, which is
+# outside the 2e-2 bar against ref-eager by construction.  Against the 64-key tiled walk of the same lines it is
+# asserted at 3e-2 (observed 3e-3 .. 2.1e-2): on top of the exact mode's P-rounding flips (the fp8 MFMA's inexact
+# accumulation), a score that is the running maximum of its row moves the quantisation grid of everything after it.
+TOL_ONLINE = 3e-2
 E4M3 = torch.float8_e4m3fn
 G = pathlib.Path(__file__).resolve().parent / "golden"
 
@@ -37,13 +42,17 @@ def test_exact_max_vs_oracle(b, h, s, d):
     assert (out8.cpu().view(torch.uint8) == ref8.view(torch.uint8)).float().mean().item() > 0.98
 
 
-@pytest.mark.parametrize("b,h,s,d", [(2, 4, 256, 64), (1, 2, 512, 128)])
-def test_online_mode_tracks_the_oracle_loosely(b, h, s, d):
-    # running-max quantisation of P deviates by a few percent from the exact-max reference by construction
+@pytest.mark.parametrize("b,h,s,d", [(2, 4, 256, 64), (1, 2, 512, 128), (1, 3, 1024, 128), (1, 2, 333, 128), (2, 1, 200, 64)])
+def test_online_mode_vs_the_tiled_oracle(b, h, s, d):
+    """exact_max=False is the reference kernel body with its key loop in 64-key tiles (what the compiled kernel
+    executes): parity bar against that walk of the same lines; against the one-tile (ref-eager) form it deviates by a
+    few percent by construction (P is quantised against the running max)."""
     q, k, v = inputs.attention_inputs(b, h, s, d, seed=5)
-    ref = orc.fp8_attention(q, k, v, b, h, torch.float32)
-    out = _run(q, k, v, b, h, out_dtype=torch.float32, exact_max=False)
-    assert rel_err(out, ref) <= 0.08
+    qd, kd = q.to(DEV), k.to(DEV)
+    v_sd = v.to(DEV).transpose(1, 2).contiguous().transpose(1, 2)  # the layout the reference's preprocessing hands over
+    out = hx.fp8_attention_kernel(qd, kd, v_sd, b, h, out_dtype=torch.float32, exact_max=False)
+    assert rel_err(out, orc.fp8_attention_tiled(q, k, v, b, h, 64, torch.float32)) <= TOL_ONLINE
+    assert rel_err(out, orc.fp8_attention(q, k, v, b, h, torch.float32)) <= 0.08
 
 
 def test_golden_fixture():
@@ -83,10 +92,36 @@ def test_tritonbench_thunk_and_layout():
     assert rel_err(out, orc.fp8_attention(q8, k8, v8, 2, 3)) <= 0.08
 
 
-@pytest.mark.parametrize("b,h,s,d", [(1, 2, 100, 64), (2, 1, 70, 80), (1, 3, 64, 32), (1, 1, 1, 16), (1, 2, 1100, 128), (1, 1, 130, 256)])
-def test_other_shapes_run_the_plain_kernel(b, h, s, d):
-    """Sequence lengths that are not a multiple of 64 and head dims other than 64 / 128: exact-max form, both V layouts,
-    both output types."""
+def _path(qd, kd, vd):
+    bh, s, d = qd.shape
+    return _lib.load().hx_fp8_attention_path(bh, s, d, vd.stride(1), vd.stride(2), qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), qd.data_ptr())
+
+
+@pytest.mark.parametrize("b,h,s,d", [(1, 2, 100, 64), (1, 2, 16, 128), (1, 1, 48, 128), (2, 2, 80, 128), (2, 1, 333, 128), (1, 1, 400, 128),
+                                     (1, 2, 1000, 64), (1, 2, 1100, 128), (1, 1, 7, 64), (1, 1, 1, 128), (1, 3, 4100, 128)])
+def test_any_sequence_length_runs_the_mfma_kernel(b, h, s, d):
+    """examples/fp8_attention.py:59,66 tile any seq_len.  The MFMA kernel masks a partial last key tile (and partial
+    last query rows); both V layouts take it ([D][S] rows must be a multiple of 16 bytes to be fetched in place -
+    otherwise the op hands the kernel the [S][D] order), both modes, both output types."""
+    q, k, v = inputs.attention_inputs(b, h, s, d, seed=s + d)
+    ref32 = orc.fp8_attention(q, k, v, b, h, torch.float32)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    v_sd = vd.transpose(1, 2).contiguous().transpose(1, 2)           # [BH, D, S] view of [BH, S, D] memory
+    assert _path(qd, kd, v_sd) == 1
+    if s > 1:
+        assert _path(qd, kd, vd) == (1 if s % 16 == 0 else 0)
+    assert rel_err(hx.fp8_attention_kernel(qd, kd, v_sd, b, h, out_dtype=torch.float32), ref32) <= TOL
+    assert rel_err(hx.fp8_attention_kernel(qd, kd, vd, b, h, out_dtype=torch.float32), ref32) <= TOL
+    out8 = hx.fp8_attention_kernel(qd, kd, v_sd, b, h)
+    assert out8.dtype == E4M3 and rel_err(out8, orc.fp8_attention(q, k, v, b, h)) <= 0.08
+    online = hx.fp8_attention_kernel(qd, kd, v_sd, b, h, out_dtype=torch.float32, exact_max=False)
+    assert rel_err(online, orc.fp8_attention_tiled(q, k, v, b, h, 64, torch.float32)) <= TOL_ONLINE
+
+
+@pytest.mark.parametrize("b,h,s,d", [(2, 1, 70, 80), (1, 3, 64, 32), (1, 1, 1, 16), (1, 1, 130, 256), (1, 2, 75, 200)])
+def test_other_head_dims(b, h, s, d):
+    """Head dims other than 64 / 128: up to 128 the op zero-pads onto the MFMA kernel, above that the plain kernel
+    runs; exact-max form, both V layouts, both output types."""
     q, k, v = inputs.attention_inputs(b, h, s, d, seed=s + d)
     ref32 = orc.fp8_attention(q, k, v, b, h, torch.float32)
     qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
@@ -126,9 +161,16 @@ def test_c4_sampled_heads_and_key_permutation():
     q, k, v = inputs.attention_c4()
     qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
     out = hx.fp8_attention_kernel(qd, kd, vd, b, h, out_dtype=torch.float32)
-    for bh in (0, 77, 127):
+    # heads are mapped to XCDs by (head & 7): one head per XCD, among them the first and the last one
+    for bh in (0, 9, 18, 27, 36, 77, 126, 127):
         ref = orc.fp8_attention(q[bh : bh + 1], k[bh : bh + 1], v[bh : bh + 1], 1, 1, torch.float32)
         assert rel_err(out[bh // h, bh % h], ref[0, 0]) <= TOL
+    assert sorted({bh & 7 for bh in (0, 9, 18, 27, 36, 77, 126, 127)}) == list(range(8))
+    # the online mode at full size against the 64-key tiled walk (two heads)
+    online = hx.fp8_attention_kernel(qd, kd, vd, b, h, out_dtype=torch.float32, exact_max=False)
+    for bh in (3, 100):
+        reft = orc.fp8_attention_tiled(q[bh : bh + 1], k[bh : bh + 1], v[bh : bh + 1], 1, 1, 64, torch.float32)
+        assert rel_err(online[bh // h, bh % h], reft[0, 0]) <= TOL_ONLINE
     perm = torch.randperm(s, generator=torch.Generator().manual_seed(1)).to(DEV)
     out_p = hx.fp8_attention_kernel(qd, kd[:, perm].contiguous(), vd[:, :, perm].contiguous(), b, h, out_dtype=torch.float32)
     # same exact row max, same quantisation grid; only MFMA summation order differs
@@ -170,7 +212,7 @@ def test_random_shapes_layouts_vs_oracle():
     rng = np.random.default_rng(99)
     for case in range(20):
         b = int(rng.integers(1, 3)); h = int(rng.integers(1, 6))
-        s = int(rng.choice([64, 128, 192, 320, 448, 512, 704]))
+        s = int(rng.choice([64, 128, 192, 320, 448, 512, 704, 90, 250, 1, 33]))
         d = int(rng.choice([64, 128]))
         v_seq_major = bool(rng.integers(0, 2))
         q, k, v = inputs.attention_inputs(b, h, s, d, seed=1000 + case)
@@ -183,3 +225,5 @@ def test_random_shapes_layouts_vs_oracle():
         assert rel_err(out, ref) <= TOL, (case, b, h, s, d, v_seq_major)
         out8 = hx.fp8_attention_kernel(q.to(DEV), k.to(DEV), vd, b, h)
         assert rel_err(out8, orc.fp8_attention(q, k, v, b, h)) <= 0.08, (case, b, h, s, d, v_seq_major)
+        online = hx.fp8_attention_kernel(q.to(DEV), k.to(DEV), vd, b, h, out_dtype=torch.float32, exact_max=False)
+        assert rel_err(online, orc.fp8_attention_tiled(q, k, v, b, h, 64, torch.float32)) <= TOL_ONLINE, (case, b, h, s, d, v_seq_major)
