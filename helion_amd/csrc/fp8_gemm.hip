@@ -13,6 +13,7 @@
 //   hx_fp8_gemm_general : bounds-checked, arbitrary strides (fallback for ragged/unaligned inputs).
 #include "hx_common.h"
 
+#include <atomic>
 #include <type_traits>
 
 // ------------------------------------------------------------------------------------------
@@ -640,30 +641,74 @@ __global__ __launch_bounds__(512) void hx_fp8_gemm_skinny(const uint8_t* __restr
 // also across the barrier that sums the eight wave partials.
 // ------------------------------------------------------------------------------------------
 #define SKD_MAXS 8
-// FULL: K == 8192, every wave owns exactly 8 k-steps (no per-step predicates).  MB: 16-row blocks of A (M <= 16*MB);
-// every block reuses the B fragment a wave has just assembled, so rows beyond 16 cost MFMAs but no extra traffic.
-template <int OUT, bool FULL, int MB>
+// The last column groups of a launch are handed out dynamically when the caller provides a ticket word: the XCDs of an
+// MI355X do not stream at the same rate (every second one finishes a static share 8-10 % later), and with one workgroup
+// per CU the launch ends with its slowest CU.  Each workgroup multiplies `nstatic` groups of a fixed, strided share and
+// then draws tickets (one fetch-and-add each; compare-and-swap loops of 256 workgroups on one word cost milliseconds)
+// until it is told to stop, so a launch makes (dynamic groups + workgroups) draws.
+// The word needs no initialisation: it holds a 40-bit tag that differs from launch to launch and a 24-bit count.
+// Workgroup 0, which the hardware dispatches first, installs {tag, 0} before anything else; a draw that finds another
+// tag was made before that store landed, waits for the tag and draws again (workgroup 0 waits for nobody, so the wait
+// ends).  The last draw of the launch clears the word, so the replay of a captured launch finds no stale tag.
+__device__ __forceinline__ unsigned long long skd_draw_issue(unsigned long long* word) {
+  // the zero offset is opaque to the compiler on purpose: for an address it can prove uniform it turns the add into a
+  // wave-wide reduction and reads the answer back on the spot, and the answer is to be awaited where it is used
+  long zero = 0;
+  asm volatile("" : "+v"(zero));
+  return __hip_atomic_fetch_add(word + zero, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ int skd_draw_result(unsigned long long* word, unsigned long long old, unsigned long long tag, int nwork,
+                                               int total) {
+  while ((old >> 24) != tag) {
+    while ((__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 24) != tag) __builtin_amdgcn_s_sleep(32);
+    old = skd_draw_issue(word);
+  }
+  const unsigned cnt = (unsigned)(old & 0xFFFFFF);
+  if (cnt + 1 == (unsigned)total) __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return cnt < (unsigned)nwork ? (int)cnt : -1;
+}
+
+template <int OUT, int NS, int MB>
 __global__ __launch_bounds__(512) void hx_fp8_gemm_skinny_direct(const uint8_t* __restrict__ A, const uint8_t* __restrict__ Bt,
                                                                 typename OutT<OUT>::T* __restrict__ C, int M, int N, int K,
                                                                 long lda, long ldb, long ldc, const float* __restrict__ scale_a,
-                                                                const float* __restrict__ scale_b) {
+                                                                const float* __restrict__ scale_b, unsigned long long* tickets,
+                                                                unsigned long long tag) {
   typedef typename OutT<OUT>::T out_t;
   __shared__ __attribute__((aligned(16))) float red[2][SK_WAVES][MB * 4][64];  // [parity][wave][4*mb + r][lane]
+  __shared__ int s_next[2];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int j = lane & 15, g = lane >> 4, odd = j & 1;
   const int steps = K >> 7;
-  const int nmine = FULL ? SKD_MAXS : (steps - w + SK_WAVES - 1) / SK_WAVES;  // this wave's k-steps (wave-uniform)
+  // this wave's k-steps (wave-uniform).  NS > 0: K is NS*1024, every wave has NS steps and the compiler can count the
+  // loads in flight; NS == 0: any K % 128 == 0, the steps are guarded at run time and every wait is for all loads.
+  constexpr bool FULL = NS > 0;
+  const int nmine = FULL ? NS : (steps - w + SK_WAVES - 1) / SK_WAVES;
 
-  const int ncg = (N + 15) >> 4;
-  const int my_groups = (ncg - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+  const int ncg = (N + 15) >> 4, grid = (int)gridDim.x;  // grid <= ncg: every workgroup has a first group, its own index
+  const bool dynamic = MB == 1 && tickets != nullptr && ncg > grid;  // (the 32-row variant has no registers to spare)
+  // static share: groups b, b + grid, ... (nstatic of them, all but the last two full rounds); ticket t is group
+  // nstatic*grid + t
+  const int nstatic = dynamic ? max(1, ncg / grid - 2) : 0x7fffffff;
+  const int first_ticket = dynamic ? nstatic * grid : 0, nwork = ncg - first_ticket, ndraws = nwork + grid;
+  if (dynamic && blockIdx.x == 0 && tid == 0)
+    __hip_atomic_store(tickets, tag << 24, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  int cg = (int)blockIdx.x, cg1;  // the group being multiplied and the one after it (-1: none)
+  if (nstatic > 1) {
+    cg1 = cg + grid < ncg ? cg + grid : -1;
+  } else {
+    if (tid == 0) s_next[0] = skd_draw_result(tickets, skd_draw_issue(tickets), tag, nwork, ndraws);
+    __syncthreads();
+    const int t1 = __builtin_amdgcn_readfirstlane(s_next[0]);
+    cg1 = t1 >= 0 ? first_ticket + t1 : -1;
+  }
 
   // per-lane source pointers of a column group (rows clamp to N-1: those columns are never stored)
   const int c_lo = (2 * g + odd) * 16, c_hi = (2 * g + (odd ^ 1)) * 16;
   const uint8_t *p0 = Bt, *p1 = Bt;
-  auto point_at = [&](int gi) {
-    const int cg = blockIdx.x + gi * gridDim.x;
+  auto point_at = [&](int cg) {
     p0 = Bt + (long)min(cg * 16 + (j >> 1), N - 1) * ldb + c_lo + (long)w * 128;
     p1 = Bt + (long)min(cg * 16 + 8 + (j >> 1), N - 1) * ldb + c_hi + (long)w * 128;
   };
@@ -673,40 +718,55 @@ __global__ __launch_bounds__(512) void hx_fp8_gemm_skinny_direct(const uint8_t* 
     x1[s] = __builtin_nontemporal_load((const v4i*)(p1 + (long)s * SK_WAVES * 128));
   };
   // the B stream starts before anything else touches memory
-  if (my_groups > 0) {
-    point_at(0);
+  point_at(cg);
 #pragma unroll
-    for (int s = 0; s < SKD_MAXS; ++s)
-      if (FULL || s < nmine) load_step(s);
-  }
+  for (int s = 0; s < SKD_MAXS; ++s)
+    if (FULL ? s < NS : s < nmine) load_step(s);
 
-  // ---- A fragments: lane (m = 16*mb + j, g) holds A[m][128*(w + 8s) + 32g .. +31]
+  // ---- A fragments, fetched exactly like the B rows (whole 128-byte lines per instruction, one exchange between
+  // neighbouring lanes): lane (j, g) ends up with A[16*mb + (j>>1) + 8*(j&1)][128*(w + 8s) + 32g .. +31], i.e. MFMA row i
+  // is matrix row (i>>1) + 8*(i&1) of the block - the store below undoes that.  (Every CU reads the same A at the same
+  // moment; with 16 rows x 32 bytes per instruction, each line fetched by two instructions, those reads held the first
+  // column group up for 3 us.)
   v8i af[MB][SKD_MAXS];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
-    const uint8_t* ap = A + (long)min(mb * 16 + j, M - 1) * lda + g * 32 + (long)w * 128;
+    const uint8_t* ap0 = A + (long)min(mb * 16 + (j >> 1), M - 1) * lda + c_lo + (long)w * 128;
+    const uint8_t* ap1 = A + (long)min(mb * 16 + 8 + (j >> 1), M - 1) * lda + c_hi + (long)w * 128;
 #pragma unroll
     for (int s = 0; s < SKD_MAXS; ++s)
-      if (FULL || s < nmine) {
-        const v4i* p = (const v4i*)(ap + (long)s * SK_WAVES * 128);
-        v4i lo = p[0], hi = p[1];
-        af[mb][s] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      if (FULL ? s < NS : s < nmine) {
+        const v4i a0 = *(const v4i*)(ap0 + (long)s * SK_WAVES * 128);
+        const v4i a1 = *(const v4i*)(ap1 + (long)s * SK_WAVES * 128);
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          af[mb][s][d] = odd ? a1[d] : a0[d];
+          af[mb][s][4 + d] = __builtin_amdgcn_mov_dpp(odd ? a0[d] : a1[d], 0xB1, 0xF, 0xF, true);  // from lane ^ 1
+        }
+        if (MB > 1) __builtin_amdgcn_sched_barrier(0);  // bounds the raw lines in flight (registers)
       }
   }
   float alpha = 1.f;
   if (scale_a) alpha = *scale_a;
   if (scale_b) alpha = alpha * *scale_b;
 
-  int parity = 0;
-  for (int gi = 0; gi < my_groups; ++gi) {
-    const bool more = gi + 1 < my_groups;
-    if (more) point_at(gi + 1);
+  int parity = 0, gi = 0;
+  // One column group.  Whether a next group exists is a compile-time property of the body: with the refill loads under
+  // a run-time condition the compiler cannot count the loads in flight and waits for the newest ones, i.e. for one full
+  // memory latency per group.
+  auto one_group = [&](auto more_c) {
+    constexpr bool more = decltype(more_c)::value;
+    // the ticket for the group after next is drawn now; its answer is picked up just before this group's barrier
+    const bool draws = more && gi + 2 >= nstatic;  // uniform; no next group: told to stop (or nothing is handed out)
+    unsigned long long drawn = 0;
+    if (draws && tid == 0) drawn = skd_draw_issue(tickets);
+    if (more) point_at(cg1);
     v4f acc[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[mb] = (v4f){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < SKD_MAXS; ++s)
-      if (FULL || s < nmine) {
+      if (FULL ? s < NS : s < nmine) {
         v8i bf;
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
@@ -719,24 +779,36 @@ __global__ __launch_bounds__(512) void hx_fp8_gemm_skinny_direct(const uint8_t* 
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) acc[mb] = hx_mfma_16x16x128_e4m3(af[mb][s], bf, acc[mb]);
       }
-    // ---- sum the 8 wave partials: acc[mb][r] is C[16mb + 4g + r][column of lane j = cg*16 + (j>>1) + 8*(j&1)]
-    const int cg = blockIdx.x + gi * gridDim.x;
+    // ---- sum the 8 wave partials: acc[mb][r] belongs to MFMA row 4g + r, column j (matrix rows / columns as below)
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
       for (int r = 0; r < 4; ++r) red[parity][w][4 * mb + r][lane] = acc[mb][r];
+    if (draws && tid == 0) s_next[gi & 1] = skd_draw_result(tickets, drawn, tag, nwork, ndraws);
     __syncthreads();
     if (tid < 256 * MB) {  // MB <= 2: 512 threads cover 16*MB rows x 16 columns
       const int l2 = tid & 63, rr = tid >> 6;  // rr = 4*mb + r
       float sum = 0.f;
 #pragma unroll
       for (int ww = 0; ww < SK_WAVES; ++ww) sum += red[parity][ww][rr][l2];
-      const int j2 = l2 & 15;
-      const int m = 16 * (rr >> 2) + 4 * (l2 >> 4) + (rr & 3), n = cg * 16 + (j2 >> 1) + 8 * (j2 & 1);
+      const int j2 = l2 & 15, i2 = 4 * (l2 >> 4) + (rr & 3);  // MFMA column / row of this value
+      const int m = 16 * (rr >> 2) + (i2 >> 1) + 8 * (i2 & 1), n = cg * 16 + (j2 >> 1) + 8 * (j2 & 1);
       if (m < M && n < N) C[(long)m * ldc + n] = (out_t)(sum * alpha);
     }
     parity ^= 1;  // the next group writes the other buffer, so one barrier per group is enough
-  }
+    int cg2 = -1;  // the group after next
+    if (draws) {
+      const int t2 = __builtin_amdgcn_readfirstlane(s_next[gi & 1]);  // slot gi & 1 is rewritten two barriers from here
+      cg2 = t2 >= 0 ? first_ticket + t2 : -1;
+    } else if (more && gi + 2 < nstatic) {
+      cg2 = cg1 + grid < ncg ? cg1 + grid : -1;
+    }
+    cg = cg1;
+    cg1 = cg2;
+    ++gi;
+  };
+  while (cg1 >= 0) one_group(std::true_type{});
+  one_group(std::false_type{});
 }
 
 // ------------------------------------------------------------------------------------------
@@ -900,6 +972,22 @@ extern "C" int hx_fp8_gemm_path(int64_t M, int64_t N, int64_t K, int64_t lda, in
   return 0;
 }
 
+static std::atomic<unsigned long long> g_skd_launches{0};
+
+template <int OUT, int MB, typename... Args>
+static void launch_skinny_direct(int ns, int grid, hipStream_t stream, Args... args) {
+  switch (ns) {  // k-steps per wave as a compile-time constant where K allows it
+#define HX_SKD_CASE(NS) \
+  case NS:              \
+    hx_launch((hx_fp8_gemm_skinny_direct<OUT, NS, MB>), dim3(grid), dim3(512), 0, stream, args...); \
+    break;
+    HX_SKD_CASE(1) HX_SKD_CASE(2) HX_SKD_CASE(3) HX_SKD_CASE(4) HX_SKD_CASE(5) HX_SKD_CASE(6) HX_SKD_CASE(7) HX_SKD_CASE(8)
+#undef HX_SKD_CASE
+    default:
+      hx_launch((hx_fp8_gemm_skinny_direct<OUT, 0, MB>), dim3(grid), dim3(512), 0, stream, args...);
+  }
+}  // makes the ticket tag of every decode launch different
+
 template <int OUT>
 static void launch_kmajor(int path, const void* a, const void* bt, void* c, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                           int64_t ldc, const float* sa, const float* sb, void* ws, size_t ws_bytes, hipStream_t stream) {
@@ -959,24 +1047,28 @@ static void launch_kmajor(int path, const void* a, const void* bt, void* c, int6
                          (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m,
                          tiles_n);
   } else {  // path == 2
-    int dev = 0, cus = 256;
-    (void)hipGetDevice(&dev);
-    (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    const int cus = hx_cu_count();
     const int ncg = (int)((N + 15) / 16);
     const int grid = ncg < cus ? ncg : cus;
-    if (K == 8192 && M <= 16)
-      hx_launch((hx_fp8_gemm_skinny_direct<OUT, true, 1>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
-                         (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb);
-    else if (K == 8192)
-      hx_launch((hx_fp8_gemm_skinny_direct<OUT, true, 2>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
-                         (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb);
-    else if (K < 8192 && M <= 16)
-      hx_launch((hx_fp8_gemm_skinny_direct<OUT, false, 1>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
-                         (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb);
-    else if (K < 8192)
-      hx_launch((hx_fp8_gemm_skinny_direct<OUT, false, 2>), dim3(grid), dim3(512), 0, stream, (const uint8_t*)a,
-                         (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb);
-    else
+    // a ticket word for the dynamic hand-out of column groups (8 bytes of the workspace, any content)
+    unsigned long long* tickets = nullptr;
+    unsigned long long tag = 0;
+    // (worth it from about 12 groups per workgroup: a ticket is a whole group, 4 us of work, and the spread between the
+    // XCDs is 8-10 %; at 7 groups per workgroup tickets measured 0.9 us slower to 0.3 us faster than strided shares, at
+    // 14 groups 3 % faster)
+    if (ws && ws_bytes >= 8 && aligned(ws, 8) && ncg >= 12 * grid && ncg < (1 << 24)) {
+      tickets = (unsigned long long*)ws;
+      tag = (g_skd_launches.fetch_add(1, std::memory_order_relaxed) % ((1ull << 40) - 1)) + 1;  // 1 .. 2^40 - 1
+    }
+    if (K <= 8192) {
+      const int ns = K % 1024 == 0 ? (int)(K / 1024) : 0;
+      if (M <= 16)
+        launch_skinny_direct<OUT, 1>(ns, grid, stream, (const uint8_t*)a, (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K,
+                                     (long)lda, (long)ldb, (long)ldc, sa, sb, tickets, tag);
+      else
+        launch_skinny_direct<OUT, 2>(ns, grid, stream, (const uint8_t*)a, (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K,
+                                     (long)lda, (long)ldb, (long)ldc, sa, sb, tickets, tag);
+    } else
       hx_launch(hx_fp8_gemm_skinny<OUT>, dim3(grid), dim3(512), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
                          (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb);
   }
@@ -1021,7 +1113,8 @@ extern "C" size_t hx_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, i
   if (ldb_k == 1) {  // column-major B: fp32 partial sums when the 128-column tile kernel would split K
     int ktps = 0;
     const int splits = tileN128_splits(M, N, K, &ktps);
-    return splits > 1 ? (size_t)splits * M * N * 4 : 0;
+    if (splits > 1) return (size_t)splits * M * N * 4;
+    return M <= 16 ? 16 : 0;  // the decode kernel' ticket word (dynamic hand-out of column groups)
   }
   if (ldb_n != 1 || K % 16 != 0) return 0;
   if (M > 16 && N % 16 == 0 && ldb_k % 16 == 0) return 0;

@@ -142,9 +142,7 @@ __global__ __launch_bounds__(QZ_THREADS) void hx_amax_final_kernel(const float* 
 }
 
 static int qz_grid(long long n) {
-  int dev = 0, cus = 256;
-  (void)hipGetDevice(&dev);
-  (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  const int cus = hx_cu_count();
   const long long need = (n / QZ_EPT + QZ_THREADS - 1) / QZ_THREADS;
   const long long cap = (long long)cus * 8;
   return (int)(need < 1 ? 1 : (need < cap ? need : cap));

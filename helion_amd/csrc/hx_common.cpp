@@ -2,6 +2,8 @@
 #include <cstdarg>
 #include <cstdio>
 
+#include <hip/hip_runtime.h>
+
 #include "../../include/hx_kernels.h"
 
 static thread_local char g_err[512] = "";
@@ -15,3 +17,16 @@ void hx_set_error(const char* fmt, ...) {
 
 extern "C" const char* hx_last_error(void) { return g_err; }
 extern "C" int hx_version(void) { return 1; }
+
+// Compute units of the current device.  The attribute query costs microseconds, so each device is asked once.
+int hx_cu_count() {
+  static int cached[64];  // 0 = not asked yet (racing first calls write the same value)
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    cached[dev] = cus;
+  }
+  return cached[dev];
+}

@@ -193,6 +193,46 @@ def test_c3_decode_shape_full_oracle():
     assert rel_err(out, ref) <= 1e-2
 
 
+@pytest.mark.parametrize("m,n,k", [
+    (16, 4096 + 16 * 37, 1024), (1, 8208, 2048), (16, 6000, 3072), (7, 4112, 5120), (16, 9000, 7168), (16, 12304, 8192),
+    (24, 5008, 4096), (32, 4128, 8192), (16, 5000, 1152), (20, 4500, 8192 - 128),
+    (16, 16 * 256 * 12, 1024), (3, 16 * 256 * 13 + 40, 2048), (16, 16 * 256 * 12 + 16, 1152),   # enough groups for tickets
+])
+def test_decode_kernel_more_column_groups_than_workgroups(m, n, k):
+    """Every k-steps-per-wave variant of the decode kernel with column groups handed out by ticket (16-row variant) or by
+    stride (32-row variant), against the oracle."""
+    assert _path(m, n, k) == 2
+    a, b, sa, sb = inputs.gemm_scaled(m, n, k, seed=n + k)
+    out = hx.fp8_gemm(a.to(DEV), b.to(DEV), scale_a=sa.to(DEV), scale_b=sb.to(DEV), out_dtype=torch.float32)
+    assert rel_err(out, orc.fp8_gemm(a, b, sa, sb, torch.float32)) <= 1e-4
+
+
+def test_decode_kernel_ticket_word_needs_no_initialisation_and_is_left_clear():
+    lib = _lib.load()
+    m, n, k = 16, 16 * 256 * 12 + 16 * 100 + 5, 2048
+    assert lib.hx_fp8_gemm_workspace_bytes(m, n, k, 1, k) >= 8
+    a, b, sa, sb = inputs.gemm_scaled(m, n, k, seed=11)
+    ad, bd = a.to(DEV), b.T.contiguous().to(DEV)   # [N][K]: the column-major B the kernel reads
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def run(ws):
+        c = torch.zeros((m, n), dtype=torch.float32, device=DEV)
+        rc = lib.hx_fp8_gemm(ad.data_ptr(), bd.data_ptr(), c.data_ptr(), m, n, k, k, 1, k, n, None, None, _lib.HX_F32,
+                             ws.data_ptr() if ws is not None else None, ws.numel() * 8 if ws is not None else 0, stream)
+        assert rc == 0, lib.hx_last_error()
+        torch.cuda.synchronize()
+        return c
+
+    static = run(None)                      # no workspace: strided shares, no tickets
+    assert rel_err(static, orc.fp8_gemm(a, b, out_dtype=torch.float32)) <= 1e-4
+    for fill in (-1, 0x7fffffffffffffff, 0x0123456789abcdef, 1, (5 << 24) | 77):   # stale contents of any kind
+        ws = torch.full((2,), fill, dtype=torch.int64, device=DEV)
+        assert torch.equal(run(ws), static)
+        assert int(ws[0].item()) == 0       # the last draw clears the word ...
+        assert torch.equal(run(ws), static)  # ... and a launch that finds it clear works as well
+        assert int(ws[0].item()) == 0 and int(ws[1].item()) == fill
+
+
 def test_c2_8192_cube_sampled_rows_and_checksum():
     a, b, sa, sb = inputs.gemm_c2()
     ad, bd = a.to(DEV), b.to(DEV)
