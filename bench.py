@@ -365,6 +365,36 @@ def bench_next_rows(steps, warmup):
     t = _time_launches(lambda: hx.moe_routing(big, 8), steps, warmup)
     out["moe_routing_1m"] = hbm(big.numel() * (8 + 8 + 4), t, "hx_moe_routing_kernel count + scan + scatter",
                                 "the same for 1048576 rows (three launches)")
+    del ex, big
+    # The shape of the reference script's own check, check(1000, 500, 200, 30): K = 500 gives 8-byte rows, which the
+    # 16-byte DMA of the MFMA kernels cannot fetch, so it runs the fp32-FMA kernel; K = 504 is the nearest shape the MFMA
+    # kernel takes (partial last k-tile).  Both are launch-latency sized; torch's time is the per-expert loop of
+    # moe_matmul_ogs_reference (index_select, mm, index_copy_) on the same GPU.
+    from helion_amd import _lib
+    lib = _lib.load()
+    for kk in (500, 504):
+        A, W, exs = inputs.moe_inputs(1000, kk, 200, 30, 1, seed=0, dtype=torch.float16, device="cuda")
+        args = hx.moe_matmul_ogs_helion_kernel_args_gen(A, W, exs)
+        counts, offsets, idx = args[2], args[3], args[4]
+        off_host = offsets.tolist()
+
+        def torch_loop():
+            C = torch.zeros(1000, 200, dtype=torch.float16, device="cuda")
+            for e in range(30):
+                if off_host[e + 1] > off_host[e]:
+                    rows = idx[off_host[e]:off_host[e + 1]].long()
+                    C.index_copy_(0, rows, A.index_select(0, rows) @ W[e])
+            return C
+
+        t = _time_launches(lambda: hx.moe_matmul_ogs(*args), steps, warmup)
+        tt = _time_launches(torch_loop, steps, warmup)
+        path = lib.hx_moe_path(1000, kk, 200, 30, 1, A.data_ptr(), W.data_ptr(), A.data_ptr())
+        out[f"moe_reference_check_shape_k{kk}"] = {
+            "workload": f"moe_matmul_ogs T1000 K{kk} N200 E30 fp16 (examples/moe_matmul_ogs.py:186" + (")" if kk == 500 else ", K rounded up to 16-byte rows)"),
+            "kernel": {0: "hx_moe_general (fp32 FMA)", 4: "hx_gemm16_tile128<partial last k-tile> (MFMA)"}.get(path, str(path)),
+            "hx_moe_path": path, "us_per_launch": t["median_ms"] * 1e3, "torch_per_expert_loop_us": tt["median_ms"] * 1e3,
+            "note": "launch-latency sized (0.2 GFLOP); no roofline fraction is meaningful",
+        }
     return out
 
 

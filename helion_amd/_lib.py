@@ -33,6 +33,7 @@ _SIGNATURES = {
          _c.c_int64, _c.c_int, _c.c_int, _c.c_void_p],
     ),
     "hx_fp8_attention_path": (_c.c_int, [_c.c_int64] * 5 + [_c.c_void_p] * 4),
+    "hx_moe_path": (_c.c_int, [_c.c_int64] * 5 + [_c.c_void_p] * 3),
     "hx_moe_grouped_gemm": (
         _c.c_int,
         [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int64,

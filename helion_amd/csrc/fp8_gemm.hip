@@ -1114,7 +1114,8 @@ extern "C" size_t hx_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, i
     int ktps = 0;
     const int splits = tileN128_splits(M, N, K, &ktps);
     if (splits > 1) return (size_t)splits * M * N * 4;
-    return M <= 16 ? 16 : 0;  // the decode kernel' ticket word (dynamic hand-out of column groups)
+    // the decode kernel's ticket word (dynamic hand-out of column groups), used from 12 groups per CU of an MI355X
+    return M <= 16 && K <= 8192 && (N + 15) / 16 >= 12 * 256 ? 16 : 0;
   }
   if (ldb_n != 1 || K % 16 != 0) return 0;
   if (M > 16 && N % 16 == 0 && ldb_k % 16 == 0) return 0;

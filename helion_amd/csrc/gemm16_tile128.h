@@ -23,7 +23,9 @@
 #define G128_BN 128
 #define G128_TILE_BYTES (128 * 128)
 
-template <bool BF, int MODE, bool BCOL = false, int NS = 2>
+// KTAIL: K is any multiple of 8 (16-byte rows): the last k-tile may be partial.  Its DMA re-reads valid chunks / k rows
+// instead of running off the operands, and the part past K is zeroed in LDS once it has landed.
+template <bool BF, int MODE, bool BCOL = false, int NS = 2, bool KTAIL = false>
 __global__ __launch_bounds__(256, 2) void hx_gemm16_tile128(const uint8_t* __restrict__ A, const uint8_t* __restrict__ W,
                                                            void* __restrict__ Cv, const int* __restrict__ num_tiles,
                                                            const MoeTile* __restrict__ table, const int32_t* __restrict__ idx, int T,
@@ -64,7 +66,10 @@ __global__ __launch_bounds__(256, 2) void hx_gemm16_tile128(const uint8_t* __res
     return (r >= 0 && r < T) ? r : -1;
   };
   const int kt0 = MODE == 2 ? (int)blockIdx.y * d.kt_per_split : 0;
-  const int nk = MODE == 2 ? min(d.kt_per_split, K / MOE_BK - kt0) : K / MOE_BK;
+  static_assert(!KTAIL || MODE != 2, "a partial last k-tile is not combined with split-K");
+  const int nk = MODE == 2 ? min(d.kt_per_split, K / MOE_BK - kt0) : KTAIL ? (K + MOE_BK - 1) / MOE_BK : K / MOE_BK;
+  const int ktail = K - (nk - 1) * MOE_BK;  // valid k of the last tile: 64 unless KTAIL
+  const bool has_tail = KTAIL && ktail != MOE_BK;
   A += (long)kt0 * (MOE_BK * 2);
   const long n0 = (long)tn * G128_BN;
 
@@ -74,7 +79,7 @@ __global__ __launch_bounds__(256, 2) void hx_gemm16_tile128(const uint8_t* __res
 
   // ---- A DMA: wave w owns tile rows [32w, 32w+32), 4 instructions of 8 rows
   const int lrow = lane >> 3, lpos = lane & 7;
-  uint32_t a_vo[4];
+  uint32_t a_vo[4], a_vo_t[KTAIL ? 4 : 1];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     int lr = w * 32 + j * 8 + lrow;
@@ -83,21 +88,25 @@ __global__ __launch_bounds__(256, 2) void hx_gemm16_tile128(const uint8_t* __res
     r = r < 0 ? 0 : r;
     const int swz = ((j & 1) ? 4 + (lrow >> 1) : (lrow >> 1)) & 7;
     a_vo[j] = (uint32_t)(r / a_div) * (uint32_t)(d.lda * 2) + (uint32_t)((lpos ^ swz) * 16);
+    // last, partial k-tile: chunks past K re-read the last valid one
+    if (KTAIL) a_vo_t[j] = (uint32_t)(r / a_div) * (uint32_t)(d.lda * 2) + (uint32_t)(min(lpos ^ swz, ktail / 8 - 1) * 16);
   }
   // ---- W DMA, row-major W: wave w owns k rows [16w, 16w+16), 4 instructions of 4 rows x 256 B; row k = 16w + 4j +
   // (lane>>4), so k & 3 and with it the swizzle do not depend on j.  Chunks past a ragged N re-read the last valid one.
   const uint8_t* We = W + (long)mt.expert * K * N * 2 + n0 * 2 + ((long)kt0 * MOE_BK + w * 16) * d.ldb * 2;  // wave-uniform
   const int wk_l = lane >> 4, wpos = lane & 15;
   const int cmax = (int)((min((long)N - n0, (long)G128_BN) >> 3) - 1);
-  const uint32_t w_vo = (uint32_t)(wk_l * d.ldb * 2 + min(wpos ^ (wk_l << 2), cmax) * 16);
+  const uint32_t w_ch = (uint32_t)(min(wpos ^ (wk_l << 2), cmax) * 16);
+  const uint32_t w_vo = (uint32_t)(wk_l * d.ldb * 2) + w_ch;
   // column-major W: wave w owns tile columns [32w, 32w+32) = rows of W^T, 4 instructions of 8 rows, like A
-  uint32_t wc_vo[BCOL ? 4 : 1];
+  uint32_t wc_vo[BCOL ? 4 : 1], wc_vo_t[BCOL && KTAIL ? 4 : 1];
   if (BCOL) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int col = (int)min(n0 + w * 32 + j * 8 + lrow, (long)N - 1);
       const int swz = ((j & 1) ? 4 + (lrow >> 1) : (lrow >> 1)) & 7;
       wc_vo[j] = (uint32_t)col * (uint32_t)(d.ldb * 2) + (uint32_t)((lpos ^ swz) * 16);
+      if (KTAIL) wc_vo_t[j] = (uint32_t)col * (uint32_t)(d.ldb * 2) + (uint32_t)(min(lpos ^ swz, ktail / 8 - 1) * 16);
     }
   }
   const uint32_t lds0 = hx_lds_addr(&smem[0][0][0]);
@@ -105,12 +114,37 @@ __global__ __launch_bounds__(256, 2) void hx_gemm16_tile128(const uint8_t* __res
     const int kt = min(kt_unclamped, nk - 1), stage = kt_unclamped % NS;
     const uint32_t la = lds0 + (uint32_t)stage * 2 * G128_TILE_BYTES + (uint32_t)w * 32 * 128;
     const uint32_t lw = lds0 + (uint32_t)stage * 2 * G128_TILE_BYTES + G128_TILE_BYTES;
+    const bool tail = has_tail && kt == nk - 1;  // (uniform)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) hx_g2l16_s(A + (long)kt * 128, a_vo[j], la + j * 1024);
+    for (int j = 0; j < 4; ++j) hx_g2l16_s(A + (long)kt * 128, KTAIL && tail ? a_vo_t[KTAIL ? j : 0] : a_vo[j], la + j * 1024);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      if (BCOL) hx_g2l16_s(W + ((long)kt0 + kt) * 128, wc_vo[BCOL ? j : 0], lw + (uint32_t)w * 32 * 128 + j * 1024);
-      else hx_g2l16_s(We + ((long)kt * MOE_BK + 4 * j) * d.ldb * 2, w_vo, lw + (uint32_t)w * 16 * 256 + j * 1024);
+      if (BCOL) {
+        hx_g2l16_s(W + ((long)kt0 + kt) * 128, KTAIL && tail ? wc_vo_t[BCOL && KTAIL ? j : 0] : wc_vo[BCOL ? j : 0],
+                   lw + (uint32_t)w * 32 * 128 + j * 1024);
+      } else if (KTAIL && tail) {  // k rows past K re-read row K-1 (offsets from the tile's first k row)
+        const int kr = min(w * 16 + 4 * j + wk_l, ktail - 1);
+        hx_g2l16_s(We + ((long)kt * MOE_BK - w * 16) * d.ldb * 2, (uint32_t)(kr * d.ldb * 2) + w_ch, lw + (uint32_t)w * 16 * 256 + j * 1024);
+      } else {
+        hx_g2l16_s(We + ((long)kt * MOE_BK + 4 * j) * d.ldb * 2, w_vo, lw + (uint32_t)w * 16 * 256 + j * 1024);
+      }
+    }
+  };
+  // Zero the part of the last k-tile past K, each wave in what it fetched itself (so its own vmcnt wait covers it):
+  // A rows (and the rows of a column-major W) 32w .. 32w+31, chunks ktail/8 .. 7; row-major W: whole k rows >= ktail.
+  auto zero_tail = [&](int stage) {
+    const v4i z = {0, 0, 0, 0};
+    const int row = w * 32 + (lane & 31);
+    for (int c = ktail / 8 + (lane >> 5); c < 8; c += 2) {
+      const int off = row * 128 + ((c ^ ((row >> 1) & 7)) * 16);
+      *(v4i*)(&smem[stage][0][0] + off) = z;
+      if (BCOL) *(v4i*)(&smem[stage][1][0] + off) = z;
+    }
+    if (!BCOL) {
+      const int k = w * 16 + (lane >> 2);
+      if (k >= ktail)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) *(v4i*)(&smem[stage][1][0] + k * 256 + ((lane & 3) * 4 + q) * 16) = z;
     }
   };
 
@@ -167,6 +201,7 @@ __global__ __launch_bounds__(256, 2) void hx_gemm16_tile128(const uint8_t* __res
   // the two copies of the loop body).  Past the last k-tile the refills read the ring's copy of the last tile again.
   auto ktile = [&](int kt) {
     __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 2) * 8));  // this wave's part of tile kt+1 has landed
+    if (has_tail && kt + 1 == nk - 1) zero_tail((kt + 1) % NS);
     __syncthreads();  // ... everybody's has, and every wave has read tile kt out of its stage: that stage is free
     issue(kt + NS);
 #pragma unroll
@@ -180,6 +215,7 @@ __global__ __launch_bounds__(256, 2) void hx_gemm16_tile128(const uint8_t* __res
   };
   for (int t = 0; t < NS; ++t) issue(t);
   __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 1) * 8));
+  if (has_tail && nk == 1) zero_tail(0);
   __syncthreads();
 #pragma unroll
   for (int ks = 0; ks < 4; ++ks) load_ks(ks, 0);

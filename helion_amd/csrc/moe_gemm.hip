@@ -211,18 +211,35 @@ extern "C" size_t hx_moe_workspace_bytes(int64_t T, int64_t E) {
   return b + (size_t)T + 256;
 }
 
-template <bool BF>
-static int launch_moe(const void* A, const void* W, void* C, const int32_t* counts, const int32_t* offsets, const int32_t* idx,
-                      int64_t T, int64_t K, int64_t N, int64_t E, int64_t a_div, void* ws, hipStream_t s) {
-  typedef typename Mfma16<BF>::T T16;
-  const bool fast = (K % MOE_BK == 0) && (N % 8 == 0) && K >= MOE_BK && (((T + a_div - 1) / a_div) * K * 2 < (1LL << 32)) && (N * 4 < (1LL << 31)) && (((uintptr_t)A | (uintptr_t)W | (uintptr_t)C) & 15) == 0;
+// Which kernel multiplies a grouped GEMM: 0 = hx_moe_general (fp32 FMAs; rows that are not 16-byte aligned, K % 8 != 0 or
+// N % 8 != 0), 1 = 32-row tiles, 2 = 128-row tiles, 3 = 256-row tiles, 4 = 128-row tiles with a partial last k-tile
+// (K % 64 != 0); 1-4 are MFMA kernels.
+static int moe_path(const void* A, const void* W, const void* C, int64_t T, int64_t K, int64_t N, int64_t E, int64_t a_div) {
+  const bool fast = (K % 8 == 0) && (N % 8 == 0) && K >= 8 && (((T + a_div - 1) / a_div) * K * 2 < (1LL << 32)) && (N * 4 < (1LL << 31)) &&
+                    (((uintptr_t)A | (uintptr_t)W | (uintptr_t)C) & 15) == 0;
+  if (!fast) return 0;
+  if (K % MOE_BK != 0) return 4;
   // 128-row tiles while the experts are small (less padding in each expert's last row tile) or the 256-row tiles would
   // not fill the chip; 256-row tiles otherwise (half the operand traffic per flop)
   const int64_t tn256 = (N + MOE_BN - 1) / MOE_BN;
   const bool small = E > 0 && (T / E < 512 || ((T + MOE_BM - 1) / MOE_BM + E / 2) * tn256 < 192);
   // a handful of rows in all: 32-row tiles (a quarter of the A bytes per stage, more weight bytes in flight per CU)
-  const bool few = T <= R32_BM;
-  const int bm = fast ? (few ? R32_BM : small ? G128_BM : MOE_BM) : 64;
+  if (T <= R32_BM) return 1;
+  return small ? 2 : 3;
+}
+
+extern "C" int hx_moe_path(int64_t T, int64_t K, int64_t N, int64_t E, int64_t a_div, const void* A, const void* W, const void* C) {
+  if (T < 0 || K < 0 || N < 0 || E < 0 || a_div < 1) return -1;
+  return moe_path(A, W, C, T, K, N, E, a_div);
+}
+
+template <bool BF>
+static int launch_moe(const void* A, const void* W, void* C, const int32_t* counts, const int32_t* offsets, const int32_t* idx,
+                      int64_t T, int64_t K, int64_t N, int64_t E, int64_t a_div, void* ws, hipStream_t s) {
+  typedef typename Mfma16<BF>::T T16;
+  const int path = moe_path(A, W, C, T, K, N, E, a_div);
+  const bool fast = path != 0;
+  const int bm = path == 1 ? R32_BM : path == 3 ? MOE_BM : path == 0 ? 64 : G128_BM;
   const int max_tiles = (int)moe_max_tiles(T, E, bm);
   int* num_tiles = (int*)ws;
   MoeTile* table = (MoeTile*)((uint8_t*)ws + 16);
@@ -248,8 +265,13 @@ static int launch_moe(const void* A, const void* W, void* C, const int32_t* coun
       hx_launch((hx_gemm16_rows32<BF, 3>), dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W,
                          (void*)C, (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, max_tiles, tiles_n,
                          (int)a_div, d);
+    } else if (path == 4) {
+      const int tiles_n = (int)((N + G128_BN - 1) / G128_BN);
+      hx_launch((hx_gemm16_tile128<BF, 0, false, 2, true>), dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A,
+                (const uint8_t*)W, (void*)C, (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, max_tiles,
+                tiles_n, (int)a_div, d);
     } else if (bm == MOE_BM) {
-      const int tiles_n = (int)tn256;
+      const int tiles_n = (int)((N + MOE_BN - 1) / MOE_BN);
       hx_launch((hx_gemm16_tile256<BF, 0>), dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W,
                          (void*)C, (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, max_tiles, tiles_n,
                          (int)a_div, d);

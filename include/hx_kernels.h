@@ -107,12 +107,18 @@ int hx_fp8_attention_path(int64_t BH, int64_t S, int64_t D, int64_t v_stride_d, 
  * HX_F16 for all three; counts [E], offsets [E+1], idx [T] are int32 device arrays.
  * max_T (the numel of the reference's dummy tensor) is accepted for signature parity and is only
  * validated (>= 0); the tile table is built on the device from counts/offsets.
- * workspace: hx_moe_workspace_bytes(T, E) bytes, 16-byte aligned. */
+ * workspace: hx_moe_workspace_bytes(T, E) bytes, 16-byte aligned.
+ * MFMA kernels: K % 8 == 0 and N % 8 == 0 (16-byte rows), 16-byte aligned pointers, A below 4 GB; a K that is not a
+ * multiple of 64 gets a zero-filled last k-tile.  Anything else, e.g. the K = 500 of the reference's own check
+ * (examples/moe_matmul_ogs.py:186, 8-byte rows), runs an fp32-FMA kernel.  hx_moe_path (a_div = 1 for this entry point):
+ * 0 = the FMA kernel, 1 / 2 / 3 = MFMA kernel with 32- / 128- / 256-row tiles, 4 = 128-row tiles with a partial last
+ * k-tile. */
 int hx_moe_grouped_gemm(const void* A, const void* W, void* C, const int32_t* counts,
                         const int32_t* offsets, const int32_t* idx, int64_t T, int64_t K, int64_t N,
                         int64_t E, int64_t max_T, int dtype, void* workspace, size_t workspace_bytes,
                         void* stream);
 size_t hx_moe_workspace_bytes(int64_t T, int64_t E);
+int hx_moe_path(int64_t T, int64_t K, int64_t N, int64_t E, int64_t a_div, const void* A, const void* W, const void* C);
 
 /* hx_moe_grouped_gemm for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, checks, kernels and

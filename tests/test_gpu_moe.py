@@ -21,24 +21,35 @@ def _run(A, W, ex):
     return hx.moe_matmul_ogs(*args)
 
 
-@pytest.mark.parametrize("T,K,N,E,topk,dtype", [
-    (1000, 500, 200, 30, 1, torch.float16),    # examples/moe_matmul_ogs.py:186 (general kernel)
-    (512, 256, 512, 4, 1, torch.bfloat16),     # tile256 kernel
-    (700, 128, 256, 5, 1, torch.float16),
-    (2048, 512, 768, 8, 2, torch.bfloat16),    # top-2 expanded rows
-    (300, 64, 256, 16, 1, torch.bfloat16),     # most tiles nearly empty
-    (37, 100, 19, 3, 1, torch.bfloat16),
-    (512, 128, 384, 4, 1, torch.bfloat16),     # tile256 kernel, ragged last column tile (N % 256 = 128)
-    (600, 64, 1408, 8, 2, torch.float16),      # N = 5.5 tiles
-    (256, 64, 8, 2, 1, torch.bfloat16),        # a single column tile with one valid 16-byte chunk
-    (300, 192, 200, 5, 1, torch.bfloat16),     # N % 8 == 0, nothing else aligned
-    (32, 256, 512, 8, 1, torch.bfloat16),      # a decode batch: the 32-row tile kernel
-    (16, 512, 264, 4, 2, torch.float16),       # ... top-2, ragged last column tile
-    (7, 64, 128, 3, 1, torch.bfloat16),        # ... one k-tile, fewer rows than experts' tiles
-    (24, 1024, 1408, 40, 1, torch.bfloat16),   # ... more experts than rows
+# path: what hx_moe_path reports - 0 the fp32-FMA kernel, 1 / 2 / 3 MFMA with 32- / 128- / 256-row tiles, 4 MFMA with
+# 128-row tiles and a zero-filled partial last k-tile
+@pytest.mark.parametrize("T,K,N,E,topk,dtype,path", [
+    (1000, 500, 200, 30, 1, torch.float16, 0),    # examples/moe_matmul_ogs.py:186: 8-byte rows, no 16-byte DMA
+    (1000, 504, 200, 30, 1, torch.float16, 4),    # ... the nearest shape with 16-byte rows: K = 7 k-tiles + 56
+    (512, 256, 512, 4, 1, torch.bfloat16, 2),
+    (700, 128, 256, 5, 1, torch.float16, 2),
+    (2048, 512, 768, 8, 2, torch.bfloat16, 2),    # top-2 expanded rows
+    (8192, 192, 2048, 2, 1, torch.bfloat16, 3),   # 256-row tiles
+    (300, 64, 256, 16, 1, torch.bfloat16, 2),     # most tiles nearly empty
+    (37, 100, 19, 3, 1, torch.bfloat16, 0),
+    (512, 128, 384, 4, 1, torch.bfloat16, 2),     # ragged last column tile (N % 128 = 0, N % 256 = 128)
+    (600, 64, 1408, 8, 2, torch.float16, 2),      # N = 5.5 tiles of 256
+    (256, 64, 8, 2, 1, torch.bfloat16, 2),        # a single column tile with one valid 16-byte chunk
+    (300, 192, 200, 5, 1, torch.bfloat16, 2),     # N % 8 == 0, nothing else aligned
+    (32, 256, 512, 8, 1, torch.bfloat16, 1),      # a decode batch: the 32-row tile kernel
+    (16, 512, 264, 4, 2, torch.float16, 1),       # ... top-2, ragged last column tile
+    (7, 64, 128, 3, 1, torch.bfloat16, 1),        # ... one k-tile, fewer rows than experts' tiles
+    (24, 1024, 1408, 40, 1, torch.bfloat16, 1),   # ... more experts than rows
+    (300, 8, 64, 3, 1, torch.bfloat16, 4),        # partial last k-tile: the only one, a single chunk
+    (300, 72, 136, 3, 1, torch.float16, 4),       # ... one full tile + 8
+    (1000, 120, 256, 7, 2, torch.bfloat16, 4),    # ... 64 + 56
+    (20, 200, 264, 4, 1, torch.bfloat16, 4),      # ... few rows, 3 tiles + 8
+    (5000, 1000, 512, 3, 1, torch.bfloat16, 4),   # ... large experts: 15 tiles + 40
 ])
-def test_shapes_vs_oracle(T, K, N, E, topk, dtype):
+def test_shapes_vs_oracle(T, K, N, E, topk, dtype, path):
     A, W, ex = inputs.moe_inputs(T // topk, K, N, E, topk, seed=T + K, dtype=dtype)
+    from helion_amd import _lib
+    assert _lib.load().hx_moe_path(A.shape[0], K, N, E, 1, 1 << 20, 1 << 20, 1 << 20) == path
     out = _run(A, W, ex)
     assert out.dtype == dtype and out.shape == (A.shape[0], N)
     assert rel_err(out, orc.moe_matmul_ogs_reference(A, W, ex)) <= 1e-2
