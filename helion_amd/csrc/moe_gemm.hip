@@ -26,29 +26,55 @@ __global__ void hx_moe_prep(const int32_t* __restrict__ counts, const int32_t* _
   const int tid = blockIdx.x * blockDim.x + threadIdx.x, nth = gridDim.x * blockDim.x;
   for (int i = tid; i < T; i += nth) flags[i] = 0;
   if (blockIdx.x != 0) return;
-  // block 0: each thread walks the experts whose index is congruent to it, after a serial prefix
-  // of tile counts (E is small: tens to a few thousand)
-  __shared__ int s_total;
-  if (threadIdx.x == 0) {
-    int t = 0;
-    for (int e = 0; e < E; ++e) {
-      int c = counts[e];
+  // block 0 builds the tile table, 256 experts at a time: tile counts, an exclusive scan of them in LDS, then every
+  // thread fills tiles of the chunk, finding a tile's expert by binary search in the scanned counts
+  __shared__ int s_first[257];  // tiles of the chunk before its expert i; s_first[256] = tiles of the chunk
+  __shared__ int s_start[256], s_cnt[256];
+  __shared__ int s_base;        // tiles before the chunk
+  const int t256 = threadIdx.x;
+  if (t256 == 0) s_base = 0;
+  for (int e0 = 0; e0 < E; e0 += 256) {
+    const int e = e0 + t256;
+    int c = 0, start = 0;
+    if (e < E) {
+      c = counts[e];
       c = c < 0 ? 0 : c;
-      const int start = offsets[e];
+      start = offsets[e];
       // clamp malformed tables so the GEMM never indexes outside idx[0..T)
       if (start < 0 || start > T) c = 0;
       if (c > T - start) c = T - start;
-      const int nt = (c + bm - 1) / bm;
-      for (int i = 0; i < nt && t < max_tiles; ++i, ++t) {
-        table[t].expert = e;
-        table[t].row_start = start + i * bm;
-        table[t].rows = min(bm, c - i * bm);
-        table[t].pad = 0;
-      }
     }
-    s_total = t;
-    *num_tiles = t;
+    s_start[t256] = start;
+    s_cnt[t256] = c;
+    if (t256 == 0) s_first[0] = 0;
+    s_first[t256 + 1] = (c + bm - 1) / bm;
+    __syncthreads();
+    for (int d = 1; d < 256; d <<= 1) {  // inclusive scan (Hillis-Steele), shifted by one
+      const int v = t256 >= d ? s_first[t256 + 1 - d] : 0;
+      __syncthreads();
+      s_first[t256 + 1] += v;
+      __syncthreads();
+    }
+    const int base = s_base, chunk_tiles = s_first[256];
+    for (int i = t256; i < chunk_tiles && base + i < max_tiles; i += 256) {
+      int lo = 0, hi = 256;  // invariant: s_first[lo] <= i < s_first[hi]
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (s_first[mid] <= i) lo = mid; else hi = mid;
+      }
+      const int j = i - s_first[lo];
+      MoeTile mt;
+      mt.expert = e0 + lo;
+      mt.row_start = s_start[lo] + j * bm;
+      mt.rows = min(bm, s_cnt[lo] - j * bm);
+      mt.pad = 0;
+      table[base + i] = mt;
+    }
+    __syncthreads();  // everybody has read s_base and the chunk's arrays
+    if (t256 == 0) s_base = base + chunk_tiles;
+    __syncthreads();
   }
+  if (t256 == 0) *num_tiles = min(s_base, max_tiles);
 }
 
 __global__ void hx_moe_mark(const int* __restrict__ num_tiles, const MoeTile* __restrict__ table, const int32_t* __restrict__ idx,

@@ -45,6 +45,8 @@ def _run(A, W, ex):
     (1000, 120, 256, 7, 2, torch.bfloat16, 4),    # ... 64 + 56
     (20, 200, 264, 4, 1, torch.bfloat16, 4),      # ... few rows, 3 tiles + 8
     (5000, 1000, 512, 3, 1, torch.bfloat16, 4),   # ... large experts: 15 tiles + 40
+    (6000, 64, 64, 700, 1, torch.bfloat16, 2),    # tile table built 256 experts at a time (three chunks, many empty)
+    (9000, 128, 128, 300, 2, torch.float16, 2),   # ... two chunks, top-2
 ])
 def test_shapes_vs_oracle(T, K, N, E, topk, dtype, path):
     A, W, ex = inputs.moe_inputs(T // topk, K, N, E, topk, seed=T + K, dtype=dtype)
