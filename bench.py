@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only c2,c3,c4,c5,next,sib] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only c2,lib,c3,c4,c5,next,sib] [--no-cpu-baseline]
 
 A "step" is one launch of the FP8 GEMM at the headline configuration (M=N=K=8192, e4m3 operands, B column-major,
 per-tensor fp32 scales, bf16 output) with inputs resident in HBM.
@@ -243,6 +243,26 @@ def bench_c2(steps, warmup):
     t = _time_launches(fn, steps, warmup)
     roof = _mfma_roofline(2.0 * 8192**3, t, PEAK_FP8_TFLOPS, FP8_FLOP_PER_CU_CLK, "hx_fp8_gemm_tile256<bf16>", "fp8_gemm_tile256_c2")
     return t, roof
+
+
+def bench_c2_library_baseline(steps, warmup):
+    """The reference's own GPU baseline for this configuration, reference_fp8_gemm_pytorch (examples/fp8_gemm.py:61-78):
+    torch._scaled_mm, i.e. the vendor library (hipBLASLt), on the C2 operands with the same scales and output type, timed
+    with the same protocol right after the headline kernel.  Not part of this library; reported for comparison only."""
+    import torch
+    from helion_amd import inputs
+
+    a, b, sa, sb = inputs.gemm_c2("cuda")
+    try:
+        fn = lambda: torch._scaled_mm(a, b, sa, sb, out_dtype=torch.bfloat16)
+        fn()
+        torch.cuda.synchronize()
+    except Exception as e:  # the library may lack an fp8 solution for this device
+        return {"workload": "torch._scaled_mm (hipBLASLt) on the C2 operands", "error": f"{type(e).__name__}: {e}"[:200]}
+    t = _time_launches(fn, steps, warmup)
+    roof = _mfma_roofline(2.0 * 8192**3, t, PEAK_FP8_TFLOPS, FP8_FLOP_PER_CU_CLK, "hipBLASLt fp8 GEMM behind torch._scaled_mm")
+    return {"workload": "torch._scaled_mm (hipBLASLt) on the C2 operands: reference_fp8_gemm_pytorch, examples/fp8_gemm.py:61-78",
+            "ms_per_launch": t["median_ms"], "value": roof["achieved"], "unit": "TFLOP/s", "roofline": roof}
 
 
 def bench_c3(steps, warmup):
@@ -523,7 +543,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--only", default="c2,c3,c4,c5,next,sib")
+    ap.add_argument("--only", default="c2,lib,c3,c4,c5,next,sib")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-settle", action="store_true", help="skip the settle phase (profiling runs that want few launches)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -558,6 +578,9 @@ def main():
 
     t, roof = bench_c2(args.steps, args.warmup)
     others = {}
+    if "lib" in only:
+        others["c2_library_baseline_scaled_mm"] = bench_c2_library_baseline(args.steps, args.warmup)
+        torch.cuda.empty_cache()
     if "c3" in only:
         others["c3_decode_gemm"] = bench_c3(args.steps, args.warmup)
         torch.cuda.empty_cache()
