@@ -35,7 +35,6 @@ import json
 import os
 import pathlib
 import statistics
-import subprocess
 import sys
 import time
 
@@ -55,7 +54,7 @@ CLOCK_PROBE_TICKS = 5000  # of the 100 MHz counter = 50 us
 
 
 # ----------------------------------------------------------------------------------------------------------------
-# device facts (amdsmi and the amd-smi tool; every field degrades to None when they are unavailable)
+# device facts (amdsmi; every field degrades to None when it is unavailable)
 # ----------------------------------------------------------------------------------------------------------------
 class _Smi:
     def __init__(self):
@@ -72,14 +71,17 @@ class _Smi:
 
     def static(self):
         out = {"market_name": None, "compute_units": None, "max_engine_clock_mhz": None}
-        try:
-            txt = subprocess.run(["amd-smi", "static", "--asic"], capture_output=True, text=True, timeout=30).stdout
-            for line in txt.splitlines():
-                if "MARKET_NAME" in line:
-                    out["market_name"] = line.split(":", 1)[1].strip()
-                    break
-        except Exception:
-            pass
+        # (through the amdsmi module only: starting the amd-smi tool from a process whose GPU is already initialised - it is,
+        # from its first instruction, under a counter-collecting profiler - is an exec the machines here refuse)
+        if self.ok:
+            for getter, key in ((self.m.amdsmi_get_gpu_asic_info, "market_name"), (self.m.amdsmi_get_gpu_board_info, "product_name")):
+                try:
+                    name = getter(self.h).get(key)
+                    if isinstance(name, str) and name.strip() and name.strip().upper() != "N/A":
+                        out["market_name"] = name.strip()
+                        break
+                except Exception:
+                    pass
         if self.ok:
             try:
                 out["compute_units"] = int(self.m.amdsmi_get_gpu_asic_info(self.h)["num_compute_units"])
@@ -387,9 +389,8 @@ def bench_next_rows(steps, warmup):
                                 "the same for 1048576 rows (three launches)")
     del ex, big
     # The shape of the reference script's own check, check(1000, 500, 200, 30): K = 500 gives 8-byte rows, which the
-    # 16-byte DMA of the MFMA kernels cannot fetch, so it runs the fp32-FMA kernel; K = 504 is the nearest shape the MFMA
-    # kernel takes (partial last k-tile).  Both are launch-latency sized; torch's time is the per-expert loop of
-    # moe_matmul_ogs_reference (index_select, mm, index_copy_) on the same GPU.
+    # 128-row MFMA kernel fetches in 4-byte pieces; K = 504 (16-byte rows) for comparison.  Both are launch-latency sized;
+    # torch's time is the per-expert loop of moe_matmul_ogs_reference (index_select, mm, index_copy_) on the same GPU.
     from helion_amd import _lib
     lib = _lib.load()
     for kk in (500, 504):
@@ -411,7 +412,8 @@ def bench_next_rows(steps, warmup):
         path = lib.hx_moe_path(1000, kk, 200, 30, 1, A.data_ptr(), W.data_ptr(), A.data_ptr())
         out[f"moe_reference_check_shape_k{kk}"] = {
             "workload": f"moe_matmul_ogs T1000 K{kk} N200 E30 fp16 (examples/moe_matmul_ogs.py:186" + (")" if kk == 500 else ", K rounded up to 16-byte rows)"),
-            "kernel": {0: "hx_moe_general (fp32 FMA)", 4: "hx_gemm16_tile128<partial last k-tile> (MFMA)"}.get(path, str(path)),
+            "kernel": {0: "hx_moe_general (fp32 FMA)", 4: "hx_gemm16_tile128<partial last k-tile> (MFMA)",
+                       5: "hx_gemm16_tile128<partial last k-tile, A by 4-byte DMA> (MFMA)"}.get(path, str(path)),
             "hx_moe_path": path, "us_per_launch": t["median_ms"] * 1e3, "torch_per_expert_loop_us": tt["median_ms"] * 1e3,
             "note": "launch-latency sized (0.2 GFLOP); no roofline fraction is meaningful",
         }

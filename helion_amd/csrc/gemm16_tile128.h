@@ -25,7 +25,9 @@
 
 // KTAIL: K is any multiple of 8 (16-byte rows): the last k-tile may be partial.  Its DMA re-reads valid chunks / k rows
 // instead of running off the operands, and the part past K is zeroed in LDS once it has landed.
-template <bool BF, int MODE, bool BCOL = false, int NS = 2, bool KTAIL = false>
+// A4 (with KTAIL, row-major W): K is any even number, so the rows of A are only 4-byte aligned: A comes in through the
+// 4-byte DMA, four lanes per 16-byte chunk (the same LDS image from four times the instructions).
+template <bool BF, int MODE, bool BCOL = false, int NS = 2, bool KTAIL = false, bool A4 = false>
 __global__ __launch_bounds__(256, 2) void hx_gemm16_tile128(const uint8_t* __restrict__ A, const uint8_t* __restrict__ W,
                                                            void* __restrict__ Cv, const int* __restrict__ num_tiles,
                                                            const MoeTile* __restrict__ table, const int32_t* __restrict__ idx, int T,
@@ -67,6 +69,8 @@ __global__ __launch_bounds__(256, 2) void hx_gemm16_tile128(const uint8_t* __res
   };
   const int kt0 = MODE == 2 ? (int)blockIdx.y * d.kt_per_split : 0;
   static_assert(!KTAIL || MODE != 2, "a partial last k-tile is not combined with split-K");
+  static_assert(!A4 || (KTAIL && !BCOL), "the 4-byte A path exists for the partial-k-tile kernel with a row-major W");
+  constexpr int DPI = A4 ? 20 : 8;  // DMA instructions per wave and k-tile
   const int nk = MODE == 2 ? min(d.kt_per_split, K / MOE_BK - kt0) : KTAIL ? (K + MOE_BK - 1) / MOE_BK : K / MOE_BK;
   const int ktail = K - (nk - 1) * MOE_BK;  // valid k of the last tile: 64 unless KTAIL
   const bool has_tail = KTAIL && ktail != MOE_BK;
@@ -80,6 +84,20 @@ __global__ __launch_bounds__(256, 2) void hx_gemm16_tile128(const uint8_t* __res
   // ---- A DMA: wave w owns tile rows [32w, 32w+32), 4 instructions of 8 rows
   const int lrow = lane >> 3, lpos = lane & 7;
   uint32_t a_vo[4], a_vo_t[KTAIL ? 4 : 1];
+  // A4: 16 instructions of 2 rows; lane = (row2, chunk position, 4-byte piece); the swizzle (row >> 1) & 7 of tile row
+  // 32w + 2jj + row2 is jj & 7, the same for the whole instruction
+  const int row2 = lane >> 5, lpos4 = (lane >> 2) & 7, piece = lane & 3;
+  uint32_t a_row4[A4 ? 16 : 1];
+  if (A4) {
+#pragma unroll
+    for (int jj = 0; jj < 16; ++jj) {
+      int lr = w * 32 + jj * 2 + row2;
+      lr = lr < mt.rows ? lr : 0;
+      int r = row_of(lr);
+      r = r < 0 ? 0 : r;
+      a_row4[jj] = (uint32_t)(r / a_div) * (uint32_t)(d.lda * 2);
+    }
+  }
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     int lr = w * 32 + j * 8 + lrow;
@@ -115,8 +133,17 @@ __global__ __launch_bounds__(256, 2) void hx_gemm16_tile128(const uint8_t* __res
     const uint32_t la = lds0 + (uint32_t)stage * 2 * G128_TILE_BYTES + (uint32_t)w * 32 * 128;
     const uint32_t lw = lds0 + (uint32_t)stage * 2 * G128_TILE_BYTES + G128_TILE_BYTES;
     const bool tail = has_tail && kt == nk - 1;  // (uniform)
+    if (A4) {
+      const int emax = tail ? ktail - 2 : MOE_BK - 2;  // last valid pair of elements of this k-tile (K is even)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) hx_g2l16_s(A + (long)kt * 128, KTAIL && tail ? a_vo_t[KTAIL ? j : 0] : a_vo[j], la + j * 1024);
+      for (int jj = 0; jj < 16; ++jj) {
+        const int e = min((lpos4 ^ (jj & 7)) * 8 + piece * 2, emax);
+        hx_g2l4_s(A + (long)kt * 128, a_row4[A4 ? jj : 0] + (uint32_t)(e * 2), la + jj * 256);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) hx_g2l16_s(A + (long)kt * 128, KTAIL && tail ? a_vo_t[KTAIL ? j : 0] : a_vo[j], la + j * 1024);
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       if (BCOL) {
@@ -135,10 +162,15 @@ __global__ __launch_bounds__(256, 2) void hx_gemm16_tile128(const uint8_t* __res
   auto zero_tail = [&](int stage) {
     const v4i z = {0, 0, 0, 0};
     const int row = w * 32 + (lane & 31);
-    for (int c = ktail / 8 + (lane >> 5); c < 8; c += 2) {
-      const int off = row * 128 + ((c ^ ((row >> 1) & 7)) * 16);
-      *(v4i*)(&smem[stage][0][0] + off) = z;
-      if (BCOL) *(v4i*)(&smem[stage][1][0] + off) = z;
+    if (A4) {  // 4-byte pieces ktail/2 .. 31 of the row (K even)
+      for (int dw = ktail / 2 + (lane >> 5); dw < 32; dw += 2)
+        *(int*)(&smem[stage][0][0] + row * 128 + (((dw >> 2) ^ ((row >> 1) & 7)) * 16) + (dw & 3) * 4) = 0;
+    } else {
+      for (int c = ktail / 8 + (lane >> 5); c < 8; c += 2) {
+        const int off = row * 128 + ((c ^ ((row >> 1) & 7)) * 16);
+        *(v4i*)(&smem[stage][0][0] + off) = z;
+        if (BCOL) *(v4i*)(&smem[stage][1][0] + off) = z;
+      }
     }
     if (!BCOL) {
       const int k = w * 16 + (lane >> 2);
@@ -200,7 +232,7 @@ __global__ __launch_bounds__(256, 2) void hx_gemm16_tile128(const uint8_t* __res
   // step is the same code (a second register set, alternating, had the compiler shuffle the accumulators between
   // the two copies of the loop body).  Past the last k-tile the refills read the ring's copy of the last tile again.
   auto ktile = [&](int kt) {
-    __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 2) * 8));  // this wave's part of tile kt+1 has landed
+    __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 2) * DPI));  // this wave's part of tile kt+1 has landed
     if (has_tail && kt + 1 == nk - 1) zero_tail((kt + 1) % NS);
     __syncthreads();  // ... everybody's has, and every wave has read tile kt out of its stage: that stage is free
     issue(kt + NS);
@@ -214,7 +246,7 @@ __global__ __launch_bounds__(256, 2) void hx_gemm16_tile128(const uint8_t* __res
     }
   };
   for (int t = 0; t < NS; ++t) issue(t);
-  __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 1) * 8));
+  __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm((NS - 1) * DPI));
   if (has_tail && nk == 1) zero_tail(0);
   __syncthreads();
 #pragma unroll

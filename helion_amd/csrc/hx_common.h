@@ -39,6 +39,10 @@ __device__ __forceinline__ void hx_g2l16(const void* gptr, void* lds_wave_base) 
 __device__ __forceinline__ void hx_g2l16_s(const void* sbase, uint32_t voff, uint32_t lds_wave_base) {
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_wave_base), "v"(voff), "s"(sbase) : "memory", "m0");
 }
+// The 4-byte form: the wave writes 256 contiguous bytes at lds_wave_base + lane*4 (for rows that are only 4-byte aligned).
+__device__ __forceinline__ void hx_g2l4_s(const void* sbase, uint32_t voff, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_wave_base), "v"(voff), "s"(sbase) : "memory", "m0");
+}
 // A wave-uniform pointer the compiler cannot prove uniform (the "s" constraint above needs SGPRs)
 __device__ __forceinline__ const uint8_t* hx_uniform_ptr(const uint8_t* p) {
   const uint64_t v = (uint64_t)p;

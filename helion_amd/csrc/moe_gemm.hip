@@ -239,11 +239,13 @@ extern "C" size_t hx_moe_workspace_bytes(int64_t T, int64_t E) {
 
 // Which kernel multiplies a grouped GEMM: 0 = hx_moe_general (fp32 FMAs; rows that are not 16-byte aligned, K % 8 != 0 or
 // N % 8 != 0), 1 = 32-row tiles, 2 = 128-row tiles, 3 = 256-row tiles, 4 = 128-row tiles with a partial last k-tile
-// (K % 64 != 0); 1-4 are MFMA kernels.
+// (K % 64 != 0), 5 = the same with A fetched in 4-byte pieces (K even but not a multiple of 8: 4-byte aligned rows, e.g.
+// the K = 500 of the reference's own check); 1-5 are MFMA kernels.
 static int moe_path(const void* A, const void* W, const void* C, int64_t T, int64_t K, int64_t N, int64_t E, int64_t a_div) {
-  const bool fast = (K % 8 == 0) && (N % 8 == 0) && K >= 8 && (((T + a_div - 1) / a_div) * K * 2 < (1LL << 32)) && (N * 4 < (1LL << 31)) &&
+  const bool fast = (K % 2 == 0) && (N % 8 == 0) && K >= 2 && (((T + a_div - 1) / a_div) * K * 2 < (1LL << 32)) && (N * 4 < (1LL << 31)) &&
                     (((uintptr_t)A | (uintptr_t)W | (uintptr_t)C) & 15) == 0;
   if (!fast) return 0;
+  if (K % 8 != 0) return 5;
   if (K % MOE_BK != 0) return 4;
   // 128-row tiles while the experts are small (less padding in each expert's last row tile) or the 256-row tiles would
   // not fill the chip; 256-row tiles otherwise (half the operand traffic per flop)
@@ -291,6 +293,11 @@ static int launch_moe(const void* A, const void* W, void* C, const int32_t* coun
       hx_launch((hx_gemm16_rows32<BF, 3>), dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W,
                          (void*)C, (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, max_tiles, tiles_n,
                          (int)a_div, d);
+    } else if (path == 5) {
+      const int tiles_n = (int)((N + G128_BN - 1) / G128_BN);
+      hx_launch((hx_gemm16_tile128<BF, 0, false, 2, true, true>), dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A,
+                (const uint8_t*)W, (void*)C, (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, max_tiles,
+                tiles_n, (int)a_div, d);
     } else if (path == 4) {
       const int tiles_n = (int)((N + G128_BN - 1) / G128_BN);
       hx_launch((hx_gemm16_tile128<BF, 0, false, 2, true>), dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A,

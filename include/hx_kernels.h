@@ -108,11 +108,12 @@ int hx_fp8_attention_path(int64_t BH, int64_t S, int64_t D, int64_t v_stride_d, 
  * max_T (the numel of the reference's dummy tensor) is accepted for signature parity and is only
  * validated (>= 0); the tile table is built on the device from counts/offsets.
  * workspace: hx_moe_workspace_bytes(T, E) bytes, 16-byte aligned.
- * MFMA kernels: K % 8 == 0 and N % 8 == 0 (16-byte rows), 16-byte aligned pointers, A below 4 GB; a K that is not a
- * multiple of 64 gets a zero-filled last k-tile.  Anything else, e.g. the K = 500 of the reference's own check
- * (examples/moe_matmul_ogs.py:186, 8-byte rows), runs an fp32-FMA kernel.  hx_moe_path (a_div = 1 for this entry point):
- * 0 = the FMA kernel, 1 / 2 / 3 = MFMA kernel with 32- / 128- / 256-row tiles, 4 = 128-row tiles with a partial last
- * k-tile. */
+ * MFMA kernels: K even and N % 8 == 0, 16-byte aligned pointers, A below 4 GB; a K that is not a multiple of 64 gets a
+ * zero-filled last k-tile, and a K that is not a multiple of 8 (rows of A only 4-byte aligned, e.g. the K = 500 of the
+ * reference's own check, examples/moe_matmul_ogs.py:186) has A fetched in 4-byte pieces.  Anything else (odd K,
+ * N % 8 != 0) runs an fp32-FMA kernel.  hx_moe_path (a_div = 1 for this entry point): 0 = the FMA kernel, 1 / 2 / 3 =
+ * MFMA kernel with 32- / 128- / 256-row tiles, 4 = 128-row tiles with a partial last k-tile, 5 = the same with A in
+ * 4-byte pieces. */
 int hx_moe_grouped_gemm(const void* A, const void* W, void* C, const int32_t* counts,
                         const int32_t* offsets, const int32_t* idx, int64_t T, int64_t K, int64_t N,
                         int64_t E, int64_t max_T, int dtype, void* workspace, size_t workspace_bytes,

@@ -22,16 +22,22 @@ def _run(A, W, ex):
 
 
 # path: what hx_moe_path reports - 0 the fp32-FMA kernel, 1 / 2 / 3 MFMA with 32- / 128- / 256-row tiles, 4 MFMA with
-# 128-row tiles and a zero-filled partial last k-tile
+# 128-row tiles and a zero-filled partial last k-tile, 5 the same with A fetched in 4-byte pieces (K even, K % 8 != 0)
 @pytest.mark.parametrize("T,K,N,E,topk,dtype,path", [
-    (1000, 500, 200, 30, 1, torch.float16, 0),    # examples/moe_matmul_ogs.py:186: 8-byte rows, no 16-byte DMA
+    (1000, 500, 200, 30, 1, torch.float16, 5),    # examples/moe_matmul_ogs.py:186: 8-byte rows, A by 4-byte DMA
     (1000, 504, 200, 30, 1, torch.float16, 4),    # ... the nearest shape with 16-byte rows: K = 7 k-tiles + 56
+    (1000, 500, 200, 30, 1, torch.bfloat16, 5),
+    (333, 2, 8, 3, 1, torch.bfloat16, 5),         # ... one pair of elements
+    (700, 70, 136, 6, 2, torch.float16, 5),       # ... 64 + 6, top-2
+    (40, 126, 64, 4, 1, torch.bfloat16, 5),       # ... 4-byte aligned rows only (K % 4 = 2), few rows
+    (2500, 1030, 256, 2, 1, torch.bfloat16, 5),   # ... 16 tiles + 6, large experts
+    (37, 101, 24, 3, 1, torch.bfloat16, 0),       # odd K: 2-byte aligned rows, the FMA kernel
     (512, 256, 512, 4, 1, torch.bfloat16, 2),
     (700, 128, 256, 5, 1, torch.float16, 2),
     (2048, 512, 768, 8, 2, torch.bfloat16, 2),    # top-2 expanded rows
     (8192, 192, 2048, 2, 1, torch.bfloat16, 3),   # 256-row tiles
     (300, 64, 256, 16, 1, torch.bfloat16, 2),     # most tiles nearly empty
-    (37, 100, 19, 3, 1, torch.bfloat16, 0),
+    (37, 100, 19, 3, 1, torch.bfloat16, 0),       # N % 8 != 0: the FMA kernel
     (512, 128, 384, 4, 1, torch.bfloat16, 2),     # ragged last column tile (N % 128 = 0, N % 256 = 128)
     (600, 64, 1408, 8, 2, torch.float16, 2),      # N = 5.5 tiles of 256
     (256, 64, 8, 2, 1, torch.bfloat16, 2),        # a single column tile with one valid 16-byte chunk
