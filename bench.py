@@ -22,9 +22,14 @@ Timing protocol, the same for every kernel timed here:
      Printed as "engine_clock_mhz" with the MFMA peak recomputed at that clock.  (amdsmi's clock readings are refreshed
      about once a second, too slow for a timed region of a few milliseconds; its socket power is printed as a hint.)
 
+The decode-shape GEMM (a 38 us kernel) is the one exception to 3: a pair of events around a single launch adds about
+2 us to it, so its figure is the average over the K launches issued back to back through the C ABI inside one event pair
+(median of five such regions); the per-launch pairs are printed beside it.
+
 The JSON line also carries the other three configurations (decode-shape GEMM, FP8 attention, MoE grouped GEMM) under
 "other_workloads" together with the kernels either side of them (casts, quantisation, routing), each with its own
-roofline object, and the ref-eager CPU path (ATen's CPU torch._scaled_mm on the 1024^3 configuration) under
+roofline object, the reference's own GPU baseline for the headline configuration (torch._scaled_mm, i.e. the vendor
+library, under the same protocol), and the ref-eager CPU path (ATen's CPU torch._scaled_mm on the 1024^3 configuration) under
 "cpu_baseline".
 """
 from __future__ import annotations
