@@ -76,8 +76,11 @@ def test_routing_properties_at_benchmark_size():
 @pytest.mark.parametrize("T_tok,K,N,E,topk,dtype", [
     (512, 256, 512, 4, 2, torch.bfloat16),     # tile256 kernel
     (300, 128, 256, 6, 4, torch.float16),
-    (1000, 500, 200, 30, 1, torch.float16),    # general kernel, the reference example's shape
+    (1000, 500, 200, 30, 1, torch.float16),    # the reference example's shape: A by 4-byte DMA
     (123, 96, 40, 5, 3, torch.bfloat16),
+    (250, 500, 136, 7, 2, torch.bfloat16),     # ... with the top-k gather (row r reads A_tok[r / 2])
+    (90, 120, 64, 6, 4, torch.float16),        # partial last k-tile with the top-k gather
+    (64, 101, 24, 3, 2, torch.bfloat16),       # odd K: the FMA kernel
 ])
 def test_topk_matmul_equals_replicated_form(T_tok, K, N, E, topk, dtype):
     A_rep, W, ex = inputs.moe_inputs(T_tok, K, N, E, topk, seed=T_tok + topk, dtype=dtype)

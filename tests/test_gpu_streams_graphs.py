@@ -24,7 +24,15 @@ def _cases():
     mb = torch.randn(264, device=DEV, generator=g).to(torch.float16)
     aq, ak, av = (torch.randn(2, 3, 200, 128, device=DEV, generator=g).to(torch.bfloat16) for _ in range(3))
     from helion_amd.matmul import bias_relu
+    da, db, _, _ = inputs.gemm_scaled(16, 16 * 256 * 12, 1024, seed=6)      # enough column groups for the ticket hand-out
+    da, db = da.to(DEV), db.to(DEV)
+    A4, W4, ex4 = (t.to(DEV) for t in inputs.moe_inputs(200, 500, 72, 5, 1, seed=7, dtype=torch.float16))   # A by 4-byte DMA
+    args4 = hx.moe_matmul_ogs_helion_kernel_args_gen(A4, W4, ex4)   # (has the reference's host sync: outside the capture)
     return {
+        "fp8_gemm_decode_tickets": lambda: hx.fp8_gemm(da, db, out_dtype=torch.float32),
+        "fp8_attention_ragged": lambda: hx.fp8_attention_kernel(q[:, :200].contiguous(), k[:, :200].contiguous(),
+                                                                v[:, :, :200].contiguous(), 1, 4, out_dtype=torch.float32),
+        "moe_partial_k_tile": lambda: hx.moe_matmul_ogs(*args4),
         "matmul_bias_relu": lambda: hx.matmul(mx, my, bias_relu(mb)),
         "matmul_split_k": lambda: hx.matmul_split_k(mx, my, split_k=4),
         "attention16": lambda: hx.attention(aq, ak, av),
