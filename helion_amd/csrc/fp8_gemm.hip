@@ -340,7 +340,8 @@ __global__ __launch_bounds__(256) void hx_transpose_u8(const uint8_t* __restrict
 // the column tiles come to about one per CU (N = 28672: 112 columns, 256 tiles); the columns of a tile past bn
 // re-read its last column (an L2 hit, no HBM traffic) and are not stored.
 // ------------------------------------------------------------------------------------------
-template <int OUT, int BM, bool PAIR = false>
+// BNT: B is streamed past a single row tile (every byte of it read once by the launch): its DMA carries the non-temporal hint.
+template <int OUT, int BM, bool PAIR = false, bool BNT = false>
 __global__ __launch_bounds__(256) void hx_fp8_gemm_tileN128(const uint8_t* __restrict__ A_, const uint8_t* __restrict__ Bt_,
                                                            typename OutT<OUT>::T* __restrict__ C_, int M, int N, int K, long lda,
                                                            long ldb, long ldc, const float* __restrict__ scale_a,
@@ -397,6 +398,7 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tileN128(const uint8_t* __res
     const int t = min(kt, nk - 1);
     const uint32_t base = lds0 + (uint32_t)(kt % NS) * STAGE;
     if (i < AJ) hx_g2l16_s(hx_uniform_ptr(A + (long)t * T256_BK), a_vo[i], base + (w + 4 * i) * 1024);
+    else if (BNT) hx_g2l16_s_nt(hx_uniform_ptr(Bt + (long)t * T256_BK), b_vo[i - AJ], base + BM * 128 + (w + 4 * (i - AJ)) * 1024);
     else hx_g2l16_s(hx_uniform_ptr(Bt + (long)t * T256_BK), b_vo[i - AJ], base + BM * 128 + (w + 4 * (i - AJ)) * 1024);
   };
   auto issue = [&](int kt) {
@@ -972,6 +974,17 @@ extern "C" int hx_fp8_gemm_path(int64_t M, int64_t N, int64_t K, int64_t lda, in
   return 0;
 }
 
+// B is read exactly once by a launch with a single row tile (always the case for the 64-row tile): non-temporal DMA then
+template <int OUT, int BM, bool PAIR, typename... Args>
+static void launch_tileN128(bool b_read_once, dim3 grid, hipStream_t stream, Args... args) {
+  if constexpr (BM == 64) {
+    hx_launch((hx_fp8_gemm_tileN128<OUT, BM, PAIR, true>), grid, dim3(256), 0, stream, args...);
+  } else {
+    if (b_read_once) hx_launch((hx_fp8_gemm_tileN128<OUT, BM, PAIR, true>), grid, dim3(256), 0, stream, args...);
+    else hx_launch((hx_fp8_gemm_tileN128<OUT, BM, PAIR, false>), grid, dim3(256), 0, stream, args...);
+  }
+}
+
 static std::atomic<unsigned long long> g_skd_launches{0};
 
 template <int OUT, int MB, typename... Args>
@@ -1015,25 +1028,25 @@ static void launch_kmajor(int path, const void* a, const void* bt, void* c, int6
     if (split) {
       float* part = (float*)ws;
       if (bm == 64)
-        hx_launch((hx_fp8_gemm_tileN128<HX_F32, 64, true>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
+        launch_tileN128<HX_F32, 64, true>(tiles_m == 1, grid, stream, (const uint8_t*)a, (const uint8_t*)bt,
                            part, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)N, nullptr, nullptr, tiles_m, bn, ktps);
       else if (bm == 256)
-        hx_launch((hx_fp8_gemm_tileN128<HX_F32, 256>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt, part,
+        launch_tileN128<HX_F32, 256, false>(tiles_m == 1, grid, stream, (const uint8_t*)a, (const uint8_t*)bt, part,
                            (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)N, nullptr, nullptr, tiles_m, bn, ktps);
       else
-        hx_launch((hx_fp8_gemm_tileN128<HX_F32, 128>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt, part,
+        launch_tileN128<HX_F32, 128, false>(tiles_m == 1, grid, stream, (const uint8_t*)a, (const uint8_t*)bt, part,
                            (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)N, nullptr, nullptr, tiles_m, bn, ktps);
       const long quads = (long)M * ((N + 3) / 4);
       hx_launch((hx_fp8_gemm_split_reduce<OUT>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream,
                          (const float*)part, (out_t*)c, (int)M, (int)N, (long)ldc, splits, sa, sb);
     } else if (bm == 64) {
-      hx_launch((hx_fp8_gemm_tileN128<OUT, 64, true>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
+      launch_tileN128<OUT, 64, true>(tiles_m == 1, grid, stream, (const uint8_t*)a, (const uint8_t*)bt,
                          (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m, bn, 0);
     } else if (bm == 256) {
-      hx_launch((hx_fp8_gemm_tileN128<OUT, 256>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
+      launch_tileN128<OUT, 256, false>(tiles_m == 1, grid, stream, (const uint8_t*)a, (const uint8_t*)bt,
                          (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m, bn, 0);
     } else {
-      hx_launch((hx_fp8_gemm_tileN128<OUT, 128>), grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
+      launch_tileN128<OUT, 128, false>(tiles_m == 1, grid, stream, (const uint8_t*)a, (const uint8_t*)bt,
                          (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m, bn, 0);
     }
   } else if (path == 1 || path == 3) {

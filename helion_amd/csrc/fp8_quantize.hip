@@ -69,7 +69,9 @@ __global__ __launch_bounds__(QZ_THREADS) void hx_cast_e4m3_kernel(QzJobs jobs, c
   for (long long v = (long long)blockIdx.x * QZ_THREADS + threadIdx.x; v < nvec; v += stride) {
     float f[QZ_EPT];
     qz_load16(src + v * QZ_EPT, f);
-    ((v4i*)dst)[v] = qz_pack16(f, mul);
+    // non-temporal store: the codes are written once and not read here (the three C4-sized casts -3 %); the loads stay
+    // plain, so the second read of a quantisation still finds what the amax pass left in the caches
+    __builtin_nontemporal_store(qz_pack16(f, mul), (v4i*)dst + v);
   }
   // ragged tail (fewer than 16 elements) by the first threads of block 0
   if (blockIdx.x == 0) {

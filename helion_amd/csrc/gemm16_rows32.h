@@ -60,7 +60,7 @@ __global__ __launch_bounds__(256, NS <= 3 ? 2 : 1) void hx_gemm16_rows32(const u
     const uint32_t lw = lds0 + (uint32_t)stage * R32_STAGE_BYTES + R32_A_BYTES + (uint32_t)w * 16 * 256;
     hx_g2l16_s(A + (long)kt * 128, a_vo, la);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) hx_g2l16_s(We + ((long)kt * MOE_BK + 4 * j) * d.ldb * 2, w_vo, lw + j * 1024);
+    for (int j = 0; j < 4; ++j) hx_g2l16_s_nt(We + ((long)kt * MOE_BK + 4 * j) * d.ldb * 2, w_vo, lw + j * 1024);  // W: read once
   };
 
   // ---- operand addressing (see the 128-row kernel): A fragment of k-step ks at a_base + (ax ^ (ks * 32)); the two

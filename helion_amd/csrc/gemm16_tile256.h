@@ -343,7 +343,9 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256(const uint8_t* __restri
       const int row = p * 4 + rb_row;
       const int r = srow[bb * 32 + row];
       const v4i v = *(const v4i*)(sb + row * RSTR + rb_ch * 16);
-      if (r >= 0 && ncol8 < N) *(v4i*)(C + (long)r * d.ldc + ncol8) = v;
+      // (non-temporal: the output is written once and not read here, and lines of it lingering in the L2s displace operand
+      // panels: dense 8192^3 -4 %, grouped +-0)
+      if (r >= 0 && ncol8 < N) __builtin_nontemporal_store(v, (v4i*)(C + (long)r * d.ldc + ncol8));
     }
   };
   // The LDS executes one wave's operations in order, so a block may be refilled as soon as the reads that drain it
