@@ -974,15 +974,11 @@ extern "C" int hx_fp8_gemm_path(int64_t M, int64_t N, int64_t K, int64_t lda, in
   return 0;
 }
 
-// B is read exactly once by a launch with a single row tile (always the case for the 64-row tile): non-temporal DMA then
+// b_read_once: non-temporal DMA for B
 template <int OUT, int BM, bool PAIR, typename... Args>
 static void launch_tileN128(bool b_read_once, dim3 grid, hipStream_t stream, Args... args) {
-  if constexpr (BM == 64) {
-    hx_launch((hx_fp8_gemm_tileN128<OUT, BM, PAIR, true>), grid, dim3(256), 0, stream, args...);
-  } else {
-    if (b_read_once) hx_launch((hx_fp8_gemm_tileN128<OUT, BM, PAIR, true>), grid, dim3(256), 0, stream, args...);
-    else hx_launch((hx_fp8_gemm_tileN128<OUT, BM, PAIR, false>), grid, dim3(256), 0, stream, args...);
-  }
+  if (b_read_once) hx_launch((hx_fp8_gemm_tileN128<OUT, BM, PAIR, true>), grid, dim3(256), 0, stream, args...);
+  else hx_launch((hx_fp8_gemm_tileN128<OUT, BM, PAIR, false>), grid, dim3(256), 0, stream, args...);
 }
 
 static std::atomic<unsigned long long> g_skd_launches{0};
@@ -1024,29 +1020,31 @@ static void launch_kmajor(int path, const void* a, const void* bt, void* c, int6
     const bool split = splits > 1 && ws && aligned(ws, 16) && ws_bytes >= (size_t)splits * M * N * 4;
     if (!split) ktps = 0;
     const dim3 grid((unsigned)(tiles_m * tiles_n), split ? splits : 1);
+    // B read exactly once by the launch, and too large to stay in the 256 MB memory-side cache between calls
+    const bool b_once = tiles_m == 1 && N * K >= (192LL << 20);
     // split-K launches write unscaled fp32 slabs into the workspace; hx_fp8_gemm_split_reduce sums, scales and casts them
     if (split) {
       float* part = (float*)ws;
       if (bm == 64)
-        launch_tileN128<HX_F32, 64, true>(tiles_m == 1, grid, stream, (const uint8_t*)a, (const uint8_t*)bt,
+        launch_tileN128<HX_F32, 64, true>(b_once, grid, stream, (const uint8_t*)a, (const uint8_t*)bt,
                            part, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)N, nullptr, nullptr, tiles_m, bn, ktps);
       else if (bm == 256)
-        launch_tileN128<HX_F32, 256, false>(tiles_m == 1, grid, stream, (const uint8_t*)a, (const uint8_t*)bt, part,
+        launch_tileN128<HX_F32, 256, false>(b_once, grid, stream, (const uint8_t*)a, (const uint8_t*)bt, part,
                            (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)N, nullptr, nullptr, tiles_m, bn, ktps);
       else
-        launch_tileN128<HX_F32, 128, false>(tiles_m == 1, grid, stream, (const uint8_t*)a, (const uint8_t*)bt, part,
+        launch_tileN128<HX_F32, 128, false>(b_once, grid, stream, (const uint8_t*)a, (const uint8_t*)bt, part,
                            (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)N, nullptr, nullptr, tiles_m, bn, ktps);
       const long quads = (long)M * ((N + 3) / 4);
       hx_launch((hx_fp8_gemm_split_reduce<OUT>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream,
                          (const float*)part, (out_t*)c, (int)M, (int)N, (long)ldc, splits, sa, sb);
     } else if (bm == 64) {
-      launch_tileN128<OUT, 64, true>(tiles_m == 1, grid, stream, (const uint8_t*)a, (const uint8_t*)bt,
+      launch_tileN128<OUT, 64, true>(b_once, grid, stream, (const uint8_t*)a, (const uint8_t*)bt,
                          (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m, bn, 0);
     } else if (bm == 256) {
-      launch_tileN128<OUT, 256, false>(tiles_m == 1, grid, stream, (const uint8_t*)a, (const uint8_t*)bt,
+      launch_tileN128<OUT, 256, false>(b_once, grid, stream, (const uint8_t*)a, (const uint8_t*)bt,
                          (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m, bn, 0);
     } else {
-      launch_tileN128<OUT, 128, false>(tiles_m == 1, grid, stream, (const uint8_t*)a, (const uint8_t*)bt,
+      launch_tileN128<OUT, 128, false>(b_once, grid, stream, (const uint8_t*)a, (const uint8_t*)bt,
                          (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m, bn, 0);
     }
   } else if (path == 1 || path == 3) {

@@ -147,11 +147,14 @@ __global__ __launch_bounds__(256, 2) void hx_gemm16_tile128(const uint8_t* __res
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       if (BCOL) {
-        hx_g2l16_s(W + ((long)kt0 + kt) * 128, KTAIL && tail ? wc_vo_t[BCOL && KTAIL ? j : 0] : wc_vo[BCOL ? j : 0],
-                   lw + (uint32_t)w * 32 * 128 + j * 1024);
+        const uint32_t vo = KTAIL && tail ? wc_vo_t[BCOL && KTAIL ? j : 0] : wc_vo[BCOL ? j : 0];
+        if (MODE != 0 && d.w_once) hx_g2l16_s_nt(W + ((long)kt0 + kt) * 128, vo, lw + (uint32_t)w * 32 * 128 + j * 1024);
+        else hx_g2l16_s(W + ((long)kt0 + kt) * 128, vo, lw + (uint32_t)w * 32 * 128 + j * 1024);
       } else if (KTAIL && tail) {  // k rows past K re-read row K-1 (offsets from the tile's first k row)
         const int kr = min(w * 16 + 4 * j + wk_l, ktail - 1);
         hx_g2l16_s(We + ((long)kt * MOE_BK - w * 16) * d.ldb * 2, (uint32_t)(kr * d.ldb * 2) + w_ch, lw + (uint32_t)w * 16 * 256 + j * 1024);
+      } else if (MODE != 0 && d.w_once) {
+        hx_g2l16_s_nt(We + ((long)kt * MOE_BK + 4 * j) * d.ldb * 2, w_vo, lw + (uint32_t)w * 16 * 256 + j * 1024);
       } else {
         hx_g2l16_s(We + ((long)kt * MOE_BK + 4 * j) * d.ldb * 2, w_vo, lw + (uint32_t)w * 16 * 256 + j * 1024);
       }

@@ -47,6 +47,8 @@ struct G16Dense {
   int bias_f32;         // bias is fp32 rather than the operand type
   int relu;
   int kt_per_split;     // MODE 2: k-tiles per blockIdx.y
+  int w_once;           // dense modes, 128-tile kernel: the launch has one row tile, so every byte of W is read once
+                        // (its DMA then carries the non-temporal hint)
 };
 
 template <bool BF, int MODE, bool BCOL = false>

@@ -171,6 +171,8 @@ static void mm_launch_fast(const void* a, const void* b, void* c, int64_t M, int
   const int tiles_m = (int)((M + tile - 1) / tile), tiles_n = (int)((N + tile - 1) / tile);
   G16Dense d = {};
   d.lda = lda; d.ldb = ldb_k; d.bias = bias; d.bias_f32 = bias_f32; d.relu = relu;
+  // one row tile and a weight matrix too large to stay in the 256 MB memory-side cache between calls: stream it
+  d.w_once = tiles_m == 1 && K * N * 2 >= (192LL << 20);
   const bool partial = splits > 1 || (out_dtype == HX_F32 && (bias || relu));
   if (!partial && out_dtype != HX_F32) {
     d.ldc = ldc;
