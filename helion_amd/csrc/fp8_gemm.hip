@@ -661,8 +661,13 @@ __device__ __forceinline__ unsigned long long skd_draw_issue(unsigned long long*
 }
 __device__ __forceinline__ int skd_draw_result(unsigned long long* word, unsigned long long old, unsigned long long tag, int nwork,
                                                int total) {
-  while ((old >> 24) != tag) {
-    while ((__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 24) != tag) __builtin_amdgcn_s_sleep(32);
+  // (the wait is bounded all the same: if two launches are given the same word at the same time - a misuse - a tag may
+  // never come back, and a workgroup that gives up and stops costs that misuse wrong results, not a hung GPU)
+  for (int spins = 0; (old >> 24) != tag; ) {
+    while ((__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 24) != tag) {
+      if (++spins > (1 << 18)) return -1;
+      __builtin_amdgcn_s_sleep(32);
+    }
     old = skd_draw_issue(word);
   }
   const unsigned cnt = (unsigned)(old & 0xFFFFFF);

@@ -4,6 +4,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include "../../include/hx_kernels.h"
 
 static thread_local char g_err[512] = "";
@@ -20,13 +22,13 @@ extern "C" int hx_version(void) { return 1; }
 
 // Compute units of the current device.  The attribute query costs microseconds, so each device is asked once.
 int hx_cu_count() {
-  static int cached[64];  // 0 = not asked yet (racing first calls write the same value)
+  static std::atomic<int> cached[64];  // 0 = not asked yet (racing first calls store the same value)
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cached[dev] == 0) {
-    int cus = 0;
+  int cus = cached[dev].load(std::memory_order_relaxed);
+  if (cus == 0) {
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
-    cached[dev] = cus;
+    cached[dev].store(cus, std::memory_order_relaxed);
   }
-  return cached[dev];
+  return cus;
 }

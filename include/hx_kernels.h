@@ -54,7 +54,8 @@ const char* hx_last_error(void);
  * of 128 — K % 16 == 0 suffices, the last k-tile is zero-padded in LDS; it reads a column-major B directly and a
  * row-major B through transposing LDS loads), the skinny (M<=16, or M<=32 with K<=8192) wave-split-K kernel
  * and a bounds-checked general kernel from the shape, strides and alignment.
- * workspace: optional device scratch of hx_fp8_gemm_workspace_bytes(...) bytes, 16-byte aligned. */
+ * workspace: optional device scratch of hx_fp8_gemm_workspace_bytes(...) bytes, 16-byte aligned, any content; it
+ *    belongs to the call until its kernels have finished (two launches in flight at once need two workspaces). */
 int hx_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int64_t lda,
                 int64_t ldb_k, int64_t ldb_n, int64_t ldc, const float* scale_a, const float* scale_b,
                 int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
@@ -62,7 +63,9 @@ int hx_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int64_t N, int
  * or N / the row stride not a multiple of 16): N*K bytes for a one-off transpose into the K-contiguous layout,
  * without which such a B runs on the slow general kernel.  Column-major B: splits*M*N*4 bytes when the 128-column
  * tile kernel would cut K into `splits` pieces (its tiles occupy less than half of the CUs and K is at least 16
- * k-tiles long; at most 32 MB), without which it runs unsplit.  0 otherwise. */
+ * k-tiles long; at most 32 MB), without which it runs unsplit; 16 bytes for a decode call (M <= 16, K <= 8192) with at
+ * least 12 column groups of 16 per CU: the word through which the last groups are handed out to whichever workgroup is
+ * free (needs no initialisation, is left zero), without which every workgroup takes a fixed share.  0 otherwise. */
 size_t hx_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t ldb_k, int64_t ldb_n);
 
 /* Which kernel hx_fp8_gemm would launch for these arguments: 0 general (or, given a workspace, transpose + fast
