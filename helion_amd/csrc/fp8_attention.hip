@@ -130,7 +130,7 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_pipe(const uint8_t* _
   const uint8_t* Vh = Vt + (long)bh * D * S;
 
   v8i qf[KSTEPS];
-  {
+  if (MODE == 0) {  // (MODE 1: pass 1 holds the Q fragments of the wave pair; this wave's are among them)
     const int qrow = min(q0 + q31, S - 1);
 #pragma unroll
     for (int t = 0; t < KSTEPS; ++t) {
@@ -302,12 +302,16 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_pipe(const uint8_t* _
     // soon as its two MFMAs are out: by then that tile has landed for every wave (the round's barrier waits for the
     // tiles of two rounds), and the refill has the rest of the round and the barrier to arrive.
     v8i kf[NF];
-    auto round = [&](v16f(&cur)[2][2], v16f(&next)[2][2], int t, int tc) {
+    // FULL: a round of the steady state - its tile, the tile two ahead and a finished previous tile all exist - so the
+    // body has no branch besides the one on pair_active.  (With the guards evaluated at run time a round was two dozen
+    // scalar branches, and the pass spent more time fetching instructions than multiplying.)
+    auto round = [&](auto full_c, v16f(&cur)[2][2], v16f(&next)[2][2], int t, int tc) __attribute__((always_inline)) {
+      constexpr bool FULL = decltype(full_c)::value;
       if (!pair_active) return;
       // (a partial last tile needs no masking here: its rows past S are re-reads of key S-1, whose score is a
       // valid one, so they cannot change the maximum)
-      if (t < ntiles) {
-        const bool more = t + 2 < ntiles;
+      if (FULL || t < ntiles) {
+        const bool more = FULL || t + 2 < ntiles;
         const uint8_t* sk2 = sm + kslot(more ? t + 2 : t);  // (no next tile: re-read this one, the values are not used)
 #pragma unroll
         for (int n = 0; n < NF; ++n) {
@@ -315,7 +319,7 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_pipe(const uint8_t* _
           next[0][kb] = hx_mfma_32x32x64_e4m3(kf[n], qp[0][ks], ks ? next[0][kb] : zero16);
           next[1][kb] = hx_mfma_32x32x64_e4m3(kf[n], qp[1][ks], ks ? next[1][kb] : zero16);
           kf[n] = load_kfrag(sk2, n);
-          if (tc >= 0) reduce_part(cur, n);
+          if (FULL || tc >= 0) reduce_part(cur, n);
           __builtin_amdgcn_sched_barrier(0);
         }
       } else if (tc >= 0) {
@@ -333,26 +337,48 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_pipe(const uint8_t* _
       for (int n = 0; n < NF; ++n) kf[n] = load_kfrag(sm + kslot(min(par, last)), n);
     }
     const int nrounds = (ntiles + 1) / 2;  // round r: tiles 2r and 2r+1
-    auto do_round = [&](v16f(&cur)[2][2], v16f(&next)[2][2], int r) {
+    // FULL rounds: 1 <= r, tiles 2r+6 and 2r+7 exist and are whole tiles (plain DMA form), so every guard is known
+    auto do_round = [&](auto full_c, v16f(&cur)[2][2], v16f(&next)[2][2], int r) __attribute__((always_inline)) {
+      constexpr bool FULL = decltype(full_c)::value;
       const int jj = 2 * r;
       // tiles jj .. jj+3 must have landed (this round's and the next round's, whose fragments this round
       // prefetches); tiles jj+4, jj+5 may still be in flight
-      if (jj + 5 <= last) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(2 * KPW));
+      if (FULL || jj + 5 <= last) __builtin_amdgcn_s_waitcnt(hx_vmcnt_imm(2 * KPW));
       else HX_WAIT_VM0();
       __syncthreads();  // ... for every wave; and every wave is done with tiles jj-2 and jj-1: their slots are free
-      if (jj + 6 < ntiles) issue_k(jj + 6, kslot(jj + 6));
-      if (jj + 7 < ntiles) issue_k(jj + 7, kslot(jj + 7));
-      // The last round multiplies out of registers (what its refills read is not used), and every wave has finished
-      // its real fragment reads before this round's barrier: the whole ring is free, and pass 2's first tiles go out
-      // now instead of after the pass.
-      if (r == nrounds - 1) issue_pass2_prologue();
+      if (FULL) {
+#pragma unroll
+        for (int i = 0; i < KPW; ++i) issue_k_one(jj + 6, kslot(jj + 6), i, std::false_type{});
+#pragma unroll
+        for (int i = 0; i < KPW; ++i) issue_k_one(jj + 7, kslot(jj + 7), i, std::false_type{});
+      } else {
+        if (jj + 6 < ntiles) issue_k(jj + 6, kslot(jj + 6));
+        if (jj + 7 < ntiles) issue_k(jj + 7, kslot(jj + 7));
+        // The last round multiplies out of registers (what its refills read is not used), and every wave has finished
+        // its real fragment reads before this round's barrier: the whole ring is free, and pass 2's first tiles go out
+        // now instead of after the pass.
+        if (r == nrounds - 1) issue_pass2_prologue();
+      }
       const int t = jj + par;
-      round(cur, next, t, tc);
-      tc = t < ntiles ? t : -1;
+      round(full_c, cur, next, t, tc);
+      tc = (FULL || t < ntiles) ? t : -1;
     };
-    for (int r = 0; r < nrounds; r += 2) {
-      do_round(ca, cb, r);
-      if (r + 1 < nrounds) do_round(cb, ca, r + 1);
+    // Even rounds read ca and write cb, odd rounds the other way round, so rounds come in pairs; three loops one after
+    // the other, each with its two rounds written out (a run-time choice between the guarded and the branch-free pair
+    // inside one loop makes the compiler shuffle the 128 accumulator registers where the two paths meet, through scratch).
+    const int r_full = last >= 8 ? (last - 8) / 2 : -1;  // the last round whose tiles 2r+6, 2r+7 lie before the last tile
+    int r = 0;
+    for (; r < 2 && r < nrounds; r += 2) {  // the first pair: no finished tile yet
+      do_round(std::false_type{}, ca, cb, r);
+      if (r + 1 < nrounds) do_round(std::false_type{}, cb, ca, r + 1);
+    }
+    for (; r + 1 <= r_full; r += 2) {
+      do_round(std::true_type{}, ca, cb, r);
+      do_round(std::true_type{}, cb, ca, r + 1);
+    }
+    for (; r < nrounds; r += 2) {
+      do_round(std::false_type{}, ca, cb, r);
+      if (r + 1 < nrounds) do_round(std::false_type{}, cb, ca, r + 1);
     }
     if (pair_active && tc >= 0) {  // the last tile's scores: round r wrote cb when r is even, ca when it is odd
       if ((nrounds - 1) & 1) {
@@ -369,6 +395,11 @@ __global__ __launch_bounds__(256, 2) void hx_fp8_attention_pipe(const uint8_t* _
     __syncthreads();
     const float smax = fmaxf(m_own, xch[(w ^ 1) * 32 + q31]);
     neg_m = -(smax * c);  // max(s*c) == max(s)*c for c > 0 (rounding is monotone)
+    // this wave's own 32 queries are block `par` of the pair's 64
+#pragma unroll
+    for (int t = 0; t < KSTEPS; ++t)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) qf[t][e] = par ? qp[1][t][e] : qp[0][t][e];
   }
 
   // ================= pass 2 (MODE 0: the only pass)
