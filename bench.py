@@ -19,7 +19,10 @@ Timing protocol, the same for every kernel timed here:
      back to back with the timed ones, while a one-wave probe kernel (hx_clock_probe) runs three times on a second
      stream: it reads the shader-clock counter against the constant 100 MHz counter over 50 us, which gives the
      engine clock the chip sustains under this kernel's load (it is power-limited well below its 2.4 GHz maximum).
-     Printed as "engine_clock_mhz" with the MFMA peak recomputed at that clock.  (amdsmi's clock readings are refreshed
+     Printed as "engine_clock_mhz" with the MFMA peak recomputed at that clock.  The probe needs a free wave slot: next
+     to a kernel whose waves fill the register file (the 256x256 tile GEMMs, fp8 and 16-bit) it only runs while a launch
+     drains and reads a chip that has just gone idle, so for those rows the printed clock is an upper bound (counters read
+     inside an instrumented build of the grouped GEMM showed 1.87 GHz where this probe printed 2.34).  (amdsmi's clock readings are refreshed
      about once a second, too slow for a timed region of a few milliseconds; its socket power is printed as a hint.)
 
 The decode-shape GEMM (a 38 us kernel) is the one exception to 3: a pair of events around a single launch adds about
