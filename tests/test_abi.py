@@ -136,3 +136,33 @@ def test_sibling_argument_errors_are_reported_without_a_launch():
     assert lib.hx_attention_path(2, 100, 70, 128, 1, A, A, A, A) == 1
     assert lib.hx_attention_path(2, 100, 70, 96, 1, A, A, A, A) == 0
     assert lib.hx_attention_path(2, 100, 70, 128, 2, A, A, A, A) == 0
+
+
+def test_moe_path_selection():
+    """Host logic only: which grouped-GEMM kernel a shape gets (the query never dereferences its pointers)."""
+    lib = _lib.load()
+    A = 1 << 20
+    assert lib.hx_moe_path(32768, 4096, 14336, 8, 1, A, A, A) == 3     # C5: 256-row tiles
+    assert lib.hx_moe_path(4000, 4096, 1024, 8, 1, A, A, A) == 2       # < 512 rows per expert: 128-row tiles
+    assert lib.hx_moe_path(2000, 4096, 14336, 64, 1, A, A, A) == 2
+    assert lib.hx_moe_path(16, 4096, 14336, 8, 1, A, A, A) == 1        # a decode step: 32 rows in all
+    assert lib.hx_moe_path(1000, 504, 200, 30, 1, A, A, A) == 4        # K % 64 != 0, K % 8 == 0: zero-filled last k-tile
+    assert lib.hx_moe_path(1000, 500, 200, 30, 1, A, A, A) == 5        # the reference's own check shape (examples/moe_matmul_ogs.py:186): K even
+    assert lib.hx_moe_path(1000, 501, 200, 30, 1, A, A, A) == 0        # odd K: rows of A not even 4-byte aligned
+    assert lib.hx_moe_path(1000, 512, 204, 30, 1, A, A, A) == 0        # N % 8 != 0
+    assert lib.hx_moe_path(1000, 512, 200, 30, 1, A + 2, A, A) == 0    # misaligned A
+    assert lib.hx_moe_path(100, 64, 64, 4, 2, A, A, A) in (1, 2)       # top-k through a_div: still an MFMA kernel
+
+
+def test_fp8_attention_path_selection():
+    lib = _lib.load()
+    A = 1 << 20
+    assert lib.hx_fp8_attention_path(128, 4096, 128, 4096, 1, A, A, A, A) == 1   # C4, v as [D][S]
+    assert lib.hx_fp8_attention_path(128, 4096, 128, 1, 128, A, A, A, A) == 1    # v as the reference's preprocessing leaves it
+    assert lib.hx_fp8_attention_path(2, 208, 128, 208, 1, A, A, A, A) == 1       # partial last key tile
+    assert lib.hx_fp8_attention_path(2, 200, 128, 1, 128, A, A, A, A) == 1
+    assert lib.hx_fp8_attention_path(2, 200, 128, 200, 1, A, A, A, A) == 0       # [D][S] rows come in 16-byte pieces: S % 16
+    assert lib.hx_fp8_attention_path(2, 128, 64, 128, 1, A, A, A, A) == 1
+    assert lib.hx_fp8_attention_path(2, 128, 96, 128, 1, A, A, A, A) == 0        # (the Python op zero-pads such heads to 128)
+    assert lib.hx_fp8_attention_path(2, 128, 256, 128, 1, A, A, A, A) == 0
+    assert lib.hx_fp8_attention_path(2, 128, 128, 128, 1, A + 8, A, A, A) == 0   # misaligned q
