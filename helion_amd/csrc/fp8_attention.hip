@@ -745,7 +745,7 @@ extern "C" int hx_fp8_attention(const void* q, const void* k, const void* v, voi
   const bool fast = att_fast_path(q, k, v, out, S, D, v_stride_d, v_stride_s, &vsd);
   if (!fast) {  // any other shape, alignment or V striding within a head (heads are D*S elements apart)
     if (D > 256 || D < 1 || BH >= 65536) {
-      hx_set_error("hx_fp8_attention: unsupported shape S=%lld D=%lld BH=%lld (MFMA kernel: D in {64,128}, S %% 64 == 0; plain kernel: D <= 256, BH < 65536)",
+      hx_set_error("hx_fp8_attention: unsupported shape S=%lld D=%lld BH=%lld (MFMA kernel: D in {64,128}, 16-byte aligned pointers, v as [D][S] with S %% 16 == 0 or as [S][D]; plain kernel: D <= 256, BH < 65536)",
                    (long long)S, (long long)D, (long long)BH);
       return HX_ERR_UNSUPPORTED;
     }
