@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only c2,lib,c3,c4,c5,next,sib] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only c2,lib,c3,c4,c5,next,sib[,lib16]] [--no-cpu-baseline]
 
 A "step" is one launch of the FP8 GEMM at the headline configuration (M=N=K=8192, e4m3 operands, B column-major,
 per-tensor fp32 scales, bf16 output) with inputs resident in HBM.
@@ -273,6 +273,51 @@ def bench_c2_library_baseline(steps, warmup):
     roof = _mfma_roofline(2.0 * 8192**3, t, PEAK_FP8_TFLOPS, FP8_FLOP_PER_CU_CLK, "hipBLASLt fp8 GEMM behind torch._scaled_mm")
     return {"workload": "torch._scaled_mm (hipBLASLt) on the C2 operands: reference_fp8_gemm_pytorch, examples/fp8_gemm.py:61-78",
             "ms_per_launch": t["median_ms"], "value": roof["achieved"], "unit": "TFLOP/s", "roofline": roof}
+
+
+def bench_16bit_library_baselines(steps, warmup):
+    """Opt-in (`--only ...,lib16`; not part of the default run): the vendor library (hipBLASLt / rocBLAS behind torch.matmul)
+    on the two 16-bit GEMM workloads, under the same protocol, for comparison only.  Dense: the 8192^3 bf16 product with a
+    row-major and with a column-major second operand.  Grouped: the body of moe_matmul_ogs_reference
+    (examples/moe_matmul_ogs.py:125-148) with its gather and scatter taken out - one torch.matmul per expert on rows already
+    sorted by expert, written into consecutive output rows - which is the least the library can do for the C5 operands."""
+    import torch
+    from helion_amd import inputs
+
+    out = {}
+    try:
+        x = torch.randn(8192, 8192, device="cuda", dtype=torch.bfloat16)
+        w = torch.randn(8192, 8192, device="cuda", dtype=torch.bfloat16)
+        for name, y in (("row_major_b", w), ("column_major_b", w.t().contiguous().t())):
+            t = _time_launches(lambda: torch.matmul(x, y), steps, warmup)
+            roof = _mfma_roofline(2.0 * 8192**3, t, PEAK_BF16_TFLOPS, BF16_FLOP_PER_CU_CLK, "vendor bf16 GEMM behind torch.matmul")
+            out["dense_8192_bf16_torch_matmul_" + name] = {"ms_per_launch": t["median_ms"], "value": roof["achieved"], "unit": "TFLOP/s",
+                                                            "roofline": roof}
+        del x, w
+        torch.cuda.empty_cache()
+        A, W, ex = inputs.moe_c5("cuda")
+        order = torch.argsort(ex, stable=True)
+        counts = torch.bincount(ex, minlength=W.shape[0]).tolist()
+        a_sorted = A[order].contiguous()
+        c_sorted = torch.empty(A.shape[0], W.shape[2], device="cuda", dtype=torch.bfloat16)
+        segs, s0 = [], 0
+        for c in counts:
+            segs.append((s0, c))
+            s0 += c
+
+        def per_expert():
+            for e, (s, c) in enumerate(segs):
+                if c:
+                    torch.matmul(a_sorted[s:s + c], W[e], out=c_sorted[s:s + c])
+
+        t = _time_launches(per_expert, steps, warmup)
+        roof = _mfma_roofline(2.0 * 32768 * 4096 * 14336, t, PEAK_BF16_TFLOPS, BF16_FLOP_PER_CU_CLK,
+                              "vendor bf16 GEMM behind torch.matmul, one call per expert")
+        out["c5_torch_matmul_per_expert_presorted"] = {"ms_per_launch": t["median_ms"], "value": roof["achieved"], "unit": "TFLOP/s",
+                                                       "rows_per_expert": counts, "roofline": roof}
+    except Exception as e:  # comparison rows must never take the benchmark down
+        out["error"] = f"{type(e).__name__}: {e}"[:300]
+    return out
 
 
 def bench_c3(steps, warmup):
@@ -643,6 +688,9 @@ def main():
         torch.cuda.empty_cache()
     if "sib" in only:
         others.update(bench_siblings(args.steps, args.warmup))
+        torch.cuda.empty_cache()
+    if "lib16" in only:  # opt-in: vendor-library rows for the 16-bit GEMMs
+        others["library_baselines_16bit"] = bench_16bit_library_baselines(args.steps, args.warmup)
         torch.cuda.empty_cache()
     line = {
         "metric": "FP8 GEMM/attention TFLOP/s + % of MI355X FP8 MFMA peak (or % HBM BW), 1 GPU",
