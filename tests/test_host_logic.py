@@ -96,3 +96,19 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "_LIB_PATH", tmp_path / "nope.so")
     with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
         _lib.load()
+
+
+def test_product_package_never_touches_the_oracle():
+    """The oracle is the checker: nothing under helion_amd/ may import, read or run it (and importing the package must not
+    pull it in as a side effect either)."""
+    import pathlib
+    import subprocess
+    import sys
+
+    root = pathlib.Path(__file__).resolve().parent.parent
+    for f in (root / "helion_amd").rglob("*"):
+        if f.suffix in (".py", ".hip", ".h", ".cpp"):
+            assert "oracle" not in f.read_text(), f
+    code = "import sys, helion_amd; assert not any(m == 'oracle' or m.startswith('oracle.') for m in sys.modules), 'oracle imported'"
+    r = subprocess.run([sys.executable, "-c", code], cwd=root, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-500:]
