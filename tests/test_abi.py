@@ -166,3 +166,29 @@ def test_fp8_attention_path_selection():
     assert lib.hx_fp8_attention_path(2, 128, 96, 128, 1, A, A, A, A) == 0        # (the Python op zero-pads such heads to 128)
     assert lib.hx_fp8_attention_path(2, 128, 256, 128, 1, A, A, A, A) == 0
     assert lib.hx_fp8_attention_path(2, 128, 128, 128, 1, A + 8, A, A, A) == 0   # misaligned q
+
+
+def test_header_is_plain_c_and_links_against_the_library(tmp_path):
+    """The boundary is a C ABI: the header must compile as C99 with nothing but the standard headers, and a C program
+    that calls a query function must link against the built library and run without a GPU."""
+    import shutil
+    import subprocess
+
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    root = pathlib.Path(__file__).resolve().parent.parent
+    src = tmp_path / "abi.c"
+    src.write_text('#include <stdio.h>\n#include "hx_kernels.h"\n'
+                   "int main(void) {\n"
+                   "  if (hx_version() <= 0) return 1;\n"
+                   "  if (hx_fp8_gemm_workspace_bytes(8192, 8192, 8192, 1, 8192) != 0) return 2;\n"
+                   "  if (hx_fp8_gemm(0, 0, 0, -1, 1, 1, 1, 1, 1, 1, 0, 0, 1, 0, 0, 0) >= 0) return 3;  /* negative size: an error, no launch */\n"
+                   '  printf("%s\\n", hx_last_error());\n'
+                   "  return 0;\n}\n")
+    lib = _lib.lib_path()
+    exe = tmp_path / "abi"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", str(root / "include"), str(src), "-o", str(exe),
+                    str(lib), f"-Wl,-rpath,{lib.parent}"], check=True, capture_output=True, text=True, timeout=120)
+    r = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, (r.returncode, r.stderr[-300:])
+    assert "hx_fp8_gemm" in r.stdout
