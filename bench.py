@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only c2,lib,c3,c4,c5,next,sib[,lib16]] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only c2,lib,c3,c4,c5,next,sib[,lib16]] [--no-cpu-baseline] [--clock-probe]
 
 A "step" is one launch of the FP8 GEMM at the headline configuration (M=N=K=8192, e4m3 operands, B column-major,
 per-tensor fp32 scales, bf16 output) with inputs resident in HBM.
@@ -15,15 +15,18 @@ Timing protocol, the same for every kernel timed here:
   3. exactly K timed launches, every launch bracketed by its own pair of HIP events on the launch stream; the
      reported time per launch is the MEDIAN of the K event pairs (mean, min and max are printed next to it, and so
      is the mean over one event pair around all K launches).
-  4. clock phase, after the timed region and outside it: CLOCK_PHASE_LAUNCHES more launches of the same kernel,
-     back to back with the timed ones, while a one-wave probe kernel (hx_clock_probe) runs three times on a second
-     stream: it reads the shader-clock counter against the constant 100 MHz counter over 50 us, which gives the
-     engine clock the chip sustains under this kernel's load (it is power-limited well below its 2.4 GHz maximum).
-     Printed as "engine_clock_mhz" with the MFMA peak recomputed at that clock.  The probe needs a free wave slot: next
-     to a kernel whose waves fill the register file (the 256x256 tile GEMMs, fp8 and 16-bit) it only runs while a launch
-     drains and reads a chip that has just gone idle, so for those rows the printed clock is an upper bound (counters read
-     inside an instrumented build of the grouped GEMM showed 1.87 GHz where this probe printed 2.34).  (amdsmi's clock readings are refreshed
-     about once a second, too slow for a timed region of a few milliseconds; its socket power is printed as a hint.)
+  4. only with --clock-probe (off by default: the default run launches nothing but the kernels under test): after the
+     timed region and outside it, CLOCK_PHASE_LAUNCHES more launches of the same kernel while a one-wave probe kernel
+     (hx_clock_probe) runs three times on a second stream: it reads the shader-clock counter against the constant
+     100 MHz counter over 50 us.  The probe needs a free wave slot: next to a kernel whose waves fill the register file
+     (the 256x256 tile GEMMs, fp8 and 16-bit) it only runs while a launch drains and reads a chip that has just gone
+     idle, so for those rows its clock is an upper bound.  Without the flag "engine_clock_mhz" is null and no
+     clock-relative peak is printed.
+
+The engine clock and the share of cycles the matrix pipes are busy are reported from hardware counters instead
+("counters" inside each roofline object): recorded rocprofv3 --pmc values (GRBM_GUI_ACTIVE over the traced duration,
+SQ_VALU_MFMA_BUSY_CYCLES over the SIMDs' cycles) kept under profiles/ and, like the traffic figure, printed only while the
+kernel's source files still hash to the digest recorded with them.
 
 The decode-shape GEMM (a 38 us kernel) is the one exception to 3: a pair of events around a single launch adds about
 2 us to it, so its figure is the average over the K launches issued back to back through the C ABI inside one event pair
@@ -59,6 +62,7 @@ SETTLE_MIN_LAUNCHES = 40
 SETTLE_SECONDS = 0.4
 CLOCK_PHASE_LAUNCHES = 6
 CLOCK_PROBE_TICKS = 5000  # of the 100 MHz counter = 50 us
+CLOCK_PROBE = False       # --clock-probe
 
 
 # ----------------------------------------------------------------------------------------------------------------
@@ -170,9 +174,11 @@ def _time_launches(fn, steps, warmup, settle=True):
     end.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    for _ in range(2):  # keep the chip loaded between the synchronisation above and the clock phase
-        fn()
-    clock = _clock_phase(fn)
+    clock = None
+    if CLOCK_PROBE:
+        for _ in range(2):  # keep the chip loaded between the synchronisation above and the clock phase
+            fn()
+        clock = _clock_phase(fn)
     per = [s.elapsed_time(e) for s, e in pairs]
     return {"median_ms": statistics.median(per), "mean_ms": sum(per) / len(per), "min_ms": min(per), "max_ms": max(per),
             "whole_region_mean_ms": start.elapsed_time(end) / steps, "wall_ms_per_step": wall_ms, "timed_launches": steps,
@@ -209,13 +215,32 @@ def _traffic(name):
     return None, None
 
 
+def _counters(name):
+    """Engine clock and matrix-pipe occupancy of a kernel from hardware counters: a recorded profile value like _traffic's,
+    read from the line `kernel_counters <name> <clock_mhz> <mfma_busy> <digest> <source files...>` of the counter summary
+    under profiles/ and reported only while <digest> matches the kernel sources as they are now.
+    clock_mhz = GRBM_GUI_ACTIVE / XCDs / traced duration; mfma_busy = SQ_VALU_MFMA_BUSY_CYCLES / SIMDs / (GRBM_GUI_ACTIVE / XCDs)."""
+    f = ROOT / "profiles" / "sq_tcc_counters_all_kernels.txt"
+    if f.exists():
+        for line in f.read_text().splitlines():
+            parts = line.split()
+            if len(parts) >= 6 and parts[0] == "kernel_counters" and parts[1] == name:
+                if _sources_digest(parts[5:]) == parts[4]:
+                    return {"clock_mhz": float(parts[2]), "mfma_busy": float(parts[3]), "file": "profiles/" + f.name,
+                            "kernel_sources": parts[5:], "sources_sha256_16": parts[4],
+                            "note": "recorded rocprofv3 --pmc values for these exact kernel sources (a profile run, not this run)"}
+                return {"clock_mhz": None, "mfma_busy": None, "file": "profiles/" + f.name,
+                        "note": "kernel sources changed since the counters were recorded: not reported"}
+    return None
+
+
 def _mfma_roofline(flops, t, peak, flop_per_cu_clk, kernel, traffic_name=None):
     ms = t["median_ms"]
     tf = flops / (ms * 1e-3) / 1e12
     traffic, src = _traffic(traffic_name) if traffic_name else (None, None)
     r = {"bound": "mfma", "achieved": tf, "peak": peak, "unit": "TFLOP/s", "frac": tf / peak, "traffic": traffic,
          "traffic_source": src, "kernel": kernel, "launch_ms": ms, "launch_ms_statistic": "median of per-launch HIP event pairs",
-         "algorithmic_flops_per_launch": flops}
+         "algorithmic_flops_per_launch": flops, "counters": _counters(traffic_name) if traffic_name else None}
     cus, fmax = _DEV.get("compute_units"), _DEV.get("max_engine_clock_mhz")
     if cus and fmax:
         r["peak_recomputed"] = cus * fmax * 1e6 * flop_per_cu_clk / 1e12
@@ -235,7 +260,7 @@ def _hbm_roofline(nbytes, t, kernel, traffic_name=None):
     traffic, src = _traffic(traffic_name) if traffic_name else (None, None)
     r = {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS, "traffic": traffic,
          "traffic_source": src, "kernel": kernel, "launch_ms": ms, "launch_ms_statistic": "median of per-launch HIP event pairs",
-         "algorithmic_bytes_per_launch": float(nbytes)}
+         "algorithmic_bytes_per_launch": float(nbytes), "counters": _counters(traffic_name) if traffic_name else None}
     r.update(_timing_fields(t))
     return r
 
@@ -631,13 +656,15 @@ def cpu_checks():
 
 
 def main():
-    global _SMI, _DEV
+    global _SMI, _DEV, CLOCK_PROBE
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--only", default="c2,lib,c3,c4,c5,next,sib")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--clock-probe", action="store_true",
+                    help="after each timed region, run the one-wave clock probe next to six more launches (off by default)")
     ap.add_argument("--no-settle", action="store_true", help="skip the settle phase (profiling runs that want few launches)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run three plain 1 GiB device copies (a known-traffic kernel to scale rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE by)")
@@ -646,6 +673,7 @@ def main():
         print("bench.py: this build measures one GPU only (no sharding, no collectives); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
+    CLOCK_PROBE = args.clock_probe
     _SMI = _Smi()
     _DEV = _SMI.static()
 

@@ -10,10 +10,10 @@ __global__ __launch_bounds__(64) void hx_clock_probe_kernel(uint64_t* __restrict
   const uint64_t c0 = __builtin_readcyclecounter();
   const uint64_t r0 = wall_clock64();
   uint64_t r1 = r0;
-  // bounded wait: every iteration sleeps ~64 clocks; the loop count caps the kernel at a few milliseconds even if the
-  // 100 MHz counter were stuck
-  for (int i = 0; i < 200000 && (long long)(r1 - r0) < ticks; ++i) {
-    __builtin_amdgcn_s_sleep(1);
+  // bounded, sparse wait: every iteration sleeps ~8000 clocks (3-4 us) before it reads the 100 MHz counter again, and
+  // 64 iterations (about 0.25 ms) end the kernel even if that counter were stuck
+  for (int i = 0; i < 64 && (long long)(r1 - r0) < ticks; ++i) {
+    __builtin_amdgcn_s_sleep(127);
     r1 = wall_clock64();
   }
   const uint64_t c1 = __builtin_readcyclecounter();
@@ -25,8 +25,8 @@ __global__ __launch_bounds__(64) void hx_clock_probe_kernel(uint64_t* __restrict
 }
 
 extern "C" int hx_clock_probe(uint64_t* out2, int64_t ticks_100mhz, void* stream) {
-  if (!out2 || ticks_100mhz <= 0 || ticks_100mhz > 1000000) {
-    hx_set_error("hx_clock_probe: out2 must be a device pointer to two uint64 and 0 < ticks <= 1000000 (10 ms)");
+  if (!out2 || ticks_100mhz <= 0 || ticks_100mhz > 10000) {
+    hx_set_error("hx_clock_probe: out2 must be a device pointer to two uint64 and 0 < ticks <= 10000 (100 us)");
     return HX_ERR_BAD_ARG;
   }
   hx_launch(hx_clock_probe_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, out2, (long long)ticks_100mhz);

@@ -224,10 +224,12 @@ int hx_attention(const void* q, const void* k, const void* v, void* out, int64_t
 int hx_attention_path(int64_t BH, int64_t M, int64_t N, int64_t D, int dtype, const void* q, const void* k, const void* v,
                       const void* out);
 
-/* Measurement aid, no counterpart in the reference: one wave that measures the engine clock of the XCD it lands on
- * as (shader-clock counter delta) / (100 MHz counter delta) over `ticks_100mhz` ticks of the latter (at most
- * 1000000 = 10 ms).  out2: device pointer to two uint64 {shader clocks, 100 MHz ticks}; MHz = 100 * out2[0] / out2[1].
- * Launched on a second stream while another kernel runs, it reads the clock that kernel is sustained at. */
+/* ---- Diagnostics (not part of the drop-in interface; no counterpart in the reference) --------------------------------
+ * One wave that measures the engine clock of the XCD it lands on as (shader-clock counter delta) / (100 MHz counter
+ * delta) over `ticks_100mhz` ticks of the latter (at most 10000 = 100 us; the wave sleeps 3-4 us between two readings of
+ * the counter).  out2: device pointer to two uint64 {shader clocks, 100 MHz ticks}; MHz = 100 * out2[0] / out2[1].
+ * Launched on a second stream while another kernel runs, it reads the clock that kernel is sustained at, provided that
+ * kernel leaves a wave slot free.  Only `bench.py --clock-probe` calls it. */
 int hx_clock_probe(uint64_t* out2, int64_t ticks_100mhz, void* stream);
 
 #ifdef __cplusplus
