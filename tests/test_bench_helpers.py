@@ -51,6 +51,42 @@ def test_traffic_is_reported_only_for_the_sources_it_was_recorded_with(tmp_path,
     assert bench._traffic("mykernel")[0] is None
 
 
+def test_counters_are_reported_only_for_the_sources_they_were_recorded_with(tmp_path, monkeypatch):
+    root = tmp_path
+    (root / "profiles").mkdir()
+    (root / "helion_amd" / "csrc").mkdir(parents=True)
+    (root / "helion_amd" / "csrc" / "k.hip").write_text("kernel v1")
+    monkeypatch.setattr(bench, "ROOT", root)
+    digest = bench._sources_digest(["k.hip"])
+    (root / "profiles" / "sq_tcc_counters_all_kernels.txt").write_text(f"text\nkernel_counters mykernel 1929 0.758 {digest} k.hip\n")
+    c = bench._counters("mykernel")
+    assert c["clock_mhz"] == 1929.0 and c["mfma_busy"] == 0.758 and c["sources_sha256_16"] == digest
+    assert bench._counters("another") is None
+    (root / "helion_amd" / "csrc" / "k.hip").write_text("kernel v2")
+    c = bench._counters("mykernel")
+    assert c["clock_mhz"] is None and c["mfma_busy"] is None and "changed" in c["note"]
+
+
+def test_roofline_carries_counters_and_no_probe_fields_by_default(tmp_path, monkeypatch):
+    """Without --clock-probe no probe kernel runs: engine_clock_mhz stays null and no clock-relative peak is printed."""
+    assert bench.CLOCK_PROBE is False
+    r = bench._mfma_roofline(2.0 * 8192**3, _T, bench.PEAK_FP8_TFLOPS, bench.FP8_FLOP_PER_CU_CLK, "k", "fp8_gemm_tile256_c2")
+    assert r["engine_clock_mhz"] is None
+    assert "peak_at_achieved_clock" not in r and "frac_of_peak_at_achieved_clock" not in r
+    assert "counters" in r  # a dict (current digest or the reason it is withheld)
+    assert r["counters"] is None or "note" in r["counters"]
+
+
+def test_recorded_counter_lines_are_well_formed():
+    f = bench.ROOT / "profiles" / "sq_tcc_counters_all_kernels.txt"
+    lines = [l.split() for l in f.read_text().splitlines() if l.startswith("kernel_counters ")]
+    assert any(p[1] == "fp8_gemm_tile256_c2" for p in lines)
+    for p in lines:
+        assert 500 < float(p[2]) < 2600 and 0.0 <= float(p[3]) <= 1.0 and len(p[4]) == 16
+        for src in p[5:]:
+            assert (bench.ROOT / "helion_amd" / "csrc" / src).exists(), src
+
+
 def test_headline_traffic_record_names_existing_sources():
     """Every recorded traffic line must name kernel source files that exist (whether its digest is current is the bench's
     business at run time)."""
