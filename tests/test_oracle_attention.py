@@ -155,3 +155,31 @@ def test_tiled_is_tile_invariant_when_p_is_exact():
     a = orc.fp8_attention_tiled(q, k, v, 1, 1, 16, torch.float32)
     b = orc.fp8_attention(q, k, v, 1, 1, torch.float32)
     assert torch.allclose(a, b, rtol=0, atol=1e-6)
+
+
+def test_tiled_rescale_path_against_the_closed_form_when_p_is_not_quantised(monkeypatch):
+    """Pins the alpha path (l and acc rescaled when the running max moves) by mathematics rather than by a second
+    statement of the recurrence: with the e4m3 cast of p taken out (here only, through a patch local to this test) the
+    online recurrence is an exact re-association of softmax(scores) @ v, so for any tiling it must equal the closed form
+    evaluated in float64 - and it must do so on rows whose maximum moves from tile to tile, where alpha != 1.  A dropped
+    or inverted alpha, or one applied to only one of l and acc, fails this by orders of magnitude."""
+    monkeypatch.setattr(orc, "to_e4m3", lambda x: x)  # p stays fp32 ...
+    decode = orc.dq
+    monkeypatch.setattr(orc, "dq", lambda t: t if t.dtype == torch.float32 else decode(t))  # ... and is used as it is
+    s, d, tile = 96, 32, 16
+    q, k, v = _inputs(1, 1, s, d, 21)
+    qd, kd, vd = (orc.e4m3_decode(t[0].view(torch.uint8).numpy()).astype(np.float64) for t in (q, k, v))
+    c = float(np.float32((1.0 / math.sqrt(float(d))) * 1.44269504))
+    sc = qd @ kd.T * c
+    # the running max must move in later tiles for most rows, or the test would not exercise alpha
+    tile_of_max = sc.argmax(1) // tile
+    first_tile_max = sc[:, :tile].max(1)
+    moves = (sc.max(1) > first_tile_max + 0.5).sum()
+    assert moves >= s // 2 and (tile_of_max > 0).sum() >= s // 2
+    w = np.exp2(sc - sc.max(1, keepdims=True))
+    want = (w @ vd.T) / w.sum(1, keepdims=True)
+    for t in (tile, 32, 40):
+        got = orc.fp8_attention_tiled(q, k, v, 1, 1, t, torch.float32)[0, 0].numpy().astype(np.float64)
+        assert np.abs(got - want).max() <= 2e-6 * max(1.0, np.abs(want).max())
+    one = orc.fp8_attention_tiled(q, k, v, 1, 1, s, torch.float32)[0, 0].numpy().astype(np.float64)
+    assert np.abs(one - want).max() <= 2e-6 * max(1.0, np.abs(want).max())

@@ -21,10 +21,11 @@ def _tables(ex, E):
     return counts, offsets, idx
 
 
-def _both(T, K, N, E, dtype, seed, poison):
+def _both(T, K, N, E, dtype, seed, poison, path):
     lib = _lib.load()
     A, W, ex = inputs.moe_inputs(T, K, N, E, 1, seed=seed, dtype=dtype)
     A, W, ex = A.to(DEV), W.to(DEV), ex.to(DEV)
+    assert lib.hx_moe_path(T, K, N, E, 1, A.data_ptr(), W.data_ptr(), A.data_ptr()) == path  # the kernel this case is meant for
     if E > 2:
         ex[ex == 1] = 0  # an empty expert
     counts, offsets, idx = _tables(ex, E)
@@ -51,12 +52,15 @@ def _both(T, K, N, E, dtype, seed, poison):
 
 
 def test_two_calls_in_a_row_second_smaller():
-    # first call: 256-row tile kernel, two-launch table build (T > 4096); second: fewer rows, fewer experts, the
-    # one-launch table build and the 128-row tiles -- it reads only what it wrote itself into the shared array
-    _both(6000, 256, 512, 8, torch.bfloat16, seed=11, poison=3.0)
-    _both(700, 128, 264, 5, torch.float16, seed=12, poison=-2.0)
-    # and a larger one again, through the general kernel (K % 64 != 0)
-    _both(1000, 500, 200, 30, torch.float16, seed=13, poison=1.0)
+    # first call: 128-row MFMA tiles, two-launch table build (T > 4096); second: fewer rows, fewer experts, the one-launch
+    # table build -- it reads only what it wrote itself into the shared array
+    _both(6000, 256, 512, 8, torch.bfloat16, seed=11, poison=3.0, path=2)
+    _both(700, 128, 264, 5, torch.float16, seed=12, poison=-2.0, path=2)
+    # a larger one again: the reference's own check shape, K = 500 (rows of A only 4-byte aligned): the 128-row MFMA
+    # tiles with a partial last k-tile and A fetched in 4-byte pieces
+    _both(1000, 500, 200, 30, torch.float16, seed=13, poison=1.0, path=5)
+    # and an odd K, which only the fp32-FMA kernel takes
+    _both(900, 251, 200, 6, torch.float16, seed=14, poison=-1.0, path=0)
 
 
 def test_rejects_sizes_beyond_the_built_in_scratch():
