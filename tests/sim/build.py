@@ -1,0 +1,101 @@
+"""Builds tests/sim/libhx_sim.so: the kernel sources of helion_amd/csrc compiled for the host CPU against the execution
+model in hx_sim.h / hx_sim.cpp, behind the same C ABI as the real library (test infrastructure: nothing under helion_amd/
+refers to it).
+
+    python tests/sim/build.py [-q]
+
+The sources are copied into tests/sim/_build with two kinds of change, both listed here and nowhere else:
+  * helion_amd/csrc/hx_common.h is replaced by tests/sim/hx_common.h (the same names; inline assembly and the launch
+    helper expressed through the model);
+  * the inline assembly inside the kernel files themselves (REWRITES below) is replaced by the C it stands for.
+Everything else is compiled exactly as the device compiler sees it."""
+from __future__ import annotations
+
+import hashlib
+import pathlib
+import re
+import shutil
+import subprocess
+import sys
+
+SIM = pathlib.Path(__file__).resolve().parent
+ROOT = SIM.parent.parent
+CSRC = ROOT / "helion_amd" / "csrc"
+BUILD = SIM / "_build"
+LIB = SIM / "libhx_sim.so"
+CXX = "/opt/rocm/llvm/bin/clang++"
+UNITS = ["hx_common.cpp", "fp8_gemm.hip", "fp8_attention.hip", "moe_gemm.hip", "moe_routing.hip", "fp8_quantize.hip",
+         "matmul16.hip", "attention16.hip", "diag.hip"]
+FLAGS = ["-std=c++17", "-O1", "-g", "-fPIC", "-fno-strict-aliasing", "-ffp-contract=off", "-Wno-unknown-attributes",
+         "-Wno-unused-value", "-Wno-builtin-macro-redefined", "-Wno-reserved-macro-identifier", "-Wno-macro-redefined",
+         "-Wno-ignored-attributes", "-Wno-pass-failed", "-Wno-unknown-pragmas", "-fno-stack-protector", "-mf16c"]
+
+# (file, what the device source says, what the host build compiles instead)
+REWRITES = [
+    ("fp8_attention.hip", 'asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));', "d = fmaxf(fmaxf(a, b), c);"),
+    ("fp8_attention.hip", 'asm volatile("" : "+v"(nv));', ";"),
+    ("fp8_gemm.hip", 'asm volatile("" : "+v"(zero));', ";"),
+    ("gemm16_tile256.h", 'asm volatile("" : "+v"(t));', ";"),
+    ("hx_common.cpp", "#include <hip/hip_runtime.h>", ""),
+    ("hx_common.cpp", '#include "../../include/hx_kernels.h"', '#include "hx_kernels.h"'),
+]
+
+
+def _stamp() -> str:
+    h = hashlib.sha256()
+    for p in sorted(list(CSRC.glob("*.hip")) + list(CSRC.glob("*.h")) + list(CSRC.glob("*.cpp")) + list(SIM.glob("hx_*"))
+                    + [SIM / "build.py", ROOT / "include" / "hx_kernels.h"]):
+        h.update(p.name.encode())
+        h.update(p.read_bytes())
+    return h.hexdigest()
+
+
+def is_current() -> bool:
+    s = BUILD / "stamp"
+    return LIB.exists() and s.exists() and s.read_text() == _stamp()
+
+
+def build(verbose: bool = False) -> pathlib.Path:
+    if BUILD.exists():
+        shutil.rmtree(BUILD)
+    BUILD.mkdir(parents=True)
+    for p in list(CSRC.glob("*.hip")) + list(CSRC.glob("*.h")) + list(CSRC.glob("*.cpp")):
+        if p.name == "hx_common.h":
+            continue
+        text = p.read_text()
+        for name, old, new in REWRITES:
+            if name == p.name:
+                if old not in text:
+                    raise RuntimeError(f"{p.name}: the text a host rewrite applies to is gone: {old!r}")
+                text = text.replace(old, new)
+        if re.search(r"\basm\b", text):
+            raise RuntimeError(f"{p.name}: inline assembly without a host rewrite")
+        (BUILD / (p.name.replace(".hip", ".cpp") if p.suffix == ".hip" else p.name)).write_text(text)
+    shutil.copy(SIM / "hx_common.h", BUILD / "hx_common.h")
+    procs, objs = [], []
+    common = [CXX, *FLAGS, "-I", str(ROOT / "include"), "-I", str(SIM), "-include", str(SIM / "hx_sim.h")]
+    for u in UNITS:
+        src = BUILD / u.replace(".hip", ".cpp")
+        obj = BUILD / (src.stem + ".o")
+        cmd = [*common, "-c", str(src), "-o", str(obj)]
+        if verbose:
+            print(" ".join(cmd))
+        procs.append((u, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        objs.append(str(obj))
+    obj = BUILD / "hx_sim.o"
+    procs.append(("hx_sim.cpp", subprocess.Popen([CXX, *FLAGS, "-I", str(SIM), "-c", str(SIM / "hx_sim.cpp"), "-o", str(obj)],
+                                                 stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+    objs.append(str(obj))
+    for u, p in procs:
+        out, _ = p.communicate()
+        if p.returncode != 0:
+            raise RuntimeError(f"host build of {u} failed:\n{out[-6000:]}")
+        if verbose and out.strip():
+            print(out)
+    subprocess.check_call([CXX, "-shared", "-fPIC", "-o", str(LIB), *objs])
+    (BUILD / "stamp").write_text(_stamp())
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(verbose="-q" not in sys.argv))

@@ -1,0 +1,104 @@
+"""Python side of the host execution model (tests/sim/hx_sim.h): loads tests/sim/libhx_sim.so - the kernel sources
+compiled for the CPU behind the library's own C ABI - and hands out operand buffers that sit between inaccessible pages.
+Used by the `not gpu` tests only; the package under helion_amd/ never touches it."""
+from __future__ import annotations
+
+import ctypes
+import pathlib
+import sys
+
+import torch
+
+SIM = pathlib.Path(__file__).resolve().parent
+sys.path.insert(0, str(SIM))
+import build as _build  # noqa: E402
+
+from helion_amd import _lib as _real  # noqa: E402  (for the signature table and the dtype tags only)
+
+_c = ctypes
+_lib = None
+
+
+def load():
+    global _lib
+    if _lib is None:
+        if not _build.is_current():
+            _build.build()
+        lib = ctypes.CDLL(str(_build.LIB))
+        for name, (res, args) in _real._SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = res, args
+        lib.hx_sim_alloc.restype, lib.hx_sim_alloc.argtypes = _c.c_void_p, [_c.c_size_t, _c.c_int]
+        lib.hx_sim_free_all.restype, lib.hx_sim_free_all.argtypes = None, []
+        lib.hx_sim_config.restype, lib.hx_sim_config.argtypes = None, [_c.c_int, _c.c_int, _c.c_int]
+        lib.hx_sim_last_fault.restype, lib.hx_sim_last_fault.argtypes = _c.c_char_p, []
+        lib.hx_sim_reset.restype, lib.hx_sim_reset.argtypes = None, []
+        lib.hx_sim_counters.restype, lib.hx_sim_counters.argtypes = None, [_c.POINTER(_c.c_uint64)]
+        lib.hx_sim_cvt_pk_fp8.restype, lib.hx_sim_cvt_pk_fp8.argtypes = _c.c_int, [_c.c_float, _c.c_float]
+        _lib = lib
+    return _lib
+
+
+# the scheduling / DMA-landing variants a kernel must give the same answer under:
+# (dma_lazy, wave_order, interleave)
+VARIANTS = {"eager": (0, 0, 0), "lazy": (1, 0, 0), "lazy-reverse": (1, 1, 0), "eager-interleaved": (0, 1, 1), "lazy-interleaved": (1, 0, 1)}
+
+
+class Arena:
+    """Operand buffers for one test case.  `end_flush` puts the last byte of every buffer right before an inaccessible
+    page (overruns fault at the first byte); otherwise the first byte sits right behind one (underruns do)."""
+
+    def __init__(self, end_flush: bool = True):
+        self.lib = load()
+        self.end_flush = end_flush
+        self._keep = []
+
+    def empty(self, nbytes: int) -> torch.Tensor:
+        nbytes = max(int(nbytes), 1)
+        p = self.lib.hx_sim_alloc(nbytes, 1 if self.end_flush else 0)
+        assert p, "hx_sim_alloc failed"
+        raw = (_c.c_uint8 * nbytes).from_address(p)
+        self._keep.append(raw)
+        return torch.frombuffer(raw, dtype=torch.uint8)
+
+    def put(self, t: torch.Tensor) -> torch.Tensor:
+        """A copy of the contiguous tensor `t` in a guarded buffer, same dtype and shape."""
+        t = t.contiguous()
+        b = self.empty(t.numel() * t.element_size())
+        b[: t.numel() * t.element_size()].copy_(t.view(torch.uint8).reshape(-1))
+        return b[: t.numel() * t.element_size()].view(t.dtype).reshape(t.shape)
+
+    def out(self, shape, dtype, fill=None) -> torch.Tensor:
+        n = 1
+        for s in shape:
+            n *= int(s)
+        es = torch.empty((), dtype=dtype).element_size()
+        b = self.empty(n * es)
+        t = b[: n * es].view(dtype).reshape(shape)
+        if fill is not None:
+            t.view(torch.uint8).fill_(fill)
+        return t
+
+    def close(self):
+        self._keep.clear()
+        self.lib.hx_sim_free_all()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+
+def check(rc: int, what: str) -> None:
+    if rc == 0:
+        return
+    lib = load()
+    msg = lib.hx_last_error().decode("utf-8", "replace")
+    fault = lib.hx_sim_last_fault().decode("utf-8", "replace")
+    lib.hx_sim_reset()
+    raise AssertionError(f"{what}: rc {rc}: {msg} | {fault}")
+
+
+def configure(variant: str) -> None:
+    load().hx_sim_config(*VARIANTS[variant])
