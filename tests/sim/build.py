@@ -7,7 +7,9 @@ refers to it).
 The sources are copied into tests/sim/_build with two kinds of change, both listed here and nowhere else:
   * helion_amd/csrc/hx_common.h is replaced by tests/sim/hx_common.h (the same names; inline assembly and the launch
     helper expressed through the model);
-  * the inline assembly inside the kernel files themselves (REWRITES below) is replaced by the C it stands for.
+  * the inline assembly inside the kernel files themselves (REWRITES below) is replaced by the C it stands for, and the
+    one place where a kernel relies on the lanes of a wave executing an instruction together is marked as a wave-wide
+    step.
 Everything else is compiled exactly as the device compiler sees it."""
 from __future__ import annotations
 
@@ -36,6 +38,11 @@ REWRITES = [
     ("fp8_attention.hip", 'asm volatile("" : "+v"(nv));', ";"),
     ("fp8_gemm.hip", 'asm volatile("" : "+v"(zero));', ";"),
     ("gemm16_tile256.h", 'asm volatile("" : "+v"(t));', ";"),
+    # The lanes of a wave execute one instruction together: all of them have read the slot before the first lane of the
+    # group stores the advanced one.  The model runs the lanes of a wave one after the other between two cross-lane
+    # instructions, so the place where the kernel relies on that order is marked as one.
+    ("moe_routing.hip", "    const int slot = hist[w][e];  // every lane of the group reads before its first lane advances the slot\n",
+     "    const int slot = hist[w][e];\n    hxsim::wave_sync(__LINE__);\n"),
     ("hx_common.cpp", "#include <hip/hip_runtime.h>", ""),
     ("hx_common.cpp", '#include "../../include/hx_kernels.h"', '#include "hx_kernels.h"'),
 ]
@@ -43,7 +50,7 @@ REWRITES = [
 
 def _stamp() -> str:
     h = hashlib.sha256()
-    for p in sorted(list(CSRC.glob("*.hip")) + list(CSRC.glob("*.h")) + list(CSRC.glob("*.cpp")) + list(SIM.glob("hx_*"))
+    for p in sorted(list(CSRC.glob("*.hip")) + list(CSRC.glob("*.h")) + list(CSRC.glob("*.cpp")) + list(SIM.glob("hx_*")) + [SIM / "selftest_kernels.cpp"]
                     + [SIM / "build.py", ROOT / "include" / "hx_kernels.h"]):
         h.update(p.name.encode())
         h.update(p.read_bytes())
@@ -82,8 +89,13 @@ def build(verbose: bool = False) -> pathlib.Path:
             print(" ".join(cmd))
         procs.append((u, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
         objs.append(str(obj))
+    shutil.copy(SIM / "selftest_kernels.cpp", BUILD / "selftest_kernels.cpp")
+    obj = BUILD / "selftest_kernels.o"
+    procs.append(("selftest_kernels.cpp", subprocess.Popen([*common, "-c", str(BUILD / "selftest_kernels.cpp"), "-o", str(obj)],
+                                                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+    objs.append(str(obj))
     obj = BUILD / "hx_sim.o"
-    procs.append(("hx_sim.cpp", subprocess.Popen([CXX, *FLAGS, "-I", str(SIM), "-c", str(SIM / "hx_sim.cpp"), "-o", str(obj)],
+    procs.append(("hx_sim.cpp", subprocess.Popen([CXX, *FLAGS, "-O3", "-I", str(SIM), "-c", str(SIM / "hx_sim.cpp"), "-o", str(obj)],
                                                  stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
     objs.append(str(obj))
     for u, p in procs:
@@ -92,7 +104,7 @@ def build(verbose: bool = False) -> pathlib.Path:
             raise RuntimeError(f"host build of {u} failed:\n{out[-6000:]}")
         if verbose and out.strip():
             print(out)
-    subprocess.check_call([CXX, "-shared", "-fPIC", "-o", str(LIB), *objs])
+    subprocess.check_call([CXX, "-shared", "-fPIC", "-o", str(LIB), *objs, "-ldl"])
     (BUILD / "stamp").write_text(_stamp())
     return LIB
 

@@ -98,7 +98,7 @@ static inline void hx_launch(void (*kernel)(KArgs...), dim3 grid, dim3 block, un
   static_assert(sizeof...(KArgs) == sizeof...(Args), "hx_launch: argument count does not match the kernel's");
   (void)shmem;
   std::tuple<KArgs...> vals{static_cast<KArgs>(args)...};
-  const hipError_t e = hxsim::run(grid, block, [&]() { std::apply(kernel, vals); }, __PRETTY_FUNCTION__);
+  const hipError_t e = hxsim::run(grid, block, [&]() { std::apply(kernel, vals); }, (const void*)kernel);
   if (e != hipSuccess && hx_tls_launch_err == hipSuccess) hx_tls_launch_err = e;
 }
 static inline hipError_t hx_launch_status() {

@@ -2,6 +2,8 @@
 // instructions, the DMA queues, guarded operand buffers.  Test infrastructure only.
 #include "hx_sim.h"
 
+#include <cxxabi.h>
+#include <dlfcn.h>
 #include <signal.h>
 #include <stdarg.h>
 #include <stdlib.h>
@@ -84,7 +86,19 @@ static const size_t STACK = 512 << 10;
 static const int MAX_LANES = 1024;
 static bool faulted;
 static std::string fault_msg;
-static const char* launch_name = "";
+static const void* launch_fn;
+static std::string kernel_name() {
+  Dl_info info;
+  if (launch_fn && dladdr(launch_fn, &info) && info.dli_sname) {
+    int st = 0;
+    char* d = abi::__cxa_demangle(info.dli_sname, nullptr, nullptr, &st);
+    std::string s = st == 0 && d ? d : info.dli_sname;
+    free(d);
+    const size_t paren = s.find('(');
+    return paren == std::string::npos ? s : s.substr(0, paren);
+  }
+  return "?";
+}
 static uint64_t n_coll, n_dma, n_barrier, ticks;
 
 struct Buf {
@@ -108,8 +122,8 @@ static void fail(const char* fmt, ...) {
     va_end(ap);
     char where[200] = "";
     if (cur)
-      snprintf(where, sizeof where, " [kernel %s, workgroup (%u,%u,%u), work-item %d]", launch_name, geo.block_idx.x, geo.block_idx.y,
-               geo.block_idx.z, cur->tid);
+      snprintf(where, sizeof where, " [kernel %s, workgroup (%u,%u,%u), work-item %d]", kernel_name().c_str(), geo.block_idx.x,
+               geo.block_idx.y, geo.block_idx.z, cur->tid);
     fault_msg = std::string(msg) + where;
     faulted = true;
   }
@@ -119,8 +133,10 @@ static void fail(const char* fmt, ...) {
   }
 }
 
-static std::string describe_address(const void* p) {
+static std::string describe_address(const void* p, size_t n = 1) {
   const uint8_t* a = (const uint8_t*)p;
+  for (const Buf& b : bufs)
+    if (a >= b.base && a < b.base + b.bytes && a + n > b.base + b.bytes) a = b.base + b.bytes;  // starts inside, runs over the end
   char s[300];
   for (size_t i = 0; i < bufs.size(); ++i) {
     const Buf& b = bufs[i];
@@ -198,7 +214,7 @@ static uint8_t* lds_ptr(uint32_t addr, int bytes, const char* what) {
 void dma(const void* gptr, uint32_t lds_dst, int bytes) {
   ++n_dma;
   if (!bufs.empty() && !in_a_buffer(gptr, bytes))
-    fail("global->LDS DMA reads %d bytes out of bounds: address %p is %s", bytes, gptr, describe_address(gptr).c_str());
+    fail("global->LDS DMA reads %d bytes at %p out of bounds: %s", bytes, gptr, describe_address(gptr, bytes).c_str());
   cur->t = Dma{(const uint8_t*)gptr, lds_ptr(lds_dst, bytes, "global->LDS DMA"), bytes};
   collective(C_DMA, 0);  // one wave instruction: the active lanes' transfers travel (and are waited for) together
 }
@@ -548,7 +564,7 @@ static void run_workgroup(dim3 block) {
     for (Wave& w : waves) land_until(w, w.q.size());  // transfers still in flight when the wave ends do complete
 }
 
-hipError_t run(dim3 grid, dim3 block, const std::function<void()>& fn, const char* what) {
+hipError_t run(dim3 grid, dim3 block, const std::function<void()>& fn, const void* kernel) {
   static bool once = false;
   if (!once) {
     once = true;
@@ -567,12 +583,13 @@ hipError_t run(dim3 grid, dim3 block, const std::function<void()>& fn, const cha
   }
   const long nthreads = (long)block.x * block.y * block.z;
   if (nthreads < 1 || nthreads > MAX_LANES || grid.x < 1 || grid.y < 1 || grid.z < 1) {
-    fault_msg = std::string("invalid launch geometry for ") + what;
+    launch_fn = kernel;
+    fault_msg = std::string("invalid launch geometry for ") + kernel_name();
     return hipErrorLaunchFailure;
   }
   if (faulted) return hipErrorLaunchFailure;  // a fault is sticky until hx_sim_reset, like a device fault is
   body = &fn;
-  launch_name = what;
+  launch_fn = kernel;
   geo.block_dim = {block.x, block.y, block.z};
   geo.grid_dim = {grid.x, grid.y, grid.z};
   for (unsigned z = 0; z < grid.z && !faulted; ++z)

@@ -93,7 +93,7 @@ uint64_t clock100mhz();
 enum { MFMA_F8_32x32x64 = 0, MFMA_F8_16x16x128, MFMA_BF16_32x32x16, MFMA_F16_32x32x16, MFMA_BF16_16x16x32, MFMA_F16_16x16x32 };
 
 // runs `fn` once per work-item of the grid; returns hipSuccess or hipErrorLaunchFailure (message: hx_sim_last_fault)
-hipError_t run(dim3 grid, dim3 block, const std::function<void()>& fn, const char* what);
+hipError_t run(dim3 grid, dim3 block, const std::function<void()>& fn, const void* kernel);
 
 }  // namespace hxsim
 

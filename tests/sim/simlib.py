@@ -35,6 +35,7 @@ def load():
         lib.hx_sim_reset.restype, lib.hx_sim_reset.argtypes = None, []
         lib.hx_sim_counters.restype, lib.hx_sim_counters.argtypes = None, [_c.POINTER(_c.c_uint64)]
         lib.hx_sim_cvt_pk_fp8.restype, lib.hx_sim_cvt_pk_fp8.argtypes = _c.c_int, [_c.c_float, _c.c_float]
+        lib.hx_sim_selftest.restype, lib.hx_sim_selftest.argtypes = _c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int]
         _lib = lib
     return _lib
 

@@ -1,0 +1,108 @@
+"""Every fp8_gemm kernel path executed on the CPU in the host execution model (tests/sim: the kernel sources themselves,
+compiled for the host) and compared with the oracle, with operands in guarded buffers and under the scheduling / DMA
+landing variants.  The model sums each MFMA exactly, so where the output type rounds the same way the comparison is bit
+for bit; the tolerance is the GPU tests' one.  What this adds to the GPU tests: it runs without a GPU, an access one byte
+outside an operand stops the launch, and a transfer that is read before its wait (or a stage reused before its barrier)
+gives a wrong answer in at least one variant instead of usually getting away with it."""
+import pytest
+import torch
+
+from oracle import oracle as orc
+from tests._util import rel_err
+from tests.sim import simlib, simops
+
+E4 = torch.float8_e4m3fn
+FAST = ["lazy-reverse", "eager-interleaved"]
+ALL = list(simlib.VARIANTS)
+
+
+def _ops(m, n, k, seed, rowmajor):
+    g = torch.Generator().manual_seed(seed)
+    a = (torch.randn(m, k, generator=g) * 0.5).to(E4)
+    bt = (torch.randn(n, k, generator=g) * 0.5).to(E4)
+    return a, (bt.t().contiguous() if rowmajor else bt.t())
+
+
+# path (hx_fp8_gemm_path): 1 = 256x256 tiles, 2 = skinny (M <= 32), 3 = 256x256 guarded edges / K tail, 4 = row-major B
+# read in place, 5 = 128-column tiles, 0 = plain kernel
+@pytest.mark.parametrize("m,n,k,rowmajor,path", [
+    (512, 512, 256, False, 5),      # (small problems prefer the 128-column tiles)
+    (256, 256, 384, False, 5),
+    (300, 260, 400, False, 3),      # ragged M, N and a 16-byte K tail
+    (256, 256, 400, False, 3),
+    (256, 512, 144, False, 3),      # one full k-tile + 16
+    (256, 256, 16, False, 3),       # a single partial k-tile
+    (256, 256, 256, True, 4),
+    (300, 272, 400, True, 4),       # row-major B with ragged edges and a K tail
+    (16, 512, 2048, False, 2),
+    (32, 1024, 4096, False, 2),     # two 16-row blocks
+    (8, 4096, 1024, False, 2),      # ticketed column groups (>= 12 per workgroup at this width)
+    (1, 256, 512, False, 2),
+    (16, 256, 16384, False, 2),     # K > 8192: A panel staged through the LDS
+    (16, 256, 512, True, 0),        # row-major B for a skinny problem: transposed through the workspace (the query says 0)
+    (40, 512, 1024, False, 5),      # 64-row decode tile
+    (64, 1792, 1024, False, 5),
+    (128, 1024, 2048, False, 5),
+    (200, 640, 512, False, 5),
+    (256, 256, 8192, False, 5),     # few tiles, long K: split-K slabs + reduce
+    (33, 100, 1000, False, 0),      # K % 16 != 0: plain kernel
+    (5, 7, 24, False, 0),
+])
+def test_paths_against_the_oracle(m, n, k, rowmajor, path):
+    a, y = _ops(m, n, k, m + n + k, rowmajor)
+    sa, sb = torch.tensor(1.5), torch.tensor(0.75)
+    ref = orc.fp8_gemm(a, y, 1.5, 0.75, torch.bfloat16)
+    for variant in FAST:
+        simlib.configure(variant)
+        out = simops.fp8_gemm(a, y, sa, sb, torch.bfloat16, want_path=path)
+        assert rel_err(out, ref) <= 1e-2, variant
+
+
+def test_path_1_the_256_tile_kernel_with_1_2_3_and_5_k_tiles():
+    # enough tiles that the library picks 256x256 (the benchmark kernel); every k-tile count that has its own code shape:
+    # 1 (prologue only), 2 (no steady-state iteration), 3 and 5 (steady state, odd counts end on either stage)
+    for k in (128, 256, 384, 640):
+        a, y = _ops(2048, 2304, k, k, False)
+        ref = orc.fp8_gemm(a, y, 1.0, 1.0, torch.float32)
+        simlib.configure("lazy-reverse")
+        out = simops.fp8_gemm(a, y, None, None, torch.float32, want_path=1)
+        assert rel_err(out, ref) <= 1e-6, k
+
+
+@pytest.mark.parametrize("variant", ALL)
+@pytest.mark.parametrize("m,n,k,rowmajor,path", [(300, 260, 400, False, 3), (256, 512, 384, True, 4),
+                                                 (16, 1024, 2048, False, 2), (64, 896, 1024, False, 5)])
+def test_every_variant_on_one_case_per_path(variant, m, n, k, rowmajor, path):
+    a, y = _ops(m, n, k, 99, rowmajor)
+    simlib.configure(variant)
+    out = simops.fp8_gemm(a, y, None, None, torch.float16, want_path=path)
+    assert rel_err(out, orc.fp8_gemm(a, y, 1.0, 1.0, torch.float16)) <= 1e-2
+
+
+@pytest.mark.parametrize("end_flush", [True, False])
+def test_ragged_shapes_touch_no_byte_outside_their_operands(end_flush):
+    """Seeded sweep over ragged M / N / K (K % 16 == 0 and not), both layouts of B, every output type, with the operands'
+    last (or first) byte against an inaccessible page."""
+    import numpy as np
+    rng = np.random.default_rng(3 if end_flush else 4)
+    simlib.configure("lazy")
+    for case in range(14):
+        m = int(rng.choice([1, 7, 16, 17, 33, 100, 257, 300]))
+        n = int(rng.choice([16, 24, 100, 128, 272, 520]))
+        k = int(rng.choice([16, 48, 100, 128, 400, 1040]))
+        rowmajor = bool(rng.integers(0, 2))
+        od = [torch.float16, torch.bfloat16, torch.float32][int(rng.integers(0, 3))]
+        a, y = _ops(m, n, k, 1000 + case, rowmajor)
+        out = simops.fp8_gemm(a, y, None, None, od, end_flush=end_flush)
+        assert rel_err(out, orc.fp8_gemm(a, y, 1.0, 1.0, od)) <= 1e-2, (case, m, n, k, rowmajor, od)
+
+
+def test_ticket_word_with_stale_contents():
+    """The ticketed decode kernel's workspace word needs no initialisation: run it with the word holding ones, a
+    previous launch's tag and a large count."""
+    a, y = _ops(16, 4096, 1024, 5, False)
+    ref = orc.fp8_gemm(a, y, 1.0, 1.0, torch.bfloat16)
+    simlib.configure("lazy")
+    for stale in (0xFF, 0x00, 0x01, 0xA5):
+        out = simops.fp8_gemm(a, y, None, None, torch.bfloat16, want_path=2, poison_ws=lambda nb: torch.full((nb,), stale, dtype=torch.uint8))
+        assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), stale
