@@ -10,3 +10,15 @@ def rel_err(out: torch.Tensor, ref: torch.Tensor) -> float:
     a, b = torch.nan_to_num(a), torch.nan_to_num(b)
     denom = b.abs().max().item()
     return ((a - b).abs().max().item() / denom) if denom > 0 else (a - b).abs().max().item()
+
+
+def attention_close(out, ref, max_tol=1e-2, mean_tol=2e-5):
+    """fp8 attention results computed with the same quantisation points agree to fp32 rounding except where one
+    un-normalised p sits on an e4m3 rounding boundary and an exp2 / fused-multiply-add ulp decides it the other way: such
+    a flip moves one output row by up to ~5e-3 of max|ref|.  So: the largest deviation stays below `max_tol` and the mean
+    deviation (which a systematic error would raise, a handful of flips does not) below `mean_tol`, both relative to
+    max|ref|."""
+    o, r = out.float().cpu(), ref.float().cpu()
+    scale = float(r.abs().max())
+    d = (o - r).abs()
+    return bool(torch.isfinite(o).all()) and float(d.max()) <= max_tol * scale and float(d.mean()) <= mean_tol * scale

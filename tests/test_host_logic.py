@@ -112,3 +112,17 @@ def test_product_package_never_touches_the_oracle():
     code = "import sys, helion_amd; assert not any(m == 'oracle' or m.startswith('oracle.') for m in sys.modules), 'oracle imported'"
     r = subprocess.run([sys.executable, "-c", code], cwd=root, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stderr[-500:]
+
+
+def test_product_package_never_touches_the_host_execution_model():
+    """tests/sim (the kernel sources compiled for the CPU) is a checker like the oracle: nothing under helion_amd/ or in
+    bench.py may refer to it, and the library the package loads is the hipcc-built one only."""
+    import pathlib
+
+    root = pathlib.Path(__file__).resolve().parent.parent
+    for f in list((root / "helion_amd").rglob("*")) + [root / "bench.py"]:
+        if f.suffix in (".py", ".hip", ".h", ".cpp"):
+            text = f.read_text()
+            assert "hx_sim" not in text and "hxsim" not in text and "tests.sim" not in text and "tests/sim" not in text, f
+    from helion_amd import _lib
+    assert _lib.lib_path().name == "libhx_kernels.so" and _lib.lib_path().parent.name == "helion_amd"
