@@ -8,6 +8,7 @@ import ctypes
 import pathlib
 
 HX_F16, HX_BF16, HX_F32, HX_E4M3 = 0, 1, 2, 3
+HX_FEATURE_SKINNY_ROWMAJOR = 1
 
 _LIB_PATH = pathlib.Path(__file__).resolve().parent / "libhx_kernels.so"
 _lib = None
@@ -16,6 +17,8 @@ _c = ctypes
 _SIGNATURES = {
     "hx_version": (_c.c_int, []),
     "hx_last_error": (_c.c_char_p, []),
+    "hx_set_features": (_c.c_uint, [_c.c_uint]),
+    "hx_get_features": (_c.c_uint, []),
     "hx_fp8_gemm": (
         _c.c_int,
         [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64,
@@ -115,3 +118,9 @@ def check(rc: int, what: str) -> None:
     if rc < 0:
         raise ValueError(f"{what}: {msg} (code {rc})")
     raise RuntimeError(f"{what}: {msg} (hipError {rc})")
+
+
+def set_features(mask: int) -> int:
+    """Switch opt-in kernel paths on (HX_FEATURE_* bits, see include/hx_kernels.h); returns the previous mask.  These are
+    paths that have passed the CPU-side checks but not yet a run on the hardware, which is why they default to off."""
+    return load().hx_set_features(int(mask))

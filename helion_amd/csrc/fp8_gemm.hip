@@ -818,6 +818,8 @@ __global__ __launch_bounds__(512) void hx_fp8_gemm_skinny_direct(const uint8_t* 
   one_group(std::false_type{});
 }
 
+#include "fp8_gemm_skinny_rm.h"
+
 // ------------------------------------------------------------------------------------------
 // general: 64x64 tile, 256 threads, 4x4 outputs per thread, fp32 FMAs on decoded e4m3.
 // ------------------------------------------------------------------------------------------
@@ -972,11 +974,51 @@ static bool gemm_path_rowmajor_ok(int64_t M, int64_t N, int64_t K, int64_t lda, 
          aligned(b, 16) && lda < (1LL << 27) && ldb_k < (1LL << 27) && M * lda < (1LL << 32) && K * ldb_k < (1LL << 32);
 }
 
+// Row-major B for a decode batch, streamed in place by hx_fp8_gemm_skinny_rm (opt-in: HX_FEATURE_SKINNY_ROWMAJOR).  The
+// shape part of the test is what the workspace query can evaluate; the call adds strides and alignment.
+static bool skinny_rm_shape_ok(int64_t M, int64_t N, int64_t K, int64_t ldb_k) {
+  return hx_feature(HX_FEATURE_SKINNY_ROWMAJOR) && M >= 1 && M <= 32 && K >= 1024 && K % 1024 == 0 && N % 16 == 0 && ldb_k % 16 == 0 &&
+         ldb_k >= N && 8 * ldb_k < (1LL << 32);
+}
+static bool skinny_rm_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, const void* a, const void* b) {
+  return skinny_rm_shape_ok(M, N, K, ldb_k) && lda % 8 == 0 && lda >= K && aligned(a, 8) && aligned(b, 16);
+}
+// k per workgroup (8192, 4096 or 1024: the kernel's instantiations) and the number of k splits: the largest piece with
+// which column groups x splits still come to half the chip's CUs, else the smallest piece
+static int skinny_rm_plan(int64_t N, int64_t K, int* kwg) {
+  const int64_t ngroups = (N + SKR_COLS - 1) / SKR_COLS;
+  for (int64_t k : {8192, 4096, 1024}) {
+    if (K % k != 0) continue;
+    *kwg = (int)k;
+    if (ngroups * (K / k) >= 128) break;
+  }
+  return (int)(K / *kwg);
+}
+
 extern "C" int hx_fp8_gemm_path(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
                                 const void* a, const void* b, const void* c) {
   if (ldb_k == 1) return gemm_path_kmajor(M, N, K, lda, ldb_n, ldc, a, b, c);
+  if (ldb_n == 1 && skinny_rm_ok(M, N, K, lda, ldb_k, a, b)) return 6;
   if (ldb_n == 1 && gemm_path_rowmajor_ok(M, N, K, lda, ldb_k, a, b)) return 4;
   return 0;
+}
+
+template <int OUT, int MB, int NSTEP, typename... Args>
+static void launch_skinny_rm_n(bool nt, dim3 grid, hipStream_t stream, Args... args) {
+  if (nt) hx_launch((hx_fp8_gemm_skinny_rm<OUT, MB, NSTEP, true>), grid, dim3(256), 0, stream, args...);
+  else hx_launch((hx_fp8_gemm_skinny_rm<OUT, MB, NSTEP, false>), grid, dim3(256), 0, stream, args...);
+}
+template <int OUT, typename... Args>
+static void launch_skinny_rm(int mb, int kwg, bool nt, dim3 grid, hipStream_t stream, Args... args) {
+  if (mb == 1) {
+    if (kwg == 8192) launch_skinny_rm_n<OUT, 1, 64>(nt, grid, stream, args...);
+    else if (kwg == 4096) launch_skinny_rm_n<OUT, 1, 32>(nt, grid, stream, args...);
+    else launch_skinny_rm_n<OUT, 1, 8>(nt, grid, stream, args...);
+  } else {
+    if (kwg == 8192) launch_skinny_rm_n<OUT, 2, 64>(nt, grid, stream, args...);
+    else if (kwg == 4096) launch_skinny_rm_n<OUT, 2, 32>(nt, grid, stream, args...);
+    else launch_skinny_rm_n<OUT, 2, 8>(nt, grid, stream, args...);
+  }
 }
 
 // b_read_once: non-temporal DMA for B
@@ -1096,7 +1138,30 @@ static int launch_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int
                            hipStream_t stream) {
   typedef typename OutT<OUT>::T out_t;
   int path = hx_fp8_gemm_path(M, N, K, lda, ldb_k, ldb_n, ldc, a, b, c);
-  if (path != 0) {
+  if (path == 6) {
+    int kwg = 1024;
+    const int splits = skinny_rm_plan(N, K, &kwg);
+    const int ngroups = (int)((N + SKR_COLS - 1) / SKR_COLS), cus = hx_cu_count();
+    const bool nt = N * K >= (192LL << 20);
+    const int mb = M <= 16 ? 1 : 2;
+    if (splits == 1) {
+      launch_skinny_rm<OUT>(mb, kwg, nt, dim3((unsigned)(ngroups < cus ? ngroups : cus), 1), stream, (const uint8_t*)a,
+                            (const uint8_t*)b, (out_t*)c, (int)M, (int)N, (long)lda, (long)ldb_k, (long)ldc, sa, sb, ngroups, 0L);
+    } else if (ws && aligned(ws, 16) && ws_bytes >= (size_t)splits * M * N * 4) {
+      // every split writes an unscaled fp32 slab; hx_fp8_gemm_split_reduce sums them in a fixed order, scales and casts
+      float* part = (float*)ws;
+      launch_skinny_rm<HX_F32>(mb, kwg, nt, dim3((unsigned)(ngroups < cus ? ngroups : cus), (unsigned)splits), stream,
+                               (const uint8_t*)a, (const uint8_t*)b, part, (int)M, (int)N, (long)lda, (long)ldb_k, (long)N,
+                               (const float*)nullptr, (const float*)nullptr, ngroups, (long)(M * N));
+      const long quads = (long)M * ((N + 3) / 4);
+      hx_launch((hx_fp8_gemm_split_reduce<OUT>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, (const float*)part,
+                (out_t*)c, (int)M, (int)N, (long)ldc, splits, sa, sb);
+    } else {
+      path = gemm_path_rowmajor_ok(M, N, K, lda, ldb_k, a, b) ? 4 : 0;  // no room for the partial sums: the paths without them
+    }
+  }
+  if (path == 6) {
+  } else if (path != 0) {
     launch_kmajor<OUT>(path, a, b, c, M, N, K, lda, path == 4 ? ldb_k : ldb_n, ldc, sa, sb, ws, ws_bytes, stream);
   } else {
     // row-major B with a workspace: transpose it once into K-contiguous form, then take a fast path
@@ -1134,6 +1199,11 @@ extern "C" size_t hx_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, i
     return M <= 16 && K <= 8192 && (N + 15) / 16 >= 12 * 256 ? 16 : 0;
   }
   if (ldb_n != 1 || K % 16 != 0) return 0;
+  if (skinny_rm_shape_ok(M, N, K, ldb_k)) {  // streamed in place: fp32 partial sums only when K is split over workgroups
+    int kwg = 1024;
+    const int splits = skinny_rm_plan(N, K, &kwg);
+    return splits > 1 ? (size_t)splits * M * N * 4 : 0;
+  }
   if (M > 16 && N % 16 == 0 && ldb_k % 16 == 0) return 0;
   return (size_t)(N * K);
 }

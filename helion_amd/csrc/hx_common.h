@@ -118,7 +118,8 @@ __device__ __forceinline__ float hx_e4m3_to_f32(uint8_t code) {
 }
 
 void hx_set_error(const char* fmt, ...);
-int hx_cu_count();  // compute units of the current device (looked up once per device, 256 if the query fails)
+int hx_cu_count();
+bool hx_feature(unsigned bit);  // is this opt-in kernel path (HX_FEATURE_* of the C header) switched on  // compute units of the current device (looked up once per device, 256 if the query fails)
 
 // Kernel launches go through hipLaunchKernel, whose own return code is the launch's status: the library never
 // reads (and so never clears) the caller's sticky HIP error state, and a foreign earlier error is never

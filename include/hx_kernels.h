@@ -40,6 +40,18 @@ enum {
 int hx_version(void);
 const char* hx_last_error(void);
 
+/* Opt-in kernel paths.  A path listed here has passed the CPU-side checks (the kernel source executed lane by lane
+ * on the host against the oracle, with every operand access bounds-checked) but has not yet been run on an MI355X, so
+ * it is compiled in and off by default: calls take the kernels that have.  hx_set_features replaces the process-wide
+ * mask (returns the previous one); its initial value is the environment variable HX_FEATURES (a number).  The
+ * hx_*_path and hx_*_workspace_bytes queries answer for the mask in force when they are called. */
+enum {
+  HX_FEATURE_SKINNY_ROWMAJOR = 1 /* hx_fp8_gemm, M <= 32, row-major b (ldb_n == 1), K % 1024 == 0, N % 16 == 0: b is
+                                    streamed in place (path 6) instead of being transposed through the workspace */
+};
+unsigned hx_set_features(unsigned mask);
+unsigned hx_get_features(void);
+
 /* Replaces the device side of `fp8_gemm(x, y)` (reference: examples/fp8_gemm.py:29-57, whose
  * generated launcher is test/test_examples.expected:821-841) and of its baseline
  * `torch._scaled_mm` call (examples/fp8_gemm.py:61-78).

@@ -91,6 +91,7 @@ inline float hx_e4m3_to_f32(uint8_t code) { return __builtin_amdgcn_cvt_f32_fp8(
 
 void hx_set_error(const char* fmt, ...);
 int hx_cu_count();
+bool hx_feature(unsigned bit);
 
 inline thread_local hipError_t hx_tls_launch_err = hipSuccess;
 template <typename... KArgs, typename... Args>

@@ -451,11 +451,11 @@ static void resolve(int wave_first, const std::vector<int>& g) {
         return;
       }
       const int kind = first.i0;
-      const bool f8 = kind == MFMA_F8_32x32x64 || kind == MFMA_F8_16x16x128;
+      const bool f8 = kind == MFMA_F8_32x32x64 || kind == MFMA_F8_16x16x128 || kind == MFMA_F8_16x16x32;
       const bool big = kind == MFMA_F8_32x32x64 || kind == MFMA_BF16_32x32x16 || kind == MFMA_F16_32x32x16;
       const bool bf = kind == MFMA_BF16_32x32x16 || kind == MFMA_BF16_16x16x32;
       const int MN = big ? 32 : 16;              // rows of A = columns of B
-      const int KL = f8 ? 32 : 8;                // k values one lane supplies
+      const int KL = f8 && kind != MFMA_F8_16x16x32 ? 32 : 8;  // k values one lane supplies
       const int K = KL * (64 / MN);
       static float A[32][128], B[32][128];
       for (int p = 0; p < 64; ++p) {
@@ -605,13 +605,16 @@ hipError_t run(dim3 grid, dim3 block, const std::function<void()>& fn, const voi
 }  // namespace hxsim
 
 const char* hipGetErrorString(hipError_t e) { return e == hipSuccess ? "no error" : hxsim::fault_msg.c_str(); }
+// The modelled chip has 256 CUs unless a test asks for fewer (1 .. 63), which makes the code paths that depend on the
+// ratio of work items to CUs (several column groups per workgroup, tickets, k splits) reachable at small sizes.  The
+// library caches the CU count per device id, so every setting is its own device id.
+static int sim_cus = 256;
 hipError_t hipGetDevice(int* dev) {
-  *dev = 0;
+  *dev = sim_cus % 64;
   return hipSuccess;
 }
 hipError_t hipDeviceGetAttribute(int* value, hipDeviceAttribute_t, int) {
-  const char* e = getenv("HX_SIM_CUS");
-  *value = e ? atoi(e) : 256;
+  *value = sim_cus;
   return hipSuccess;
 }
 
@@ -639,6 +642,11 @@ void hx_sim_config(int dma_lazy, int wave_order, int interleave) {
   if (dma_lazy >= 0) hxsim::cfg.dma_lazy = dma_lazy;
   if (wave_order >= 0) hxsim::cfg.wave_order = wave_order;
   if (interleave >= 0) hxsim::cfg.interleave = interleave;
+}
+int hx_sim_set_cus(int n) {
+  const int old = sim_cus;
+  if (n == 256 || (n >= 1 && n <= 63)) sim_cus = n;
+  return old;
 }
 const char* hx_sim_last_fault() { return hxsim::fault_msg.c_str(); }
 void hx_sim_reset() {

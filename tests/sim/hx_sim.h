@@ -90,7 +90,7 @@ int cvt_pk_fp8(float a, float b, int old, bool hi);
 float cvt_f32_fp8(int v, int sel);
 uint64_t clock100mhz();
 
-enum { MFMA_F8_32x32x64 = 0, MFMA_F8_16x16x128, MFMA_BF16_32x32x16, MFMA_F16_32x32x16, MFMA_BF16_16x16x32, MFMA_F16_16x16x32 };
+enum { MFMA_F8_32x32x64 = 0, MFMA_F8_16x16x128, MFMA_F8_16x16x32, MFMA_BF16_32x32x16, MFMA_F16_32x32x16, MFMA_BF16_16x16x32, MFMA_F16_16x16x32 };
 
 // runs `fn` once per work-item of the grid; returns hipSuccess or hipErrorLaunchFailure (message: hx_sim_last_fault)
 hipError_t run(dim3 grid, dim3 block, const std::function<void()>& fn, const void* kernel);
@@ -174,6 +174,7 @@ inline T shfl_xor(T v, int mask, int site) {
   hxsim::mfma_t<hxsim::MFMA_F8_32x32x64, hxs_v8i, hxs_v16f>((a), (b), (c), __LINE__)
 #define __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, cbsz, blgp, o0, s0, o1, s1) \
   hxsim::mfma_t<hxsim::MFMA_F8_16x16x128, hxs_v8i, hxs_v4f>((a), (b), (c), __LINE__)
+#define __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a, b, c, x, y, z) hxsim::mfma_t<hxsim::MFMA_F8_16x16x32, long, hxs_v4f>((long)(a), (long)(b), (c), __LINE__)
 #define __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, x, y, z) hxsim::mfma_t<hxsim::MFMA_BF16_32x32x16, hxs_v8bf, hxs_v16f>((a), (b), (c), __LINE__)
 #define __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, x, y, z) hxsim::mfma_t<hxsim::MFMA_F16_32x32x16, hxs_v8h, hxs_v16f>((a), (b), (c), __LINE__)
 #define __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, x, y, z) hxsim::mfma_t<hxsim::MFMA_BF16_16x16x32, hxs_v8bf, hxs_v4f>((a), (b), (c), __LINE__)

@@ -35,6 +35,7 @@ def load():
         lib.hx_sim_reset.restype, lib.hx_sim_reset.argtypes = None, []
         lib.hx_sim_counters.restype, lib.hx_sim_counters.argtypes = None, [_c.POINTER(_c.c_uint64)]
         lib.hx_sim_cvt_pk_fp8.restype, lib.hx_sim_cvt_pk_fp8.argtypes = _c.c_int, [_c.c_float, _c.c_float]
+        lib.hx_sim_set_cus.restype, lib.hx_sim_set_cus.argtypes = _c.c_int, [_c.c_int]
         lib.hx_sim_selftest.restype, lib.hx_sim_selftest.argtypes = _c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int]
         _lib = lib
     return _lib
@@ -103,3 +104,29 @@ def check(rc: int, what: str) -> None:
 
 def configure(variant: str) -> None:
     load().hx_sim_config(*VARIANTS[variant])
+
+
+class features:
+    """with simlib.features(mask): the opt-in kernel paths of the mask are on inside the block."""
+
+    def __init__(self, mask: int):
+        self.mask = mask
+
+    def __enter__(self):
+        self.old = load().hx_set_features(self.mask)
+
+    def __exit__(self, *exc):
+        load().hx_set_features(self.old)
+
+
+class cus:
+    """with simlib.cus(n): the modelled chip has n compute units (1 .. 63, or 256) inside the block."""
+
+    def __init__(self, n: int):
+        self.n = n
+
+    def __enter__(self):
+        self.old = load().hx_sim_set_cus(self.n)
+
+    def __exit__(self, *exc):
+        load().hx_sim_set_cus(self.old)

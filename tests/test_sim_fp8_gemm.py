@@ -106,3 +106,65 @@ def test_ticket_word_with_stale_contents():
     for stale in (0xFF, 0x00, 0x01, 0xA5):
         out = simops.fp8_gemm(a, y, None, None, torch.bfloat16, want_path=2, poison_ws=lambda nb: torch.full((nb,), stale, dtype=torch.uint8))
         assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), stale
+
+
+# ---- opt-in path 6: row-major B streamed in place for a decode batch (HX_FEATURE_SKINNY_ROWMAJOR) ---------------------
+@pytest.mark.parametrize("m,n,k,od", [
+    (16, 256, 1024, torch.bfloat16),
+    (1, 16, 1024, torch.float16),        # a single 16-byte chunk of columns
+    (7, 144, 2048, torch.bfloat16),      # ragged last column group (one valid chunk), two k splits
+    (16, 2048, 4096, torch.bfloat16),    # k split four ways (partial sums through the workspace)
+    (32, 384, 8192, torch.bfloat16),     # two 16-row blocks, 64 slices per wave
+    (20, 640, 1024, torch.float32),
+])
+def test_rowmajor_decode_kernel(m, n, k, od):
+    from helion_amd import _lib
+    g = torch.Generator().manual_seed(m + n + k)
+    a = (torch.randn(m, k, generator=g) * 0.5).to(E4)
+    y = (torch.randn(k, n, generator=g) * 0.5).to(E4)  # row-major [K, N]
+    ref = orc.fp8_gemm(a, y, 1.5, 0.5, od)
+    with simlib.features(_lib.HX_FEATURE_SKINNY_ROWMAJOR):
+        for variant in ("lazy-reverse", "eager-interleaved"):
+            simlib.configure(variant)
+            out = simops.fp8_gemm(a, y, torch.tensor(1.5), torch.tensor(0.5), od, want_path=6, end_flush=(variant != "eager-interleaved"))
+            assert rel_err(out, ref) <= 1e-2, variant
+    # and switched off (the default) the same call takes the old route
+    simlib.configure("lazy")
+    out = simops.fp8_gemm(a, y, torch.tensor(1.5), torch.tensor(0.5), od, want_path=0 if m <= 16 else 4)
+    assert rel_err(out, ref) <= 1e-2
+
+
+@pytest.mark.parametrize("variant", ALL)
+def test_rowmajor_decode_kernel_every_variant(variant):
+    from helion_amd import _lib
+    g = torch.Generator().manual_seed(8)
+    a = (torch.randn(16, 2048, generator=g) * 0.5).to(E4)
+    y = (torch.randn(2048, 1296, generator=g) * 0.5).to(E4)
+    simlib.configure(variant)
+    with simlib.features(_lib.HX_FEATURE_SKINNY_ROWMAJOR):
+        out = simops.fp8_gemm(a, y, None, None, torch.bfloat16, want_path=6)
+    assert rel_err(out, orc.fp8_gemm(a, y, 1.0, 1.0, torch.bfloat16)) <= 1e-2
+
+
+def test_rowmajor_decode_kernel_ring_runs_on_across_column_groups():
+    """More column groups than workgroups (a chip of 3 CUs in the model): a workgroup's ring carries the next group's first
+    slices while the current group is reduced, and the last group re-fetches its own."""
+    from helion_amd import _lib
+    g = torch.Generator().manual_seed(9)
+    a = (torch.randn(16, 1024, generator=g) * 0.5).to(E4)
+    y = (torch.randn(1024, 1168, generator=g) * 0.5).to(E4)  # 10 column groups, the last with one valid chunk
+    ref = orc.fp8_gemm(a, y, 1.0, 1.0, torch.bfloat16)
+    with simlib.features(_lib.HX_FEATURE_SKINNY_ROWMAJOR), simlib.cus(3):
+        for variant in ALL:
+            simlib.configure(variant)
+            out = simops.fp8_gemm(a, y, None, None, torch.bfloat16, want_path=6)
+            assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), variant
+
+
+def test_rowmajor_decode_needs_no_transpose_workspace_at_the_benchmark_shape():
+    from helion_amd import _lib
+    lib = simlib.load()
+    assert lib.hx_fp8_gemm_workspace_bytes(16, 28672, 8192, 28672, 1) == 28672 * 8192  # default: transposed copy
+    with simlib.features(_lib.HX_FEATURE_SKINNY_ROWMAJOR):
+        assert lib.hx_fp8_gemm_workspace_bytes(16, 28672, 8192, 28672, 1) == 0
+        assert lib.hx_fp8_gemm_path(16, 28672, 8192, 8192, 28672, 1, 28672, 1 << 20, 1 << 20, 1 << 20) == 6

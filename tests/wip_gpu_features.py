@@ -1,0 +1,38 @@
+"""GPU parity of the opt-in kernel paths (helion_amd.set_features).  NOT collected by pytest on purpose (the file name
+does not start with test_): these paths have passed the CPU-side checks in the host execution model but have never run on
+an MI355X.  Run it by naming the file:  python -m pytest tests/wip_gpu_features.py -x -q --timeout 120
+and rename it to test_gpu_features.py once it passes there."""
+import pytest
+import torch
+
+import helion_amd as hx
+from helion_amd import _lib
+from oracle import oracle as orc
+from tests._util import rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+E4 = torch.float8_e4m3fn
+
+
+@pytest.fixture
+def rowmajor_decode():
+    old = hx.set_features(hx.HX_FEATURE_SKINNY_ROWMAJOR)
+    yield
+    hx.set_features(old)
+
+
+@pytest.mark.parametrize("m,n,k,od", [(16, 256, 1024, torch.bfloat16), (1, 16, 1024, torch.float16), (7, 144, 2048, torch.bfloat16),
+                                      (16, 2048, 4096, torch.bfloat16), (32, 384, 8192, torch.bfloat16), (20, 640, 1024, torch.float32),
+                                      (16, 40000, 1024, torch.bfloat16), (16, 28672, 8192, torch.bfloat16)])
+def test_rowmajor_decode_kernel(rowmajor_decode, m, n, k, od):
+    g = torch.Generator().manual_seed(m + n + k)
+    a = (torch.randn(m, k, generator=g) * 0.5).to(E4)
+    y = (torch.randn(k, n, generator=g) * 0.5).to(E4)
+    sa, sb = torch.tensor(1.5), torch.tensor(0.5)
+    lib = _lib.load()
+    ad, yd = a.to(DEV), y.to(DEV)
+    assert lib.hx_fp8_gemm_path(m, n, k, k, n, 1, n, ad.data_ptr(), yd.data_ptr(), ad.data_ptr()) == 6
+    print(f"rowmajor decode case M={m} N={n} K={k} {od}", flush=True)
+    out = hx.fp8_gemm(ad, yd, scale_a=sa.to(DEV), scale_b=sb.to(DEV), out_dtype=od)
+    assert rel_err(out, orc.fp8_gemm(a, y, 1.5, 0.5, od)) <= 1e-2
