@@ -14,6 +14,7 @@
 #include "hx_common.h"
 
 #include <atomic>
+#include <chrono>
 #include <type_traits>
 
 // ------------------------------------------------------------------------------------------
@@ -652,6 +653,11 @@ __global__ __launch_bounds__(512) void hx_fp8_gemm_skinny(const uint8_t* __restr
 // Workgroup 0, which the hardware dispatches first, installs {tag, 0} before anything else; a draw that finds another
 // tag was made before that store landed, waits for the tag and draws again (workgroup 0 waits for nobody, so the wait
 // ends).  The last draw of the launch clears the word, so the replay of a captured launch finds no stale tag.
+// The wait is bounded (a few milliseconds): a workgroup whose tag never comes back - two launches sharing one word at the
+// same time, a misuse - stops drawing and stores {1 << 63 | tag} into the word after the ticket word; the launch then ends
+// normally with the column groups that workgroup would have drawn not computed.  The library only ever sets that second
+// word: a caller who wants to know zeroes it beforehand and looks at it afterwards.
+#define SKD_MAX_SPINS (1 << 12)
 __device__ __forceinline__ unsigned long long skd_draw_issue(unsigned long long* word) {
   // the zero offset is opaque to the compiler on purpose: for an address it can prove uniform it turns the add into a
   // wave-wide reduction and reads the answer back on the spot, and the answer is to be awaited where it is used
@@ -661,11 +667,12 @@ __device__ __forceinline__ unsigned long long skd_draw_issue(unsigned long long*
 }
 __device__ __forceinline__ int skd_draw_result(unsigned long long* word, unsigned long long old, unsigned long long tag, int nwork,
                                                int total) {
-  // (the wait is bounded all the same: if two launches are given the same word at the same time - a misuse - a tag may
-  // never come back, and a workgroup that gives up and stops costs that misuse wrong results, not a hung GPU)
   for (int spins = 0; (old >> 24) != tag; ) {
     while ((__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 24) != tag) {
-      if (++spins > (1 << 18)) return -1;
+      if (++spins > SKD_MAX_SPINS) {
+        __hip_atomic_store(word + 1, (1ull << 63) | tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return -1;
+      }
       __builtin_amdgcn_s_sleep(32);
     }
     old = skd_draw_issue(word);
@@ -1029,6 +1036,20 @@ static void launch_tileN128(bool b_read_once, dim3 grid, hipStream_t stream, Arg
 }
 
 static std::atomic<unsigned long long> g_skd_launches{0};
+// The ticket tag of a decode launch: a counter scrambled together with a per-process value, so that whatever an
+// uninitialised (or recycled) workspace word holds matches a launch's tag with probability 2^-40 instead of "whenever it
+// holds a small integer"; never zero.
+static unsigned long long skd_next_tag() {
+  static const unsigned long long salt = [] {
+    unsigned long long x = (unsigned long long)(uintptr_t)&g_skd_launches ^ (unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count();
+    return x * 0x9E3779B97F4A7C15ull;
+  }();
+  unsigned long long z = (g_skd_launches.fetch_add(1, std::memory_order_relaxed) + 1) * 0x9E3779B97F4A7C15ull + salt;  // splitmix64
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  z = (z ^ (z >> 31)) & ((1ull << 40) - 1);
+  return z ? z : 1;
+}
 
 template <int OUT, int MB, typename... Args>
 static void launch_skinny_direct(int ns, int grid, hipStream_t stream, Args... args) {
@@ -1042,7 +1063,7 @@ static void launch_skinny_direct(int ns, int grid, hipStream_t stream, Args... a
     default:
       hx_launch((hx_fp8_gemm_skinny_direct<OUT, 0, MB>), dim3(grid), dim3(512), 0, stream, args...);
   }
-}  // makes the ticket tag of every decode launch different
+}
 
 template <int OUT>
 static void launch_kmajor(int path, const void* a, const void* bt, void* c, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
@@ -1114,9 +1135,9 @@ static void launch_kmajor(int path, const void* a, const void* bt, void* c, int6
     // (worth it from about 12 groups per workgroup: a ticket is a whole group, 4 us of work, and the spread between the
     // XCDs is 8-10 %; at 7 groups per workgroup tickets measured 0.9 us slower to 0.3 us faster than strided shares, at
     // 14 groups 3 % faster)
-    if (ws && ws_bytes >= 8 && aligned(ws, 8) && ncg >= 12 * grid && ncg < (1 << 24)) {
-      tickets = (unsigned long long*)ws;
-      tag = (g_skd_launches.fetch_add(1, std::memory_order_relaxed) % ((1ull << 40) - 1)) + 1;  // 1 .. 2^40 - 1
+    if (ws && ws_bytes >= 16 && aligned(ws, 8) && ncg >= 12 * grid && ncg < (1 << 24)) {
+      tickets = (unsigned long long*)ws;  // word 0: {tag, count}; word 1: the give-up record
+      tag = skd_next_tag();
     }
     if (K <= 8192) {
       const int ns = K % 1024 == 0 ? (int)(K / 1024) : 0;

@@ -62,12 +62,22 @@ unsigned hx_get_features(void);
  * c: [M,N] of out_dtype (HX_F16 = reference default, HX_BF16, HX_F32), element (m,n) at c[m*ldc+n].
  * scale_a/scale_b: device pointers to one fp32 each, or NULL for 1.0 (the reference hard-codes
  *    1.0, helion/language/matmul_ops.py:232-233).
+ * hx_fp8_gemm_path: 0 plain kernel (or a row-major b transposed through the workspace), 1 256x256 tiles, 2 decode kernel,
+ * 3 256x256 tiles with guarded edges / K tail, 4 256x256 tiles on a row-major b, 5 128-column tiles, 6 decode kernel on a
+ * row-major b (opt-in).
  * Chooses between the 256x256 MFMA tile kernel (with guarded edge tiles when M or N is ragged or K is not a multiple
  * of 128 — K % 16 == 0 suffices, the last k-tile is zero-padded in LDS; it reads a column-major B directly and a
  * row-major B through transposing LDS loads), the skinny (M<=16, or M<=32 with K<=8192) wave-split-K kernel
  * and a bounds-checked general kernel from the shape, strides and alignment.
  * workspace: optional device scratch of hx_fp8_gemm_workspace_bytes(...) bytes, 16-byte aligned, any content; it
- *    belongs to the call until its kernels have finished (two launches in flight at once need two workspaces). */
+ *    belongs to the call until its kernels have finished (two launches in flight at once need two workspaces).
+ *    A decode call (path 2) with at least 12 column groups of 16 per CU hands its last groups out by ticket through the
+ *    first 8 bytes (any content before, zero after).  Sharing that word between two launches in flight is the misuse
+ *    above: a workgroup then waits a few milliseconds at most for its launch's tag, stops drawing, and stores a value with
+ *    bit 63 set into bytes 8..15.  The library only ever sets those bytes; a caller who wants the record zeroes them
+ *    before the call and reads them after it.
+ *    With HX_FEATURE_SKINNY_ROWMAJOR on, a row-major b for M <= 32 with K % 1024 == 0 and N % 16 == 0 is streamed in
+ *    place (path 6) and needs scratch only for fp32 partial sums when few column groups meet a long K. */
 int hx_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int64_t lda,
                 int64_t ldb_k, int64_t ldb_n, int64_t ldc, const float* scale_a, const float* scale_b,
                 int out_dtype, void* workspace, size_t workspace_bytes, void* stream);

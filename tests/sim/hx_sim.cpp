@@ -71,6 +71,7 @@ struct Config {
   int dma_lazy = 0;    // 0: a DMA lands when it is issued; 1: when the wave's vmcnt wait (or its end) forces it
   int wave_order = 0;  // 0: waves 0, 1, 2 ..; 1: the other way round
   int interleave = 0;  // 0: a wave runs until it blocks at a barrier; 1: the waves take turns after every cross-lane instruction
+  int wg_reverse = 0;  // 1: the workgroups of a launch run last to first (workgroup 0 is NOT the first to start)
   int poison_lds = 1;  // fill the LDS with 0xFF (NaN in e4m3, bf16, f16 and f32) before every workgroup
 };
 
@@ -592,12 +593,12 @@ hipError_t run(dim3 grid, dim3 block, const std::function<void()>& fn, const voi
   launch_fn = kernel;
   geo.block_dim = {block.x, block.y, block.z};
   geo.grid_dim = {grid.x, grid.y, grid.z};
-  for (unsigned z = 0; z < grid.z && !faulted; ++z)
-    for (unsigned y = 0; y < grid.y && !faulted; ++y)
-      for (unsigned x = 0; x < grid.x && !faulted; ++x) {
-        geo.block_idx = {x, y, z};
-        run_workgroup(block);
-      }
+  const unsigned long total = (unsigned long)grid.x * grid.y * grid.z;
+  for (unsigned long i = 0; i < total && !faulted; ++i) {
+    const unsigned long id = cfg.wg_reverse ? total - 1 - i : i;
+    geo.block_idx = {(unsigned)(id % grid.x), (unsigned)((id / grid.x) % grid.y), (unsigned)(id / ((unsigned long)grid.x * grid.y))};
+    run_workgroup(block);
+  }
   body = nullptr;
   return faulted ? hipErrorLaunchFailure : hipSuccess;
 }
@@ -642,6 +643,11 @@ void hx_sim_config(int dma_lazy, int wave_order, int interleave) {
   if (dma_lazy >= 0) hxsim::cfg.dma_lazy = dma_lazy;
   if (wave_order >= 0) hxsim::cfg.wave_order = wave_order;
   if (interleave >= 0) hxsim::cfg.interleave = interleave;
+}
+int hx_sim_set_wg_reverse(int on) {
+  const int old = hxsim::cfg.wg_reverse;
+  hxsim::cfg.wg_reverse = on != 0;
+  return old;
 }
 int hx_sim_set_cus(int n) {
   const int old = sim_cus;

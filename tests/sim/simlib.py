@@ -35,6 +35,7 @@ def load():
         lib.hx_sim_reset.restype, lib.hx_sim_reset.argtypes = None, []
         lib.hx_sim_counters.restype, lib.hx_sim_counters.argtypes = None, [_c.POINTER(_c.c_uint64)]
         lib.hx_sim_cvt_pk_fp8.restype, lib.hx_sim_cvt_pk_fp8.argtypes = _c.c_int, [_c.c_float, _c.c_float]
+        lib.hx_sim_set_wg_reverse.restype, lib.hx_sim_set_wg_reverse.argtypes = _c.c_int, [_c.c_int]
         lib.hx_sim_set_cus.restype, lib.hx_sim_set_cus.argtypes = _c.c_int, [_c.c_int]
         lib.hx_sim_selftest.restype, lib.hx_sim_selftest.argtypes = _c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int]
         _lib = lib
@@ -130,3 +131,14 @@ class cus:
 
     def __exit__(self, *exc):
         load().hx_sim_set_cus(self.old)
+
+
+class workgroups_last_to_first:
+    """with simlib.workgroups_last_to_first(): the workgroups of a launch run in reverse order, each to completion, so
+    workgroup 0 is the last to start (a workgroup that waits for something workgroup 0 does can only give up)."""
+
+    def __enter__(self):
+        self.old = load().hx_sim_set_wg_reverse(1)
+
+    def __exit__(self, *exc):
+        load().hx_sim_set_wg_reverse(self.old)

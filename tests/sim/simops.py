@@ -17,7 +17,8 @@ def _p(t):
     return t.data_ptr() if t is not None else None
 
 
-def fp8_gemm(x, y, scale_a=None, scale_b=None, out_dtype=torch.bfloat16, end_flush=True, want_path=None, lda=None, poison_ws=None):
+def fp8_gemm(x, y, scale_a=None, scale_b=None, out_dtype=torch.bfloat16, end_flush=True, want_path=None, lda=None, poison_ws=None,
+             ws_after=None, ws_bytes=None):
     """x [M,K] e4m3 (row-major), y [K,N] e4m3 with any of the two layouts the op passes on (strides kept)."""
     lib = simlib.load()
     m, k = x.shape
@@ -41,13 +42,15 @@ def fp8_gemm(x, y, scale_a=None, scale_b=None, out_dtype=torch.bfloat16, end_flu
         if want_path is not None:
             got = lib.hx_fp8_gemm_path(m, n, k, lda, ldb_k, ldb_n, n, X.data_ptr(), Y.data_ptr(), C.data_ptr())
             assert got == want_path, f"fp8_gemm path {got}, expected {want_path}"
-        wsb = lib.hx_fp8_gemm_workspace_bytes(m, n, k, ldb_k, ldb_n)
+        wsb = lib.hx_fp8_gemm_workspace_bytes(m, n, k, ldb_k, ldb_n) if ws_bytes is None else ws_bytes
         ws = ar.empty(wsb) if wsb else None
         if ws is not None and poison_ws is not None:
             ws.copy_(poison_ws(wsb))
         rc = lib.hx_fp8_gemm(X.data_ptr(), Y.data_ptr(), C.data_ptr(), m, n, k, lda, ldb_k, ldb_n, n, _p(sa), _p(sb), _DT[out_dtype],
                              _p(ws), wsb, None)
         simlib.check(rc, "hx_fp8_gemm")
+        if ws_after is not None and ws is not None:
+            ws_after.append(ws.clone())
         return C.clone()
 
 

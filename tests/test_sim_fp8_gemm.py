@@ -108,6 +108,29 @@ def test_ticket_word_with_stale_contents():
         assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), stale
 
 
+def test_ticket_wait_gives_up_and_says_so():
+    """A workgroup that draws a ticket before workgroup 0 has installed the launch's tag waits for the tag - for a bounded
+    time.  With the workgroups run last to first, each to completion, the tag can never arrive: every workgroup but 0 must
+    stop waiting, leave the give-up record in the second workspace word and end normally."""
+    a, y = _ops(16, 4096, 1024, 5, False)
+    ref = orc.fp8_gemm(a, y, 1.0, 1.0, torch.bfloat16)
+    simlib.configure("lazy")
+    zero = lambda nb: torch.zeros(nb, dtype=torch.uint8)  # (only the give-up record needs it: the ticket word itself may hold anything)
+    with simlib.cus(8):
+        after = []
+        out = simops.fp8_gemm(a, y, None, None, torch.bfloat16, want_path=2, ws_after=after, ws_bytes=16, poison_ws=zero)   # in order: nothing to wait for
+        assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+        words = after[0].view(torch.int64)
+        assert int(words[0]) == 0 and int(words[1]) == 0     # ticket word cleared by the last draw, no give-up recorded
+        with simlib.workgroups_last_to_first():
+            after = []
+            out = simops.fp8_gemm(a, y, None, None, torch.bfloat16, want_path=2, ws_after=after, ws_bytes=16, poison_ws=zero)  # completes: no hang, no fault
+        words = after[0].view(torch.int64)
+        assert int(words[1]) < 0                             # bit 63 set: somebody gave up
+        # (here the result is complete all the same: workgroup 0, started last, draws every ticket the others left)
+        assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+
+
 # ---- opt-in path 6: row-major B streamed in place for a decode batch (HX_FEATURE_SKINNY_ROWMAJOR) ---------------------
 @pytest.mark.parametrize("m,n,k,od", [
     (16, 256, 1024, torch.bfloat16),
