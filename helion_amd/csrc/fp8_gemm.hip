@@ -313,8 +313,10 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256(const uint8_t* __rest
 // byte transpose: src[K][N] (row stride lds_, N contiguous) -> dst[N][K] contiguous.  Turns a row-major B into
 // the K-contiguous layout the MFMA kernels read; 64x64 tiles through LDS.
 // ------------------------------------------------------------------------------------------
+// dst_ld >= K: row stride of dst; its bytes K .. dst_ld-1 are written as zeros (a K that is padded up to the next multiple
+// of 16 for the MFMA kernels).
 __global__ __launch_bounds__(256) void hx_transpose_u8(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, int K, int N,
-                                                      long src_ld) {
+                                                      long src_ld, int dst_ld) {
   __shared__ uint8_t t[64][64 + 4];
   const int k0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
@@ -325,8 +327,23 @@ __global__ __launch_bounds__(256) void hx_transpose_u8(const uint8_t* __restrict
   __syncthreads();
   for (int r = ty; r < 64; r += 4) {
     const int n = n0 + r, k = k0 + tx;
-    if (n < N && k < K) dst[(long)n * K + k] = t[tx][r];
+    if (n < N && k < dst_ld) dst[(long)n * dst_ld + k] = t[tx][r];  // k >= K: the tile holds zeros there
   }
+}
+
+// rows of K bytes (row stride src_ld, any alignment) -> rows of K16 = dst_ld bytes, zero-padded; 16 bytes per work-item
+__global__ __launch_bounds__(256) void hx_pad_rows_u8(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, int rows, int K,
+                                                     long src_ld, int dst_ld) {
+  const int cpr = dst_ld >> 4;
+  const long id = (long)blockIdx.x * 256 + threadIdx.x;
+  if (id >= (long)rows * cpr) return;
+  const int row = (int)(id / cpr), k0 = (int)(id % cpr) * 16;
+  const uint8_t* s = src + (long)row * src_ld;
+  uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+  for (int b = 0; b < 16; ++b)
+    if (k0 + b < K) w[b >> 2] |= (uint32_t)s[k0 + b] << (8 * (b & 3));
+  *(v4i*)(dst + (long)row * dst_ld + k0) = (v4i){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
 }
 
 // ------------------------------------------------------------------------------------------
@@ -981,6 +998,37 @@ static bool gemm_path_rowmajor_ok(int64_t M, int64_t N, int64_t K, int64_t lda, 
          aligned(b, 16) && lda < (1LL << 27) && ldb_k < (1LL << 27) && M * lda < (1LL << 32) && K * ldb_k < (1LL << 32);
 }
 
+// Any K / any alignment through the MFMA kernels (opt-in: HX_FEATURE_FP8_GEMM_ANY_K): which operands are copied into the
+// workspace as zero-padded K-contiguous rows, where, and the kernel path the copies then take.
+struct Repack {
+  bool copy_a;
+  int copy_b;  // 0 no, 1 pad rows of a K-contiguous B, 2 transpose a row-major B
+  int64_t K16;
+  size_t b_off, bytes;
+  int path;
+};
+static size_t repack_bytes(int64_t M, int64_t N, int64_t K16, bool copy_a, bool copy_b, size_t* b_off) {
+  size_t ab = copy_a ? (((size_t)(M * K16) + 255) & ~(size_t)255) : 0;
+  *b_off = ab;
+  return ab + (copy_b ? (size_t)(N * K16) : 0);
+}
+static bool repack_plan(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc, const void* a,
+                        const void* b, const void* c, void* ws, size_t ws_bytes, Repack* rp) {
+  if (!hx_feature(HX_FEATURE_FP8_GEMM_ANY_K) || !ws || !aligned(ws, 16) || K < 1) return false;
+  rp->K16 = (K + 15) & ~(int64_t)15;
+  rp->copy_a = !(K % 16 == 0 && lda % 16 == 0 && aligned(a, 16));
+  if (ldb_k == 1) rp->copy_b = (K % 16 == 0 && ldb_n % 16 == 0 && aligned(b, 16)) ? 0 : 1;
+  else if (ldb_n == 1 && ldb_k >= N) rp->copy_b = 2;
+  else return false;  // B strided in both dimensions: the plain kernel
+  if (!rp->copy_a && !rp->copy_b) return false;
+  rp->bytes = repack_bytes(M, N, rp->K16, rp->copy_a, rp->copy_b != 0, &rp->b_off);
+  if (ws_bytes < rp->bytes) return false;
+  const void* a2 = rp->copy_a ? (const void*)ws : a;
+  const void* b2 = rp->copy_b ? (const void*)((const uint8_t*)ws + rp->b_off) : b;
+  rp->path = gemm_path_kmajor(M, N, rp->K16, rp->copy_a ? rp->K16 : lda, rp->copy_b ? rp->K16 : ldb_n, ldc, a2, b2, c);
+  return rp->path != 0;
+}
+
 // Row-major B for a decode batch, streamed in place by hx_fp8_gemm_skinny_rm (opt-in: HX_FEATURE_SKINNY_ROWMAJOR).  The
 // shape part of the test is what the workspace query can evaluate; the call adds strides and alignment.
 static bool skinny_rm_shape_ok(int64_t M, int64_t N, int64_t K, int64_t ldb_k) {
@@ -1187,12 +1235,29 @@ static int launch_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int
   } else {
     // row-major B with a workspace: transpose it once into K-contiguous form, then take a fast path
     int tpath = 0;
+    Repack rp;
     if (ldb_n == 1 && ldb_k >= N && ws && ws_bytes >= (size_t)(N * K) && aligned(ws, 16))
       tpath = gemm_path_kmajor(M, N, K, lda, K, ldc, a, ws, c);
     if (tpath != 0) {
       dim3 tg((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64));
-      hx_launch(hx_transpose_u8, tg, dim3(256), 0, stream, (const uint8_t*)b, (uint8_t*)ws, (int)K, (int)N, (long)ldb_k);
+      hx_launch(hx_transpose_u8, tg, dim3(256), 0, stream, (const uint8_t*)b, (uint8_t*)ws, (int)K, (int)N, (long)ldb_k, (int)K);
       launch_kmajor<OUT>(tpath, a, ws, c, M, N, K, lda, K, ldc, sa, sb, nullptr, 0, stream);
+    } else if (repack_plan(M, N, K, lda, ldb_k, ldb_n, ldc, a, b, c, ws, ws_bytes, &rp)) {
+      // Any K, any alignment (opt-in): A and / or B are copied once into the workspace as K-contiguous rows padded with
+      // zeros to K16 = the next multiple of 16 - zeros add nothing to a dot product - and the MFMA kernels run on the copies.
+      uint8_t* wa = (uint8_t*)ws;
+      uint8_t* wb = (uint8_t*)ws + rp.b_off;
+      if (rp.copy_a)
+        hx_launch(hx_pad_rows_u8, dim3((unsigned)((M * (rp.K16 / 16) + 255) / 256)), dim3(256), 0, stream, (const uint8_t*)a, wa, (int)M,
+                  (int)K, (long)lda, (int)rp.K16);
+      if (rp.copy_b == 1)
+        hx_launch(hx_pad_rows_u8, dim3((unsigned)((N * (rp.K16 / 16) + 255) / 256)), dim3(256), 0, stream, (const uint8_t*)b, wb, (int)N,
+                  (int)K, (long)ldb_n, (int)rp.K16);
+      else if (rp.copy_b == 2)
+        hx_launch(hx_transpose_u8, dim3((unsigned)((N + 63) / 64), (unsigned)((rp.K16 + 63) / 64)), dim3(256), 0, stream, (const uint8_t*)b,
+                  wb, (int)K, (int)N, (long)ldb_k, (int)rp.K16);
+      launch_kmajor<OUT>(rp.path, rp.copy_a ? (const void*)wa : a, rp.copy_b ? (const void*)wb : b, c, M, N, rp.K16,
+                         rp.copy_a ? rp.K16 : lda, rp.copy_b ? rp.K16 : ldb_n, ldc, sa, sb, nullptr, 0, stream);
     } else {
       dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
       hx_launch(hx_fp8_gemm_general<OUT>, grid, dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)b, (out_t*)c,
@@ -1212,6 +1277,10 @@ extern "C" size_t hx_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, i
   // contiguous; N or the row stride not a multiple of 16) but that could take a fast path after a transpose needs
   // N*K bytes of scratch; a column-major B needs scratch only for split-K partial sums.
   if (M <= 0 || N <= 0 || K <= 0) return 0;
+  if (hx_feature(HX_FEATURE_FP8_GEMM_ANY_K) && K % 16 != 0 && (ldb_k == 1 || ldb_n == 1)) {  // both operands repacked, K padded
+    size_t off;
+    return repack_bytes(M, N, (K + 15) & ~(int64_t)15, true, true, &off);
+  }
   if (ldb_k == 1) {  // column-major B: fp32 partial sums when the 128-column tile kernel would split K
     int ktps = 0;
     const int splits = tileN128_splits(M, N, K, &ktps);

@@ -191,3 +191,51 @@ def test_rowmajor_decode_needs_no_transpose_workspace_at_the_benchmark_shape():
     with simlib.features(_lib.HX_FEATURE_SKINNY_ROWMAJOR):
         assert lib.hx_fp8_gemm_workspace_bytes(16, 28672, 8192, 28672, 1) == 0
         assert lib.hx_fp8_gemm_path(16, 28672, 8192, 8192, 28672, 1, 28672, 1 << 20, 1 << 20, 1 << 20) == 6
+
+
+# ---- opt-in: any K through the MFMA kernels (HX_FEATURE_FP8_GEMM_ANY_K) --------------------------------------------------
+@pytest.mark.parametrize("m,n,k,rowmajor", [
+    (300, 260, 1000, False),   # K % 16 = 8: both operands padded, guarded-edge tile kernel
+    (33, 100, 1001, False),    # odd K: byte-aligned rows
+    (16, 512, 2047, False),    # a decode batch: K padded to 2048, the skinny kernel
+    (64, 1792, 1023, False),   # 64-row decode tile
+    (200, 272, 100, True),     # row-major B: transposed and padded in one pass
+    (5, 7, 24, False),         # K % 16 = 8, tiny
+    (256, 256, 3, True),       # K below one chunk
+])
+def test_any_k_through_the_mfma_kernels(m, n, k, rowmajor):
+    import ctypes
+    from helion_amd import _lib
+    a, y = _ops(m, n, k, 77 + k, rowmajor)
+    ref = orc.fp8_gemm(a, y, 1.5, 0.75, torch.bfloat16)
+    lib, c = simlib.load(), (ctypes.c_uint64 * 4)()
+    for variant in FAST:
+        simlib.configure(variant)
+        lib.hx_sim_counters(c)
+        before = c[0]
+        with simlib.features(_lib.HX_FEATURE_FP8_GEMM_ANY_K):
+            out = simops.fp8_gemm(a, y, torch.tensor(1.5), torch.tensor(0.75), torch.bfloat16, want_path=0)
+        lib.hx_sim_counters(c)
+        assert c[0] > before, "the plain kernel ran (it has no cross-lane instructions): the repacked route was not taken"
+        assert rel_err(out, ref) <= 1e-2, variant
+
+
+def test_any_k_route_really_runs_matrix_instructions():
+    """The repacked call must multiply with MFMAs (the model counts cross-lane instructions; the plain kernel has none)."""
+    import ctypes
+    from helion_amd import _lib
+    lib = simlib.load()
+    a, y = _ops(64, 128, 1000, 3, False)
+    simlib.configure("lazy")
+
+    def cross_lane_instructions(mask):
+        c = (ctypes.c_uint64 * 4)()
+        lib.hx_sim_counters(c)
+        before = c[0]
+        with simlib.features(mask):
+            simops.fp8_gemm(a, y, None, None, torch.bfloat16)
+        lib.hx_sim_counters(c)
+        return c[0] - before
+
+    assert cross_lane_instructions(0) == 0
+    assert cross_lane_instructions(_lib.HX_FEATURE_FP8_GEMM_ANY_K) > 100

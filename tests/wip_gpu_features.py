@@ -36,3 +36,22 @@ def test_rowmajor_decode_kernel(rowmajor_decode, m, n, k, od):
     print(f"rowmajor decode case M={m} N={n} K={k} {od}", flush=True)
     out = hx.fp8_gemm(ad, yd, scale_a=sa.to(DEV), scale_b=sb.to(DEV), out_dtype=od)
     assert rel_err(out, orc.fp8_gemm(a, y, 1.5, 0.5, od)) <= 1e-2
+
+
+@pytest.fixture
+def any_k():
+    old = hx.set_features(hx.HX_FEATURE_FP8_GEMM_ANY_K)
+    yield
+    hx.set_features(old)
+
+
+@pytest.mark.parametrize("m,n,k,rowmajor", [(300, 260, 1000, False), (33, 100, 1001, False), (16, 512, 2047, False), (64, 1792, 1023, False),
+                                            (200, 272, 100, True), (5, 7, 24, False), (256, 256, 3, True), (2048, 2048, 4100, False)])
+def test_any_k_through_the_mfma_kernels(any_k, m, n, k, rowmajor):
+    g = torch.Generator().manual_seed(77 + k)
+    a = (torch.randn(m, k, generator=g) * 0.5).to(E4)
+    bt = (torch.randn(n, k, generator=g) * 0.5).to(E4)
+    y = bt.t().contiguous() if rowmajor else bt.t()
+    print(f"any-K case M={m} N={n} K={k} rowmajor={rowmajor}", flush=True)
+    out = hx.fp8_gemm(a.to(DEV), y.to(DEV), out_dtype=torch.bfloat16)
+    assert rel_err(out, orc.fp8_gemm(a, y, 1.0, 1.0, torch.bfloat16)) <= 1e-2
