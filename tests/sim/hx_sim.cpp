@@ -49,6 +49,7 @@ struct Dma {
   const uint8_t* src;
   uint8_t* dst;
   int bytes;
+  bool idem;  // re-fetch of what the destination already holds (see C_DMA)
 };
 
 struct Lane {
@@ -86,6 +87,7 @@ static uint8_t* stacks;
 static const size_t STACK = 512 << 10;
 static const int MAX_LANES = 1024;
 static bool faulted;
+static bool sched_ctx;  // `cur` names a lane only for attribution: the code runs on the scheduler's own stack
 static std::string fault_msg;
 static const void* launch_fn;
 static std::string kernel_name() {
@@ -128,7 +130,7 @@ static void fail(const char* fmt, ...) {
     fault_msg = std::string(msg) + where;
     faulted = true;
   }
-  if (cur) {
+  if (cur && !sched_ctx) {
     void* dummy;
     hx_sim_switch(&dummy, sched_sp);  // this work-item never runs again
   }
@@ -196,10 +198,91 @@ static void collective(int kind, int site) {
   yield_to_scheduler();
 }
 
+// ---- LDS access discipline -----------------------------------------------------------------------------------------
+// The kernel objects are compiled with load / store tracing (the compiler calls __sanitizer_cov_load*/store* with the
+// address of every memory access), so the model sees every LDS access, not only the DMA and the transposing reads it
+// executes itself, and can check the one rule the hardware gives: two accesses to the same LDS bytes from different
+// waves, at least one of them a write, are ordered only by a workgroup barrier between them; and a DMA transfer writes
+// its bytes at some unknown moment between its issue and the wave's vmcnt wait that covers it.  Per 4-byte word of the
+// LDS the model keeps the last writer (wave, barrier epoch), the readers of the current epoch and whether a DMA into it is
+// in flight; an access that is not ordered against those by a barrier (or, within one wave, by program order) is
+// reported with the kernel, the workgroup, both waves and the LDS offset.  Lanes of one wave execute together and are
+// never checked against each other.
+struct Shadow {
+  uint32_t wepoch, repoch;  // epoch of the last write / of the reads in rmask; 0 = never
+  uint16_t rmask;           // waves that read it in epoch repoch
+  uint8_t wwave;            // wave of the last write
+  uint8_t inflight;         // 1 + wave of the DMA in flight into it, 0 = none
+};
+static Shadow* shadow;           // one entry per 4 bytes of the LDS section
+static uint32_t epoch = 1;       // barrier epoch of the running workgroup
+static bool check_lds = true;
+static size_t dirty_lo = ~(size_t)0, dirty_hi = 0;  // LDS bytes written by the running workgroup (what to poison again)
+static uint64_t n_lds_checked;
+
+static void lds_race(const char* what, size_t off, int w, const Shadow& s) {
+  fail("LDS race: %s at LDS offset %zu by wave %d in barrier epoch %u (last write: wave %d epoch %u; readers of epoch %u: mask 0x%x; DMA in "
+       "flight from wave %d)",
+       what, off, w, epoch, (int)s.wwave, s.wepoch, s.repoch, (unsigned)s.rmask, (int)s.inflight - 1);
+}
+enum { ACC_READ, ACC_WRITE, ACC_DMA_ISSUE, ACC_DMA_LAND };
+static void lds_access(const void* p, size_t n, int kind) {
+  const size_t off = (const char*)p - __start_hx_lds;
+  if (kind != ACC_READ) {
+    if (off < dirty_lo) dirty_lo = off;
+    if (off + n > dirty_hi) dirty_hi = off + n;
+  }
+  if (!check_lds || !cur) return;
+  const int w = cur->tid >> 6;
+  ++n_lds_checked;
+  for (size_t i = off >> 2; i <= (off + n - 1) >> 2; ++i) {
+    Shadow& s = shadow[i];
+    const bool other_writer = s.wepoch == epoch && s.wwave != w;
+    const bool other_reader = s.repoch == epoch && (s.rmask & ~(1u << w)) != 0;
+    switch (kind) {
+      case ACC_READ:
+        if (s.inflight) return lds_race(s.inflight - 1 == w ? "read of bytes whose DMA has not been waited for" : "read of bytes another wave's DMA is still writing", i * 4, w, s);
+        if (other_writer) return lds_race("read of bytes another wave wrote since the last barrier", i * 4, w, s);
+        if (s.repoch != epoch) s.repoch = epoch, s.rmask = 0;
+        s.rmask |= (uint16_t)(1u << w);
+        break;
+      case ACC_WRITE:
+        if (s.inflight) return lds_race("write to bytes a DMA is still writing", i * 4, w, s);
+        if (other_writer) return lds_race("write to bytes another wave wrote since the last barrier", i * 4, w, s);
+        if (other_reader) return lds_race("write to bytes another wave read since the last barrier", i * 4, w, s);
+        s.wepoch = epoch, s.wwave = (uint8_t)w;
+        break;
+      case ACC_DMA_ISSUE:
+        if (s.inflight) return lds_race("DMA into bytes another DMA is still writing", i * 4, w, s);
+        if (other_writer) return lds_race("DMA into bytes another wave wrote since the last barrier", i * 4, w, s);
+        if (other_reader) return lds_race("DMA into bytes another wave read since the last barrier", i * 4, w, s);
+        s.inflight = (uint8_t)(w + 1);
+        break;
+      case ACC_DMA_LAND:
+        s.inflight = 0;
+        if (other_reader) return lds_race("DMA waited for in the epoch in which another wave already read its bytes", i * 4, w, s);
+        s.wepoch = epoch, s.wwave = (uint8_t)w;
+        break;
+    }
+  }
+}
+static inline void traced(const void* p, size_t n, bool write) {
+  if ((const char*)p >= __start_hx_lds && (const char*)p < __stop_hx_lds) lds_access(p, n, write ? ACC_WRITE : ACC_READ);
+}
+
 // ---- DMA ----------------------------------------------------------------------------------------------------------
+static Lane* checker_lane;  // a lane of the wave on whose behalf the scheduler touches the LDS (DMA issue / landing)
 static void land_until(Wave& w, size_t upto) {
   for (; w.landed < upto; ++w.landed)
-    for (const Dma& t : w.q[w.landed]) memcpy(t.dst, t.src, t.bytes);
+    for (const Dma& t : w.q[w.landed]) {
+      memcpy(t.dst, t.src, t.bytes);
+      if (checker_lane && !t.idem) {
+        Lane* keep = cur;
+        cur = checker_lane, sched_ctx = true;
+        lds_access(t.dst, t.bytes, ACC_DMA_LAND);
+        cur = keep, sched_ctx = false;
+      }
+    }
 }
 
 uint32_t lds_addr(const void* p) {
@@ -216,7 +299,7 @@ void dma(const void* gptr, uint32_t lds_dst, int bytes) {
   ++n_dma;
   if (!bufs.empty() && !in_a_buffer(gptr, bytes))
     fail("global->LDS DMA reads %d bytes at %p out of bounds: %s", bytes, gptr, describe_address(gptr, bytes).c_str());
-  cur->t = Dma{(const uint8_t*)gptr, lds_ptr(lds_dst, bytes, "global->LDS DMA"), bytes};
+  cur->t = Dma{(const uint8_t*)gptr, lds_ptr(lds_dst, bytes, "global->LDS DMA"), bytes, false};
   collective(C_DMA, 0);  // one wave instruction: the active lanes' transfers travel (and are waited for) together
 }
 
@@ -289,6 +372,7 @@ void ds_read_tr(int elem_bytes, const void* p, void* out8, int site) {
   const char* c = (const char*)p;
   if (c < __start_hx_lds || c + 8 > __stop_hx_lds) fail("transposing LDS read: %p is outside the LDS", p);
   if ((uintptr_t)p & 7) fail("transposing LDS read: address %p is not 8-byte aligned", p);
+  lds_access(p, 8, ACC_READ);
   cur->a = p;
   cur->d = out8;
   cur->i0 = elem_bytes;
@@ -372,10 +456,31 @@ static void resolve(int wave_first, const std::vector<int>& g) {
     case C_SYNC:
       break;
     case C_DMA: {
+      // (issue and landing are checked the same way whether the data is copied now or at the wait: the in-flight mark
+      // stays until the wave's wait covers the instruction)
       Wave& w = waves[wave_first / 64];
-      w.q.emplace_back();
-      for (int id : g) w.q.back().push_back(lanes[id].t);
-      if (!cfg.dma_lazy) land_until(w, w.q.size());
+      w.q.emplace_back();  // (the new instruction is w.q.back(); the ones before it and not yet landed are in flight)
+      for (int id : g) {
+        Dma& t = lanes[id].t;
+        // A transfer of exactly what its destination already holds, with no other transfer into those bytes in flight,
+        // changes nothing whenever it lands (the kernels that keep issuing DMA past their last tile re-fetch that tile
+        // into its own slot): it counts as an instruction for the waits and is otherwise left out of the access check.
+        bool quiet = memcmp(t.dst, t.src, t.bytes) == 0;
+        for (size_t i = (size_t)((char*)t.dst - __start_hx_lds) >> 2; quiet && i <= (size_t)((char*)t.dst - __start_hx_lds + t.bytes - 1) >> 2; ++i)
+          quiet = shadow[i].inflight == 0;
+        // ... and so does a second copy of a transfer of this wave that is still in flight (same source, same destination)
+        for (size_t qi = w.landed; !quiet && qi + 1 < w.q.size(); ++qi)
+          for (const Dma& o : w.q[qi])
+            if (o.src == t.src && o.dst == t.dst && o.bytes == t.bytes) quiet = true;
+        t.idem = quiet;
+        w.q.back().push_back(t);
+        if (!quiet) {
+          cur = &lanes[id], sched_ctx = true;
+          lds_access(t.dst, t.bytes, ACC_DMA_ISSUE);
+          cur = nullptr, sched_ctx = false;
+        }
+        if (!cfg.dma_lazy) memcpy(t.dst, t.src, t.bytes);
+      }
       break;
     }
     case C_WAIT: {
@@ -386,7 +491,9 @@ static void resolve(int wave_first, const std::vector<int>& g) {
           return;
         }
       const size_t keep = (size_t)first.i0;
+      checker_lane = &first;
       if (w.q.size() > keep) land_until(w, w.q.size() - keep);
+      checker_lane = nullptr;
       break;
     }
     case C_RFL:
@@ -532,7 +639,14 @@ static bool run_wave(int first, int count) {
 
 static void run_workgroup(dim3 block) {
   const int n = (int)(block.x * block.y * block.z);
-  if (cfg.poison_lds) memset(__start_hx_lds, 0xFF, __stop_hx_lds - __start_hx_lds);
+  // what the previous workgroup wrote is poisoned again (0xFF: NaN in every format the kernels use), so a read of LDS
+  // bytes this workgroup has not written shows up in the results; and every workgroup starts its own barrier epochs
+  if (dirty_hi > dirty_lo) {
+    if (cfg.poison_lds) memset(__start_hx_lds + dirty_lo, 0xFF, dirty_hi - dirty_lo);
+    memset(shadow + (dirty_lo >> 2), 0, (((dirty_hi - 1) >> 2) - (dirty_lo >> 2) + 1) * sizeof(Shadow));  // incl. in-flight marks of a stopped launch
+  }
+  dirty_lo = ~(size_t)0, dirty_hi = 0;
+  epoch += 2;
   lanes.resize(n);
   for (int i = 0; i < n; ++i) init_lane(lanes[i], i, block);
   const int nwaves = (n + 63) / 64;
@@ -549,6 +663,7 @@ static void run_workgroup(dim3 block) {
     if (done == n) break;
     if (done + at_barrier == n) {  // every wave that still runs has arrived
       ++n_barrier;
+      ++epoch;
       int any = 0;
       for (const Lane& l : lanes)
         if (l.state == BARRIER) any |= l.i0;
@@ -562,7 +677,7 @@ static void run_workgroup(dim3 block) {
     }
   }
   if (!faulted)
-    for (Wave& w : waves) land_until(w, w.q.size());  // transfers still in flight when the wave ends do complete
+    for (size_t wi = 0; wi < waves.size(); ++wi) land_until(waves[wi], waves[wi].q.size());  // transfers in flight at the end do complete
 }
 
 hipError_t run(dim3 grid, dim3 block, const std::function<void()>& fn, const void* kernel) {
@@ -572,6 +687,10 @@ hipError_t run(dim3 grid, dim3 block, const std::function<void()>& fn, const voi
     init_tables();
     stacks = (uint8_t*)mmap(nullptr, (size_t)MAX_LANES * STACK, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
     if (stacks == (uint8_t*)MAP_FAILED) abort();
+    const size_t lds_bytes = __stop_hx_lds - __start_hx_lds;
+    shadow = (Shadow*)mmap(nullptr, (lds_bytes / 4 + 1) * sizeof(Shadow), PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
+    if (shadow == (Shadow*)MAP_FAILED) abort();
+    memset(__start_hx_lds, 0xFF, lds_bytes);
     struct sigaction sa;
     memset(&sa, 0, sizeof sa);
     sa.sa_sigaction = on_segv;
@@ -581,6 +700,7 @@ hipError_t run(dim3 grid, dim3 block, const std::function<void()>& fn, const voi
     if (const char* e = getenv("HX_SIM_DMA_LAZY")) cfg.dma_lazy = atoi(e);
     if (const char* e = getenv("HX_SIM_WAVE_ORDER")) cfg.wave_order = atoi(e);
     if (const char* e = getenv("HX_SIM_INTERLEAVE")) cfg.interleave = atoi(e);
+    if (const char* e = getenv("HX_SIM_CHECK_LDS")) check_lds = atoi(e) != 0;
   }
   const long nthreads = (long)block.x * block.y * block.z;
   if (nthreads < 1 || nthreads > MAX_LANES || grid.x < 1 || grid.y < 1 || grid.z < 1) {
@@ -619,8 +739,29 @@ hipError_t hipDeviceGetAttribute(int* value, hipDeviceAttribute_t, int) {
   return hipSuccess;
 }
 
+// ---- the compiler's load / store tracing calls (kernel objects only are built with tracing) ------------------------------
+extern "C" {
+void __sanitizer_cov_load1(uint8_t* p) { hxsim::traced(p, 1, false); }
+void __sanitizer_cov_load2(uint16_t* p) { hxsim::traced(p, 2, false); }
+void __sanitizer_cov_load4(uint32_t* p) { hxsim::traced(p, 4, false); }
+void __sanitizer_cov_load8(uint64_t* p) { hxsim::traced(p, 8, false); }
+void __sanitizer_cov_load16(__int128* p) { hxsim::traced(p, 16, false); }
+void __sanitizer_cov_store1(uint8_t* p) { hxsim::traced(p, 1, true); }
+void __sanitizer_cov_store2(uint16_t* p) { hxsim::traced(p, 2, true); }
+void __sanitizer_cov_store4(uint32_t* p) { hxsim::traced(p, 4, true); }
+void __sanitizer_cov_store8(uint64_t* p) { hxsim::traced(p, 8, true); }
+void __sanitizer_cov_store16(__int128* p) { hxsim::traced(p, 16, true); }
+void __sanitizer_cov_8bit_counters_init(char*, char*) {}
+void __sanitizer_cov_pcs_init(const uintptr_t*, const uintptr_t*) {}
+}
+
 // ---- C interface for the tests ---------------------------------------------------------------------------------------
 extern "C" {
+int hx_sim_set_check_lds(int on) {
+  const int old = hxsim::check_lds;
+  hxsim::check_lds = on != 0;
+  return old;
+}
 // An operand buffer of `bytes` usable bytes between two inaccessible pages.  end_flush != 0: the last byte sits right
 // before the trailing page (an overrun of one byte faults); otherwise the first byte sits right after the leading page.
 void* hx_sim_alloc(size_t bytes, int end_flush) {
@@ -663,7 +804,7 @@ void hx_sim_counters(uint64_t out[4]) {
   out[0] = hxsim::n_coll;
   out[1] = hxsim::n_dma;
   out[2] = hxsim::n_barrier;
-  out[3] = (uint64_t)(__stop_hx_lds - __start_hx_lds);
+  out[3] = hxsim::n_lds_checked;
 }
 // the conversions, for direct tests against the oracle's codec
 int hx_sim_cvt_pk_fp8(float a, float b) {

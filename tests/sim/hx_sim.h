@@ -187,22 +187,32 @@ inline T shfl_xor(T v, int mask, int site) {
 // ---- HIP device library bits
 #define __HIP_MEMORY_SCOPE_AGENT 4
 #define __hip_atomic_fetch_add(p, v, order, scope) hxsim_fetch_add((p), (v))
-#define __hip_atomic_load(p, order, scope) (*(p))
-#define __hip_atomic_store(p, v, order, scope) (void)(*(p) = (v))
+#define __hip_atomic_load(p, order, scope) hxsim_atomic_load(p)
+#define __hip_atomic_store(p, v, order, scope) hxsim_atomic_store((p), (v))
+template <typename T>
+__attribute__((noinline, no_sanitize("coverage"))) inline T hxsim_atomic_load(const T* p) {
+  return *p;
+}
 template <typename T, typename V>
-inline T hxsim_fetch_add(T* p, V v) {  // work-items run one at a time
+__attribute__((noinline, no_sanitize("coverage"))) inline void hxsim_atomic_store(T* p, V v) {
+  *p = (T)v;
+}
+// (atomics are not plain loads and stores: kept out of the LDS access check)
+#define HXSIM_UNTRACED __attribute__((noinline, no_sanitize("coverage")))
+template <typename T, typename V>
+HXSIM_UNTRACED inline T hxsim_fetch_add(T* p, V v) {  // work-items run one at a time
   const T old = *p;
   *p = old + (T)v;
   return old;
 }
 template <typename T>
-inline T atomicMax(T* p, T v) {
+HXSIM_UNTRACED inline T atomicMax(T* p, T v) {
   const T old = *p;
   if (v > old) *p = v;
   return old;
 }
 template <typename T>
-inline T atomicAdd(T* p, T v) {
+HXSIM_UNTRACED inline T atomicAdd(T* p, T v) {
   const T old = *p;
   *p = old + v;
   return old;

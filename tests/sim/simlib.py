@@ -36,6 +36,7 @@ def load():
         lib.hx_sim_counters.restype, lib.hx_sim_counters.argtypes = None, [_c.POINTER(_c.c_uint64)]
         lib.hx_sim_cvt_pk_fp8.restype, lib.hx_sim_cvt_pk_fp8.argtypes = _c.c_int, [_c.c_float, _c.c_float]
         lib.hx_sim_set_wg_reverse.restype, lib.hx_sim_set_wg_reverse.argtypes = _c.c_int, [_c.c_int]
+        lib.hx_sim_set_check_lds.restype, lib.hx_sim_set_check_lds.argtypes = _c.c_int, [_c.c_int]
         lib.hx_sim_set_cus.restype, lib.hx_sim_set_cus.argtypes = _c.c_int, [_c.c_int]
         lib.hx_sim_selftest.restype, lib.hx_sim_selftest.argtypes = _c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int]
         _lib = lib

@@ -34,9 +34,17 @@ def test_fp8_conversion_is_the_oracles_on_every_code_midpoint_and_neighbour():
     assert (enc[~nan_w] == got[~nan_w]).all()
 
 
-def _selftest(mode, variant):
+def _selftest(mode, variant, check_lds=True):
     lib = simlib.load()
     simlib.configure(variant)
+    old = lib.hx_sim_set_check_lds(int(check_lds))
+    try:
+        return _selftest_run(lib, mode)
+    finally:
+        lib.hx_sim_set_check_lds(old)
+
+
+def _selftest_run(lib, mode):
     with simlib.Arena() as ar:
         src = ar.put(torch.arange(4096, dtype=torch.int32).view(torch.uint8)[:4096].clone())
         dst = ar.out((4096,), torch.uint8, fill=0x11)
@@ -54,17 +62,29 @@ def test_correct_protocol_passes_under_every_variant(variant):
 
 
 def test_missing_wait_is_exposed_by_latest_landing():
-    rc, _, src, dst = _selftest(1, "eager")
-    assert rc == 0 and torch.equal(src, dst)  # lands at once: the defect is invisible, as it mostly is on the hardware
-    rc, _, src, dst = _selftest(1, "lazy")
-    assert rc == 0 and not torch.equal(src, dst)  # the read came first and saw the poisoned LDS
+    """Without the access check: invisible when transfers land at issue (as it mostly is on the hardware), a read of the
+    poisoned LDS when they land as late as the wait allows."""
+    rc, _, src, dst = _selftest(1, "eager", check_lds=False)
+    assert rc == 0 and torch.equal(src, dst)
+    rc, _, src, dst = _selftest(1, "lazy", check_lds=False)
+    assert rc == 0 and not torch.equal(src, dst)
     assert bool((dst == 0xFF).all())
 
 
 def test_missing_barrier_is_exposed_by_the_wave_order():
     want = torch.roll(_selftest(0, "eager")[2].reshape(4, 1024), -1, 0).reshape(-1)  # every wave copies the next one's data
-    results = {v: torch.equal(_selftest(2, v)[3], want) for v in ("eager", "lazy-reverse")}
+    results = {v: torch.equal(_selftest(2, v, check_lds=False)[3], want) for v in ("eager", "lazy-reverse")}
     assert not all(results.values())  # at least one order reads a wave's data before that wave has fetched it
+
+
+@pytest.mark.parametrize("variant", list(simlib.VARIANTS))
+def test_lds_access_check_names_both_defects_under_every_variant(variant):
+    """With the access check (the default) neither defect depends on the schedule to show: the read of bytes whose DMA
+    has not been waited for, and the read of another wave's bytes without a barrier in between, stop the launch."""
+    rc, fault, _, _ = _selftest(1, variant)
+    assert rc != 0 and "LDS race" in fault and "DMA has not been waited for" in fault, fault
+    rc, fault, _, _ = _selftest(2, variant)
+    assert rc != 0 and "LDS race" in fault, fault
 
 
 def test_a_read_one_byte_out_of_range_stops_the_launch_with_its_address():
