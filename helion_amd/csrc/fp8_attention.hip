@@ -32,10 +32,11 @@
 #define ATT_LEAD (ATT_NS - 1)
 
 // K tile: [64 keys][D bytes]; V tile: [D rows][64 bytes].  Rows are 16-byte chunks, swizzled:
-//   row bytes 128: pos = chunk ^ ((row >> 1) & 7);   row bytes 64: pos = chunk ^ ((row >> 2) & 3)
+//   row bytes 128: pos = chunk ^ ((row >> 1) & 7);   row bytes 64: pos = chunk ^ ((row >> 2) & 3);   row bytes 256
+//   (a row fills the 256-byte bank window): pos = chunk ^ (row & 15)
 template <int RB>
 __device__ __forceinline__ int att_swz(int row) {
-  return RB == 128 ? ((row >> 1) & 7) : ((row >> 2) & 3);
+  return RB == 256 ? (row & 15) : RB == 128 ? ((row >> 1) & 7) : ((row >> 2) & 3);
 }
 // V tile in the [keys][D bytes] layout: one transposing read has 32 lanes fetch 8 consecutive key rows x two
 // adjacent 16-byte chunks; the swizzle has to spread those over all banks and must leave bit 0 (which chunk of
@@ -43,7 +44,7 @@ __device__ __forceinline__ int att_swz(int row) {
 // r, r+4 share a 64-byte quarter of it -> (r>>2)&1 into bit 1.
 template <int RB>
 __device__ __forceinline__ int att_vswz(int row) {
-  return RB == 128 ? (((row >> 1) & 3) << 1) : (((row >> 2) & 1) << 1);
+  return RB == 256 ? ((row & 7) << 1) : RB == 128 ? (((row >> 1) & 3) << 1) : (((row >> 2) & 1) << 1);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -92,8 +93,10 @@ __device__ __forceinline__ float att_max_across_halves(float x) {
   return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 
+// D = 256 (opt-in, HX_FEATURE_ATTENTION_D256): the same code with 16 KB tiles - the ring is then 128 KB and the O^T
+// accumulators 128 registers, so one workgroup per CU and one wave per SIMD.
 template <int D, int OUT, int MODE, bool VSD>
-__global__ __launch_bounds__(256, 2) void hx_fp8_attention_pipe(const uint8_t* __restrict__ Q, const uint8_t* __restrict__ Kt,
+__global__ __launch_bounds__(256, D > 128 ? 1 : 2) void hx_fp8_attention_pipe(const uint8_t* __restrict__ Q, const uint8_t* __restrict__ Kt,
                                                                 const uint8_t* __restrict__ Vt, void* __restrict__ Out, int S, int BH,
                                                                 int qtiles, float c) {
   constexpr int KSTEPS = D / 64;  // MFMA k-steps for S = K Q^T
@@ -698,7 +701,7 @@ static int launch_att(const void* q, const void* k, const void* v, void* out, in
 // 1: the MFMA kernel takes these arguments; 0: the plain kernel does.  vsd: V is [S][D] per head.
 static bool att_fast_path(const void* q, const void* k, const void* v, const void* out, int64_t S, int64_t D, int64_t v_stride_d,
                           int64_t v_stride_s, bool* vsd) {
-  bool fast = (D == 64 || D == 128) && S >= 1 && ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) == 0);
+  bool fast = (D == 64 || D == 128 || (D == 256 && hx_feature(HX_FEATURE_ATTENTION_D256))) && S >= 1 && ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) == 0);
   *vsd = false;
   if (v_stride_s == 1 && (v_stride_d == S || D == 1)) {
     *vsd = false;                                  // [D][S] per head: rows of S bytes, fetched in 16-byte pieces
@@ -766,6 +769,10 @@ extern "C" int hx_fp8_attention(const void* q, const void* k, const void* v, voi
   if (D == 128) {
     if (out_dtype == HX_F32) return launch_att<128, HX_F32>(q, k, v, out, BH, S, exact_max, vsd, c, s);
     return launch_att<128, HX_E4M3>(q, k, v, out, BH, S, exact_max, vsd, c, s);
+  }
+  if (D == 256) {
+    if (out_dtype == HX_F32) return launch_att<256, HX_F32>(q, k, v, out, BH, S, exact_max, vsd, c, s);
+    return launch_att<256, HX_E4M3>(q, k, v, out, BH, S, exact_max, vsd, c, s);
   }
   if (out_dtype == HX_F32) return launch_att<64, HX_F32>(q, k, v, out, BH, S, exact_max, vsd, c, s);
   return launch_att<64, HX_E4M3>(q, k, v, out, BH, S, exact_max, vsd, c, s);

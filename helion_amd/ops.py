@@ -100,10 +100,11 @@ def _fp8_attention_impl(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batch
     if out_dtype not in (torch.float8_e4m3fn, torch.float32):
         raise TypeError(f"unsupported out_dtype {out_dtype}")
     d_true = d
-    if d not in (64, 128) and 0 < d < 128:
+    d256 = bool(_lib.load().hx_get_features() & _lib.HX_FEATURE_ATTENTION_D256)  # opt-in: head dim 256 on the MFMA kernel
+    if d not in (64, 128) and 0 < d < 128 or (d256 and 128 < d < 256):
         # zero-pad the head dimension to what the MFMA kernel takes: q.k and the other output columns are unchanged,
         # the softmax scale still comes from the true head dimension
-        dp = 64 if d < 64 else 128
+        dp = 64 if d < 64 else 128 if d < 128 else 256
         q = torch.nn.functional.pad(q.view(torch.uint8), (0, dp - d)).view(torch.float8_e4m3fn)
         k = torch.nn.functional.pad(k.view(torch.uint8), (0, dp - d)).view(torch.float8_e4m3fn)
         v = torch.nn.functional.pad(v.contiguous().view(torch.uint8), (0, 0, 0, dp - d)).view(torch.float8_e4m3fn)
@@ -113,7 +114,7 @@ def _fp8_attention_impl(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batch
     # memory (strides (S*D, 1, D)); the kernel reads that layout directly, so only other stridings are copied.
     if bh > 1 and v.stride(0) != s * d or v.stride()[1:] not in ((s, 1), (1, d)):
         v = v.contiguous()
-    if v.stride()[1:] == (s, 1) and s % 16 != 0 and d in (64, 128) and s > 1:
+    if v.stride()[1:] == (s, 1) and s % 16 != 0 and d in (64, 128, 256) and s > 1:
         # [D][S] rows that are not a multiple of 16 bytes cannot be fetched in 16-byte pieces: hand the MFMA kernel the
         # [S][D] layout instead (one copy) rather than fall to the plain kernel
         v = v.transpose(1, 2).contiguous().transpose(1, 2)

@@ -48,10 +48,12 @@ const char* hx_last_error(void);
 enum {
   HX_FEATURE_SKINNY_ROWMAJOR = 1, /* hx_fp8_gemm, M <= 32, row-major b (ldb_n == 1), K % 1024 == 0, N % 16 == 0: b is
                                     streamed in place (path 6) instead of being transposed through the workspace */
-  HX_FEATURE_FP8_GEMM_ANY_K = 2  /* hx_fp8_gemm with K % 16 != 0 (or rows / pointers that are not 16-byte aligned) and a
+  HX_FEATURE_FP8_GEMM_ANY_K = 2, /* hx_fp8_gemm with K % 16 != 0 (or rows / pointers that are not 16-byte aligned) and a
                                     workspace: the operands are copied once into it as K-contiguous rows zero-padded to
                                     the next multiple of 16 and the MFMA kernels run on the copies, where the plain fp32
                                     kernel ran before (hx_fp8_gemm_path still answers 0 for such a call) */
+  HX_FEATURE_ATTENTION_D256 = 4  /* hx_fp8_attention with head dim 256 on the MFMA kernel (hx_fp8_attention_path 1)
+                                    instead of the one-workgroup-per-query-row kernel */
 };
 unsigned hx_set_features(unsigned mask);
 unsigned hx_get_features(void);

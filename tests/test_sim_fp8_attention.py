@@ -88,3 +88,33 @@ def test_plain_kernel_for_other_head_dims():
     simlib.configure("lazy")
     out = simops.fp8_attention(q, k, v, 1, 2, torch.float32, True, "DS", want_path=0)
     assert attention_close(out, orc.fp8_attention(q, k, v, 1, 2, torch.float32))
+
+
+# ---- opt-in: head dim 256 on the MFMA kernel (HX_FEATURE_ATTENTION_D256) ------------------------------------------------
+@pytest.mark.parametrize("s", [64, 208, 640, 1104])
+@pytest.mark.parametrize("exact", [True, False])
+def test_head_dim_256(s, exact):
+    from helion_amd import _lib
+    q, k, v = _qkv(1, s, 256, s)
+    with simlib.features(_lib.HX_FEATURE_ATTENTION_D256):
+        simlib.configure("lazy-reverse")
+        _check(q, k, v, exact, "DS")
+        simlib.configure("eager-interleaved")
+        _check(q, k, v, exact, "SD", end_flush=False)
+
+
+@pytest.mark.parametrize("variant", list(simlib.VARIANTS))
+def test_head_dim_256_every_variant_and_e4m3_output(variant):
+    from helion_amd import _lib
+    q, k, v = _qkv(2, 331, 256, 3)
+    simlib.configure(variant)
+    with simlib.features(_lib.HX_FEATURE_ATTENTION_D256):
+        _check(q, k, v, True, "SD", E4)
+        _check(q, k, v, False, "SD")
+
+
+def test_head_dim_256_is_the_plain_kernel_by_default():
+    q, k, v = _qkv(1, 48, 256, 1)
+    simlib.configure("lazy")
+    out = simops.fp8_attention(q, k, v, 1, 1, torch.float32, True, "DS", want_path=0)
+    assert attention_close(out, orc.fp8_attention(q, k, v, 1, 1, torch.float32))

@@ -55,3 +55,25 @@ def test_any_k_through_the_mfma_kernels(any_k, m, n, k, rowmajor):
     print(f"any-K case M={m} N={n} K={k} rowmajor={rowmajor}", flush=True)
     out = hx.fp8_gemm(a.to(DEV), y.to(DEV), out_dtype=torch.bfloat16)
     assert rel_err(out, orc.fp8_gemm(a, y, 1.0, 1.0, torch.bfloat16)) <= 1e-2
+
+
+@pytest.fixture
+def d256():
+    old = hx.set_features(hx.HX_FEATURE_ATTENTION_D256)
+    yield
+    hx.set_features(old)
+
+
+@pytest.mark.parametrize("s,d,exact,strided_v", [(64, 256, True, False), (208, 256, True, True), (640, 256, False, False), (1104, 256, True, False),
+                                                 (331, 256, False, True), (500, 192, True, False), (4096, 256, True, False)])
+def test_attention_head_dim_256(d256, s, d, exact, strided_v):
+    g = torch.Generator().manual_seed(s + d)
+    q, k = (torch.randn(2, s, d, generator=g).to(E4) for _ in range(2))
+    v = torch.randn(2, d, s, generator=g).to(E4)
+    vd = v.to(DEV)
+    if strided_v:
+        vd = vd.transpose(1, 2).contiguous().transpose(1, 2)
+    print(f"attention D256 case S={s} D={d} exact={exact} strided_v={strided_v}", flush=True)
+    out = hx.fp8_attention_kernel(q.to(DEV), k.to(DEV), vd, 1, 2, out_dtype=torch.float32, exact_max=exact)
+    ref = orc.fp8_attention(q, k, v, 1, 2, torch.float32) if exact else orc.fp8_attention_tiled(q, k, v, 1, 2, 64, torch.float32)
+    assert rel_err(out, ref) <= 3e-2
