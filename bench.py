@@ -493,6 +493,18 @@ def bench_next_rows(steps, warmup):
     t = _time_launches(decode64, steps, warmup)
     out["decode_gemm_m64"] = hbm(28672 * 8192 + 64 * 8192 + 2 * 64 * 28672, t, "hx_fp8_gemm_tileN128<bf16, 64 rows, paired DMA>",
                                  "fp8_gemm M64 N28672 K8192 bf16 out, 4 rotating weight buffers (HBM-cold)")
+    # the same with 128 and 256 rows (one row tile of the 128-column kernel each): still weight streaming, still HBM-bound
+    for rows in (128, 256):
+        xr = (torch.randn(rows, 8192, device="cuda") * 0.5).to(torch.float8_e4m3fn)
+
+        def decode_rows(xr=xr):
+            turn[0] = (turn[0] + 1) % len(bufs)
+            return hx.fp8_gemm(xr, bufs[turn[0]], out_dtype=torch.bfloat16)
+
+        t = _time_launches(decode_rows, steps, warmup)
+        out[f"decode_gemm_m{rows}"] = hbm(28672 * 8192 + rows * 8192 + 2 * rows * 28672, t, f"hx_fp8_gemm_tileN128<bf16, {rows} rows>",
+                                          f"fp8_gemm M{rows} N28672 K8192 bf16 out, 4 rotating weight buffers (HBM-cold)")
+        del xr
     del bufs, xa
     # routing tables at the C5 row count and at 1M rows
     _, _, ex = inputs.moe_c5("cuda")
@@ -699,27 +711,31 @@ def main():
 
     t, roof = bench_c2(args.steps, args.warmup)
     others = {}
+    def section(key, fn, merge=False):
+        """One workload group after the headline one.  A Python error in it is recorded under its name and the run goes
+        on: the headline line must come out whatever happens to a row beside it.  (A GPU fault is not an exception and
+        ends the process as it should.)"""
+        try:
+            r = fn(args.steps, args.warmup)
+            others.update(r) if merge else others.__setitem__(key, r)
+        except Exception as e:  # noqa: BLE001
+            others[key + "_error"] = f"{type(e).__name__}: {e}"[:400]
+        torch.cuda.empty_cache()
+
     if "lib" in only:
-        others["c2_library_baseline_scaled_mm"] = bench_c2_library_baseline(args.steps, args.warmup)
-        torch.cuda.empty_cache()
+        section("c2_library_baseline_scaled_mm", bench_c2_library_baseline)
     if "c3" in only:
-        others["c3_decode_gemm"] = bench_c3(args.steps, args.warmup)
-        torch.cuda.empty_cache()
+        section("c3_decode_gemm", bench_c3)
     if "c4" in only:
-        others["c4_fp8_attention"] = bench_c4(args.steps, args.warmup)
-        torch.cuda.empty_cache()
+        section("c4_fp8_attention", bench_c4)
     if "c5" in only:
-        others["c5_moe_grouped_gemm"] = bench_c5(args.steps, args.warmup)
-        torch.cuda.empty_cache()
+        section("c5_moe_grouped_gemm", bench_c5)
     if "next" in only:
-        others.update(bench_next_rows(args.steps, args.warmup))
-        torch.cuda.empty_cache()
+        section("next_rows", bench_next_rows, merge=True)
     if "sib" in only:
-        others.update(bench_siblings(args.steps, args.warmup))
-        torch.cuda.empty_cache()
+        section("siblings", bench_siblings, merge=True)
     if "lib16" in only:  # opt-in: vendor-library rows for the 16-bit GEMMs
-        others["library_baselines_16bit"] = bench_16bit_library_baselines(args.steps, args.warmup)
-        torch.cuda.empty_cache()
+        section("library_baselines_16bit", bench_16bit_library_baselines)
     line = {
         "metric": "FP8 GEMM/attention TFLOP/s + % of MI355X FP8 MFMA peak (or % HBM BW), 1 GPU",
         "value": roof["achieved"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

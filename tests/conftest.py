@@ -1,4 +1,5 @@
 import ctypes
+import os
 import pathlib
 import sys
 
@@ -11,6 +12,16 @@ if str(ROOT) not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+def pytest_runtest_logstart(nodeid, location):
+    """Names every GPU test on the real stderr before it starts (unbuffered, past pytest's capture): if a kernel takes the
+    process or the box down, the last line printed says which case it was."""
+    if "test_gpu_" in nodeid or "test_zz_no_alloc" in nodeid or "wip_gpu_" in nodeid:
+        try:
+            os.write(2, f"[gpu-test] {nodeid}\n".encode())
+        except OSError:
+            pass
 
 
 @pytest.fixture(scope="session")
