@@ -103,6 +103,9 @@ static std::string kernel_name() {
   return "?";
 }
 static uint64_t n_coll, n_dma, n_barrier, ticks;
+// work counters of the launches since the last hx_sim_work_reset: wave-level MFMA instructions, bytes moved by DMA, LDS
+// bytes read / written by ordinary and transposing accesses, workgroup barriers, workgroups
+static uint64_t w_mfma, w_dma_bytes, w_lds_read, w_lds_write, w_barriers, w_workgroups;
 
 struct Buf {
   uint8_t* base;  // first usable byte
@@ -232,6 +235,9 @@ static void lds_access(const void* p, size_t n, int kind) {
     if (off < dirty_lo) dirty_lo = off;
     if (off + n > dirty_hi) dirty_hi = off + n;
   }
+  if (kind == ACC_READ) w_lds_read += n;
+  else if (kind == ACC_WRITE) w_lds_write += n;
+  else if (kind == ACC_DMA_ISSUE) w_dma_bytes += n;
   if (!check_lds || !cur) return;
   const int w = cur->tid >> 6;
   ++n_lds_checked;
@@ -474,6 +480,7 @@ static void resolve(int wave_first, const std::vector<int>& g) {
             if (o.src == t.src && o.dst == t.dst && o.bytes == t.bytes) quiet = true;
         t.idem = quiet;
         w.q.back().push_back(t);
+        if (quiet) w_dma_bytes += t.bytes;
         if (!quiet) {
           cur = &lanes[id], sched_ctx = true;
           lds_access(t.dst, t.bytes, ACC_DMA_ISSUE);
@@ -558,6 +565,7 @@ static void resolve(int wave_first, const std::vector<int>& g) {
         fail("MFMA with %zu of 64 lanes active", g.size());
         return;
       }
+      ++w_mfma;
       const int kind = first.i0;
       const bool f8 = kind == MFMA_F8_32x32x64 || kind == MFMA_F8_16x16x128 || kind == MFMA_F8_16x16x32;
       const bool big = kind == MFMA_F8_32x32x64 || kind == MFMA_BF16_32x32x16 || kind == MFMA_F16_32x32x16;
@@ -647,6 +655,7 @@ static void run_workgroup(dim3 block) {
   }
   dirty_lo = ~(size_t)0, dirty_hi = 0;
   epoch += 2;
+  ++w_workgroups;
   lanes.resize(n);
   for (int i = 0; i < n; ++i) init_lane(lanes[i], i, block);
   const int nwaves = (n + 63) / 64;
@@ -663,6 +672,7 @@ static void run_workgroup(dim3 block) {
     if (done == n) break;
     if (done + at_barrier == n) {  // every wave that still runs has arrived
       ++n_barrier;
+      ++w_barriers;
       ++epoch;
       int any = 0;
       for (const Lane& l : lanes)
@@ -757,6 +767,11 @@ void __sanitizer_cov_pcs_init(const uintptr_t*, const uintptr_t*) {}
 
 // ---- C interface for the tests ---------------------------------------------------------------------------------------
 extern "C" {
+void hx_sim_work(uint64_t out[6], int reset) {
+  out[0] = hxsim::w_mfma, out[1] = hxsim::w_dma_bytes, out[2] = hxsim::w_lds_read, out[3] = hxsim::w_lds_write;
+  out[4] = hxsim::w_barriers, out[5] = hxsim::w_workgroups;
+  if (reset) hxsim::w_mfma = hxsim::w_dma_bytes = hxsim::w_lds_read = hxsim::w_lds_write = hxsim::w_barriers = hxsim::w_workgroups = 0;
+}
 int hx_sim_set_check_lds(int on) {
   const int old = hxsim::check_lds;
   hxsim::check_lds = on != 0;
