@@ -449,6 +449,20 @@ static float f16_to_f32(uint16_t h) {
   return s ? -v : v;
 }
 
+// D[i][j] = sum_k A[i][k] * Bt[k][j] in double (every product of two e4m3 or two 16-bit values is exact there, and so is
+// the sum of an fp8 MFMA's 64 or 128 of them): rows of D stay in registers, the inner loop runs along j
+__attribute__((target_clones("avx2", "default"))) static void mfma_product(int MN, int K, const double (*A)[128], const double (*Bt)[32],
+                                                                           double (*D)[32]) {
+  for (int i = 0; i < MN; ++i) {
+    double acc[32] = {0};
+    for (int k = 0; k < K; ++k) {
+      const double a = A[i][k];
+      for (int j = 0; j < 32; ++j) acc[j] += a * Bt[k][j];
+    }
+    for (int j = 0; j < MN; ++j) D[i][j] = acc[j];
+  }
+}
+
 // ---- evaluation of one cross-lane instruction for the lanes `g` (indices into `lanes`) of one wave --------------------
 static void resolve(int wave_first, const std::vector<int>& g) {
   Lane& first = lanes[g[0]];
@@ -573,21 +587,22 @@ static void resolve(int wave_first, const std::vector<int>& g) {
       const int MN = big ? 32 : 16;              // rows of A = columns of B
       const int KL = f8 && kind != MFMA_F8_16x16x32 ? 32 : 8;  // k values one lane supplies
       const int K = KL * (64 / MN);
-      static float A[32][128], B[32][128];
+      static double A[32][128], Bt[128][32], D[32][32];  // A[i][k], B transposed to [k][j], D = A B
       for (int p = 0; p < 64; ++p) {
         const Lane& l = lanes[wave_first + p];
         const int r = p % MN, k0 = (p / MN) * KL;
         for (int k = 0; k < KL; ++k) {
           if (f8) {
             A[r][k0 + k] = e4m3_table[((const uint8_t*)l.a)[k]];
-            B[r][k0 + k] = e4m3_table[((const uint8_t*)l.b)[k]];
+            Bt[k0 + k][r] = e4m3_table[((const uint8_t*)l.b)[k]];
           } else {
             const uint16_t ha = ((const uint16_t*)l.a)[k], hb = ((const uint16_t*)l.b)[k];
             A[r][k0 + k] = bf ? bf16_to_f32(ha) : f16_to_f32(ha);
-            B[r][k0 + k] = bf ? bf16_to_f32(hb) : f16_to_f32(hb);
+            Bt[k0 + k][r] = bf ? bf16_to_f32(hb) : f16_to_f32(hb);
           }
         }
       }
+      mfma_product(MN, K, A, Bt, D);
       const int NR = big ? 16 : 4;  // results per lane
       for (int p = 0; p < 64; ++p) {
         Lane& l = lanes[wave_first + p];
@@ -595,9 +610,7 @@ static void resolve(int wave_first, const std::vector<int>& g) {
         float out[16];
         for (int r = 0; r < NR; ++r) {
           const int i = big ? 8 * (r / 4) + 4 * (p / 32) + (r % 4) : 4 * (p / 16) + r;  // row of D (from operand A)
-          double s = 0.0;
-          for (int k = 0; k < K; ++k) s += (double)A[i][k] * (double)B[j][k];
-          out[r] = (float)((double)((const float*)l.c)[r] + s);
+          out[r] = (float)((double)((const float*)l.c)[r] + D[i][j]);
         }
         memcpy(l.d, out, NR * 4);
       }
