@@ -11,6 +11,7 @@ HX_F16, HX_BF16, HX_F32, HX_E4M3 = 0, 1, 2, 3
 HX_FEATURE_SKINNY_ROWMAJOR = 1
 HX_FEATURE_FP8_GEMM_ANY_K = 2
 HX_FEATURE_ATTENTION_D256 = 4
+HX_FEATURE_FP8_GEMM_PERSISTENT = 8
 
 _LIB_PATH = pathlib.Path(__file__).resolve().parent / "libhx_kernels.so"
 _lib = None

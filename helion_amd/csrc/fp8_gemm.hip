@@ -843,6 +843,7 @@ __global__ __launch_bounds__(512) void hx_fp8_gemm_skinny_direct(const uint8_t* 
 }
 
 #include "fp8_gemm_skinny_rm.h"
+#include "fp8_gemm_tile256p.h"
 
 // ------------------------------------------------------------------------------------------
 // general: 64x64 tile, 256 threads, 4x4 outputs per thread, fp32 FMAs on decoded e4m3.
@@ -939,7 +940,8 @@ static inline bool aligned(const void* p, size_t a) { return ((uintptr_t)p & (a 
 // its MFMAs); 256x128 0.8 us and 9 us, and only with at least three row tiles (with two, an XCD's tiles share too few
 // operand panels: 512 x 14336 x 4096 measured 40 us against 36 for 128x128).
 static int tileN128_rows(int64_t M, int64_t N, int64_t K) {
-  auto rounds = [&](int64_t bm, int64_t bn) { return (((M + bm - 1) / bm) * ((N + bn - 1) / bn) + 255) / 256; };
+  const int64_t cus = hx_cu_count();  // 256 on an MI355X
+  auto rounds = [&](int64_t bm, int64_t bn) { return (((M + bm - 1) / bm) * ((N + bn - 1) / bn) + cus - 1) / cus; };
   if (M <= 64) return 64;
   if (M <= 128) return 128;
   if (M <= 256) return 256;
@@ -1050,9 +1052,19 @@ static int skinny_rm_plan(int64_t N, int64_t K, int* kwg) {
   return (int)(K / *kwg);
 }
 
+// The persistent form of the 256x256 kernel (opt-in, HX_FEATURE_FP8_GEMM_PERSISTENT) takes a problem the plain one would
+// (path 1) when every workgroup gets at least two tiles and the k-tiles pair up; 16-bit outputs only (the launcher checks).
+static bool tile256p_ok(int64_t M, int64_t N, int64_t K) {
+  const int64_t tiles = (M / 256) * (N / 256), grid = (hx_cu_count() / 8) * 8;
+  return hx_feature(HX_FEATURE_FP8_GEMM_PERSISTENT) && K % 256 == 0 && K >= 512 && grid >= 8 && tiles >= 2 * grid;
+}
+
 extern "C" int hx_fp8_gemm_path(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
                                 const void* a, const void* b, const void* c) {
-  if (ldb_k == 1) return gemm_path_kmajor(M, N, K, lda, ldb_n, ldc, a, b, c);
+  if (ldb_k == 1) {
+    const int p = gemm_path_kmajor(M, N, K, lda, ldb_n, ldc, a, b, c);
+    return p == 1 && tile256p_ok(M, N, K) ? 7 : p;
+  }
   if (ldb_n == 1 && skinny_rm_ok(M, N, K, lda, ldb_k, a, b)) return 6;
   if (ldb_n == 1 && gemm_path_rowmajor_ok(M, N, K, lda, ldb_k, a, b)) return 4;
   return 0;
@@ -1163,9 +1175,14 @@ static void launch_kmajor(int path, const void* a, const void* bt, void* c, int6
       launch_tileN128<OUT, 128, false>(b_once, grid, stream, (const uint8_t*)a, (const uint8_t*)bt,
                          (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m, bn, 0);
     }
-  } else if (path == 1 || path == 3) {
+  } else if (path == 7 && OUT != HX_F32) {
+    const int tiles_m = (int)(M / 256), tiles_n = (int)(N / 256), grid = (hx_cu_count() / 8) * 8;
+    hx_launch((hx_fp8_gemm_tile256p<OUT == HX_F32 ? HX_BF16 : OUT>), dim3(grid), dim3(256), 0, stream, (const uint8_t*)a, (const uint8_t*)bt,
+              (typename OutT<OUT == HX_F32 ? HX_BF16 : OUT>::T*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m,
+              tiles_n);
+  } else if (path == 1 || path == 3 || path == 7) {
     const int tiles_m = (int)((M + 255) / 256), tiles_n = (int)((N + 255) / 256);
-    if (path == 1)
+    if (path != 3)
       hx_launch((hx_fp8_gemm_tile256<OUT, false, false>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
                          (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m,
                          tiles_n);

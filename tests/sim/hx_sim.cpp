@@ -61,11 +61,15 @@ struct Lane {
   int i0, i1;
   uint32_t u0, u1;
   Dma t;  // this lane's share of the DMA instruction it is issuing
+  int stores;  // global stores this lane has executed since its wave's last cross-lane instruction
 };
 
 struct Wave {
-  std::vector<std::vector<Dma>> q;  // the wave's DMA instructions in issue order (one vector = one instruction's lanes)
-  size_t landed;                    // instructions [0, landed) have written their data
+  // the wave's vmcnt-counted instructions in issue order: a DMA instruction (the vector holds its lanes' transfers) or a
+  // global store (an empty vector: it only occupies a place in the count - on this chip stores and loads share the
+  // counter and retire in order, so a store issued after a DMA makes a later counted wait reach less far back)
+  std::vector<std::vector<Dma>> q;
+  size_t landed;  // instructions [0, landed) have completed
 };
 
 struct Config {
@@ -185,6 +189,7 @@ static void init_lane(Lane& l, int tid, dim3 block) {
   l.tid = tid;
   l.tid3 = {tid % block.x, (tid / block.x) % block.y, tid / (block.x * block.y)};
   l.state = RUNNABLE;
+  l.stores = 0;
   uint64_t* top = (uint64_t*)(stacks + (size_t)(tid + 1) * STACK);
   // layout read by hx_sim_switch: six registers, then the address it returns to; the entry function then sees the
   // stack alignment of an ordinary call
@@ -272,8 +277,10 @@ static void lds_access(const void* p, size_t n, int kind) {
     }
   }
 }
+static bool in_a_buffer(const void* p, size_t n);
 static inline void traced(const void* p, size_t n, bool write) {
   if ((const char*)p >= __start_hx_lds && (const char*)p < __stop_hx_lds) lds_access(p, n, write ? ACC_WRITE : ACC_READ);
+  else if (write && cur && !sched_ctx && in_a_buffer(p, n)) ++cur->stores;  // a store to an operand: one vmcnt-counted instruction
 }
 
 // ---- DMA ----------------------------------------------------------------------------------------------------------
@@ -467,6 +474,12 @@ __attribute__((target_clones("avx2", "default"))) static void mfma_product(int M
 static void resolve(int wave_first, const std::vector<int>& g) {
   Lane& first = lanes[g[0]];
   ++n_coll;
+  {  // the global stores the wave executed since its last cross-lane instruction take their places in the vmcnt order
+    Wave& w = waves[wave_first / 64];
+    int k = 0;
+    for (int i = wave_first; i < wave_first + 64 && i < (int)lanes.size(); ++i) k = std::max(k, lanes[i].stores), lanes[i].stores = 0;
+    for (int i = 0; i < k; ++i) w.q.emplace_back();
+  }
   auto lane_of = [&](int pos) -> Lane* {  // the group's lane at position `pos` of the wave, or null if it is not in the group
     for (int id : g)
       if (id - wave_first == pos) return &lanes[id];

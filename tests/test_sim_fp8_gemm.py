@@ -239,3 +239,48 @@ def test_any_k_route_really_runs_matrix_instructions():
 
     assert cross_lane_instructions(0) == 0
     assert cross_lane_instructions(_lib.HX_FEATURE_FP8_GEMM_ANY_K) > 100
+
+
+# ---- opt-in: the persistent 256x256 kernel (HX_FEATURE_FP8_GEMM_PERSISTENT) ------------------------------------------------
+def _persistent(m, n, k, cus, variant, od=torch.bfloat16, seed=5):
+    from helion_amd import _lib
+    a, y = _ops(m, n, k, seed + m + n + k, False)
+    simlib.configure(variant)
+    with simlib.features(_lib.HX_FEATURE_FP8_GEMM_PERSISTENT), simlib.cus(cus):
+        simlib.work()
+        out = simops.fp8_gemm(a, y, torch.tensor(1.25), torch.tensor(0.5), od, want_path=7)
+        w = simlib.work()
+    return out, orc.fp8_gemm(a, y, 1.25, 0.5, od), w
+
+
+@pytest.mark.parametrize("variant", ALL)
+def test_persistent_kernel_every_variant(variant):
+    """16 tiles on 8 workgroups: every workgroup hands one tile's accumulators over inside the next tile's first k-tile and
+    ends with the plain epilogue.  K = 512 is the shortest the path takes (k-tiles 0, 1, nk-2, nk-1 and no steady loop)."""
+    out, ref, w = _persistent(1024, 1024, 512, 8, variant)
+    assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+    assert w["workgroups"] == 8 and w["mfma"] == 16 * 4 * 4 * 64  # 16 tiles x 4 k-tiles x 4 waves x 64 MFMAs: the hand-over adds none
+
+
+@pytest.mark.parametrize("m,n,k,cus,variant,od", [
+    (1024, 1280, 768, 8, "lazy", torch.bfloat16),            # 20 tiles on 8 workgroups: 3 / 2 tiles per workgroup; a steady loop of one k-tile
+    (2048, 1024, 1024, 16, "lazy-reverse", torch.bfloat16),  # 32 tiles on 16 workgroups
+    (1024, 1024, 1280, 8, "eager-interleaved", torch.float16),
+])
+def test_persistent_kernel_shapes(m, n, k, cus, variant, od):
+    out, ref, _ = _persistent(m, n, k, cus, variant, od)
+    assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+
+
+def test_persistent_kernel_is_chosen_only_where_every_workgroup_gets_two_tiles():
+    from helion_amd import _lib
+    lib = simlib.load()
+    with simlib.features(_lib.HX_FEATURE_FP8_GEMM_PERSISTENT), simlib.cus(8):
+        def path(m, n, k):
+            return lib.hx_fp8_gemm_path(m, n, k, k, 1, k, n, None, None, None)
+        assert path(1024, 1024, 512) == 7
+        assert path(768, 768, 512) != 7       # 9 tiles on 8 workgroups
+        assert path(1024, 1024, 256) != 7     # a single k-tile pair: nothing to overlap the epilogue with
+        assert path(1024, 1024, 640) != 7     # K % 256 != 0
+    with simlib.cus(8):
+        assert lib.hx_fp8_gemm_path(1024, 1024, 512, 512, 1, 512, 1024, None, None, None) != 7  # off by default

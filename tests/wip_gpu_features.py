@@ -77,3 +77,31 @@ def test_attention_head_dim_256(d256, s, d, exact, strided_v):
     out = hx.fp8_attention_kernel(q.to(DEV), k.to(DEV), vd, 1, 2, out_dtype=torch.float32, exact_max=exact)
     ref = orc.fp8_attention(q, k, v, 1, 2, torch.float32) if exact else orc.fp8_attention_tiled(q, k, v, 1, 2, 64, torch.float32)
     assert rel_err(out, ref) <= 3e-2
+
+
+@pytest.fixture
+def persistent():
+    old = hx.set_features(hx.HX_FEATURE_FP8_GEMM_PERSISTENT)
+    yield
+    hx.set_features(old)
+
+
+@pytest.mark.parametrize("m,n,k,od", [(8192, 8192, 512, torch.bfloat16), (8192, 4096, 1024, torch.float16), (5888, 8192, 768, torch.bfloat16),
+                                      (8192, 8192, 8192, torch.bfloat16)])
+def test_persistent_256_tile_kernel(persistent, m, n, k, od):
+    """Bit-equal to the default 256x256 kernel (same MFMA order per accumulator), and within tolerance of the oracle on
+    the rows the CPU finishes in seconds."""
+    g = torch.Generator().manual_seed(m + n + k)
+    a = (torch.randn(m, k, generator=g) * 0.5).to(E4).to(DEV)
+    bt = (torch.randn(n, k, generator=g) * 0.5).to(E4).to(DEV)
+    sa, sb = torch.tensor(1.25, device=DEV), torch.tensor(0.5, device=DEV)
+    lib = _lib.load()
+    assert lib.hx_fp8_gemm_path(m, n, k, k, 1, k, n, a.data_ptr(), bt.data_ptr(), a.data_ptr()) == 7
+    print(f"persistent case M={m} N={n} K={k} {od}", flush=True)
+    out = hx.fp8_gemm(a, bt.t(), scale_a=sa, scale_b=sb, out_dtype=od)
+    hx.set_features(0)
+    base = hx.fp8_gemm(a, bt.t(), scale_a=sa, scale_b=sb, out_dtype=od)
+    assert torch.equal(out.view(torch.int16), base.view(torch.int16))
+    rows = torch.arange(0, m, 131)
+    ref = orc.fp8_gemm(a[rows.to(DEV)].cpu(), bt.t().cpu(), 1.25, 0.5, od)
+    assert rel_err(out[rows.to(DEV)].cpu(), ref) <= 1e-2
