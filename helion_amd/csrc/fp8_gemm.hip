@@ -844,6 +844,7 @@ __global__ __launch_bounds__(512) void hx_fp8_gemm_skinny_direct(const uint8_t* 
 
 #include "fp8_gemm_skinny_rm.h"
 #include "fp8_gemm_tile256p.h"
+#include "fp8_gemm_decode_ring.h"
 
 // ------------------------------------------------------------------------------------------
 // general: 64x64 tile, 256 threads, 4x4 outputs per thread, fp32 FMAs on decoded e4m3.
@@ -1059,10 +1060,17 @@ static bool tile256p_ok(int64_t M, int64_t N, int64_t K) {
   return hx_feature(HX_FEATURE_FP8_GEMM_PERSISTENT) && K % 256 == 0 && K >= 512 && grid >= 8 && tiles >= 2 * grid;
 }
 
+// decode batches of 33..128 rows on the kernel with separate A / B rings (opt-in: HX_FEATURE_FP8_GEMM_DECODE_RING), where
+// hx_fp8_gemm_tileN128 runs otherwise (path 5 becomes 8)
+static bool decode_ring_ok(int64_t M, int64_t N, int64_t K) {
+  return hx_feature(HX_FEATURE_FP8_GEMM_DECODE_RING) && M > 32 && M <= 128 && tileN128_rows(M, N, K) <= 128;
+}
+
 extern "C" int hx_fp8_gemm_path(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
                                 const void* a, const void* b, const void* c) {
   if (ldb_k == 1) {
     const int p = gemm_path_kmajor(M, N, K, lda, ldb_n, ldc, a, b, c);
+    if (p == 5 && decode_ring_ok(M, N, K)) return 8;
     return p == 1 && tile256p_ok(M, N, K) ? 7 : p;
   }
   if (ldb_n == 1 && skinny_rm_ok(M, N, K, lda, ldb_k, a, b)) return 6;
@@ -1093,6 +1101,17 @@ template <int OUT, int BM, bool PAIR, typename... Args>
 static void launch_tileN128(bool b_read_once, dim3 grid, hipStream_t stream, Args... args) {
   if (b_read_once) hx_launch((hx_fp8_gemm_tileN128<OUT, BM, PAIR, true>), grid, dim3(256), 0, stream, args...);
   else hx_launch((hx_fp8_gemm_tileN128<OUT, BM, PAIR, false>), grid, dim3(256), 0, stream, args...);
+}
+
+template <int OUT, typename... Args>
+static void launch_decode_ring(int bm, bool b_read_once, dim3 grid, hipStream_t stream, Args... args) {
+  if (bm == 64) {
+    if (b_read_once) hx_launch((hx_fp8_gemm_decode_ring<OUT, 64, true, true>), grid, dim3(256), 0, stream, args...);
+    else hx_launch((hx_fp8_gemm_decode_ring<OUT, 64, true, false>), grid, dim3(256), 0, stream, args...);
+  } else {
+    if (b_read_once) hx_launch((hx_fp8_gemm_decode_ring<OUT, 128, false, true>), grid, dim3(256), 0, stream, args...);
+    else hx_launch((hx_fp8_gemm_decode_ring<OUT, 128, false, false>), grid, dim3(256), 0, stream, args...);
+  }
 }
 
 static std::atomic<unsigned long long> g_skd_launches{0};
@@ -1140,7 +1159,7 @@ static void launch_kmajor(int path, const void* a, const void* bt, void* c, int6
       hx_launch((hx_fp8_gemm_tile256<OUT, true, true>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, (const uint8_t*)a,
                          (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m,
                          tiles_n);
-  } else if (path == 5) {
+  } else if (path == 5 || path == 8) {  // (8: the same plan on hx_fp8_gemm_decode_ring, chosen below)
     const int bm = tileN128_rows(M, N, K), bn = tileN128_pitch(M, N);
     const int tiles_m = (int)((M + bm - 1) / bm), tiles_n = (int)((N + bn - 1) / bn);
     int ktps = 0;
@@ -1153,7 +1172,10 @@ static void launch_kmajor(int path, const void* a, const void* bt, void* c, int6
     // split-K launches write unscaled fp32 slabs into the workspace; hx_fp8_gemm_split_reduce sums, scales and casts them
     if (split) {
       float* part = (float*)ws;
-      if (bm == 64)
+      if (decode_ring_ok(M, N, K))
+        launch_decode_ring<HX_F32>(bm, b_once, grid, stream, (const uint8_t*)a, (const uint8_t*)bt, part, (int)M, (int)N, (int)K, (long)lda,
+                                   (long)ldb, (long)N, (const float*)nullptr, (const float*)nullptr, bn, ktps);
+      else if (bm == 64)
         launch_tileN128<HX_F32, 64, true>(b_once, grid, stream, (const uint8_t*)a, (const uint8_t*)bt,
                            part, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)N, nullptr, nullptr, tiles_m, bn, ktps);
       else if (bm == 256)
@@ -1165,6 +1187,9 @@ static void launch_kmajor(int path, const void* a, const void* bt, void* c, int6
       const long quads = (long)M * ((N + 3) / 4);
       hx_launch((hx_fp8_gemm_split_reduce<OUT>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream,
                          (const float*)part, (out_t*)c, (int)M, (int)N, (long)ldc, splits, sa, sb);
+    } else if (decode_ring_ok(M, N, K)) {
+      launch_decode_ring<OUT>(bm, b_once, grid, stream, (const uint8_t*)a, (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda,
+                              (long)ldb, (long)ldc, sa, sb, bn, 0);
     } else if (bm == 64) {
       launch_tileN128<OUT, 64, true>(b_once, grid, stream, (const uint8_t*)a, (const uint8_t*)bt,
                          (out_t*)c, (int)M, (int)N, (int)K, (long)lda, (long)ldb, (long)ldc, sa, sb, tiles_m, bn, 0);

@@ -110,6 +110,10 @@ static uint64_t n_coll, n_dma, n_barrier, ticks;
 // work counters of the launches since the last hx_sim_work_reset: wave-level MFMA instructions, bytes moved by DMA, LDS
 // bytes read / written by ordinary and transposing accesses, workgroup barriers, workgroups
 static uint64_t w_mfma, w_dma_bytes, w_lds_read, w_lds_write, w_barriers, w_workgroups;
+// DMA bytes of the running workgroup that are issued and not yet covered by a wait of the issuing wave (what the code
+// lets be in flight); over the launches since the last reset: the largest value, and its sum / count right after every wait
+static uint64_t fly_bytes, w_fly_max, w_fly_after_wait, w_waits;
+static const uint8_t *fly_lo, *fly_hi;  // if set: only transfers whose source lies in [fly_lo, fly_hi) are counted
 
 struct Buf {
   uint8_t* base;  // first usable byte
@@ -289,6 +293,7 @@ static void land_until(Wave& w, size_t upto) {
   for (; w.landed < upto; ++w.landed)
     for (const Dma& t : w.q[w.landed]) {
       memcpy(t.dst, t.src, t.bytes);
+      if (!fly_lo || (t.src >= fly_lo && t.src < fly_hi)) fly_bytes -= t.bytes;
       if (checker_lane && !t.idem) {
         Lane* keep = cur;
         cur = checker_lane, sched_ctx = true;
@@ -507,6 +512,8 @@ static void resolve(int wave_first, const std::vector<int>& g) {
             if (o.src == t.src && o.dst == t.dst && o.bytes == t.bytes) quiet = true;
         t.idem = quiet;
         w.q.back().push_back(t);
+        if (!fly_lo || (t.src >= fly_lo && t.src < fly_hi)) fly_bytes += t.bytes;
+        if (fly_bytes > w_fly_max) w_fly_max = fly_bytes;
         if (quiet) w_dma_bytes += t.bytes;
         if (!quiet) {
           cur = &lanes[id], sched_ctx = true;
@@ -528,6 +535,7 @@ static void resolve(int wave_first, const std::vector<int>& g) {
       checker_lane = &first;
       if (w.q.size() > keep) land_until(w, w.q.size() - keep);
       checker_lane = nullptr;
+      w_fly_after_wait += fly_bytes, ++w_waits;
       break;
     }
     case C_RFL:
@@ -682,6 +690,7 @@ static void run_workgroup(dim3 block) {
   dirty_lo = ~(size_t)0, dirty_hi = 0;
   epoch += 2;
   ++w_workgroups;
+  fly_bytes = 0;
   lanes.resize(n);
   for (int i = 0; i < n; ++i) init_lane(lanes[i], i, block);
   const int nwaves = (n + 63) / 64;
@@ -747,6 +756,8 @@ hipError_t run(dim3 grid, dim3 block, const std::function<void()>& fn, const voi
   if (faulted) return hipErrorLaunchFailure;  // a fault is sticky until hx_sim_reset, like a device fault is
   body = &fn;
   launch_fn = kernel;
+  static const bool trace = getenv("HX_SIM_TRACE_LAUNCHES") != nullptr;  // one line per launch on stderr
+  if (trace) fprintf(stderr, "[hx_sim] launch %s grid (%u,%u,%u) block %ld\n", kernel_name().c_str(), grid.x, grid.y, grid.z, nthreads);
   geo.block_dim = {block.x, block.y, block.z};
   geo.grid_dim = {grid.x, grid.y, grid.z};
   const unsigned long total = (unsigned long)grid.x * grid.y * grid.z;
@@ -793,10 +804,17 @@ void __sanitizer_cov_pcs_init(const uintptr_t*, const uintptr_t*) {}
 
 // ---- C interface for the tests ---------------------------------------------------------------------------------------
 extern "C" {
-void hx_sim_work(uint64_t out[6], int reset) {
+void hx_sim_work(uint64_t out[9], int reset) {
   out[0] = hxsim::w_mfma, out[1] = hxsim::w_dma_bytes, out[2] = hxsim::w_lds_read, out[3] = hxsim::w_lds_write;
   out[4] = hxsim::w_barriers, out[5] = hxsim::w_workgroups;
-  if (reset) hxsim::w_mfma = hxsim::w_dma_bytes = hxsim::w_lds_read = hxsim::w_lds_write = hxsim::w_barriers = hxsim::w_workgroups = 0;
+  out[6] = hxsim::w_fly_max, out[7] = hxsim::w_fly_after_wait, out[8] = hxsim::w_waits;
+  if (reset) {
+    hxsim::w_mfma = hxsim::w_dma_bytes = hxsim::w_lds_read = hxsim::w_lds_write = hxsim::w_barriers = hxsim::w_workgroups = 0;
+    hxsim::w_fly_max = hxsim::w_fly_after_wait = hxsim::w_waits = 0;
+  }
+}
+void hx_sim_in_flight_source(const void* p, size_t bytes) {  // (nullptr: every transfer counts)
+  hxsim::fly_lo = (const uint8_t*)p, hxsim::fly_hi = (const uint8_t*)p + bytes;
 }
 int hx_sim_set_check_lds(int on) {
   const int old = hxsim::check_lds;

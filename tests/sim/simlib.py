@@ -37,6 +37,7 @@ def load():
         lib.hx_sim_cvt_pk_fp8.restype, lib.hx_sim_cvt_pk_fp8.argtypes = _c.c_int, [_c.c_float, _c.c_float]
         lib.hx_sim_set_wg_reverse.restype, lib.hx_sim_set_wg_reverse.argtypes = _c.c_int, [_c.c_int]
         lib.hx_sim_work.restype, lib.hx_sim_work.argtypes = None, [_c.POINTER(_c.c_uint64), _c.c_int]
+        lib.hx_sim_in_flight_source.restype, lib.hx_sim_in_flight_source.argtypes = None, [_c.c_void_p, _c.c_size_t]
         lib.hx_sim_set_check_lds.restype, lib.hx_sim_set_check_lds.argtypes = _c.c_int, [_c.c_int]
         lib.hx_sim_set_cus.restype, lib.hx_sim_set_cus.argtypes = _c.c_int, [_c.c_int]
         lib.hx_sim_selftest.restype, lib.hx_sim_selftest.argtypes = _c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int]
@@ -148,7 +149,11 @@ class workgroups_last_to_first:
 
 def work(reset: bool = True) -> dict:
     """What the launches since the last reset did: wave-level MFMA instructions, bytes moved global -> LDS by DMA, LDS
-    bytes read / written by the kernels' own loads and stores (transposing reads included), workgroup barriers, workgroups."""
-    c = (_c.c_uint64 * 6)()
+    bytes read / written by the kernels' own loads and stores (transposing reads included), workgroup barriers, workgroups;
+    the most DMA bytes one workgroup had issued and not yet waited for, and the mean of that figure right after its waits
+    (the window of bytes the code lets be in flight: its upper and lower edge)."""
+    c = (_c.c_uint64 * 9)()
     load().hx_sim_work(c, int(reset))
-    return dict(zip(("mfma", "dma_bytes", "lds_read", "lds_write", "barriers", "workgroups"), (int(x) for x in c)))
+    d = dict(zip(("mfma", "dma_bytes", "lds_read", "lds_write", "barriers", "workgroups", "dma_in_flight_max"), (int(x) for x in c)))
+    d["dma_in_flight_after_waits"] = c[7] / c[8] if c[8] else 0.0
+    return d

@@ -18,8 +18,9 @@ def _p(t):
 
 
 def fp8_gemm(x, y, scale_a=None, scale_b=None, out_dtype=torch.bfloat16, end_flush=True, want_path=None, lda=None, poison_ws=None,
-             ws_after=None, ws_bytes=None):
-    """x [M,K] e4m3 (row-major), y [K,N] e4m3 with any of the two layouts the op passes on (strides kept)."""
+             ws_after=None, ws_bytes=None, in_flight_of_b=False):
+    """x [M,K] e4m3 (row-major), y [K,N] e4m3 with any of the two layouts the op passes on (strides kept).
+    in_flight_of_b: simlib.work()'s in-flight figures count only the DMA that reads y."""
     lib = simlib.load()
     m, k = x.shape
     n = y.shape[1]
@@ -46,8 +47,11 @@ def fp8_gemm(x, y, scale_a=None, scale_b=None, out_dtype=torch.bfloat16, end_flu
         ws = ar.empty(wsb) if wsb else None
         if ws is not None and poison_ws is not None:
             ws.copy_(poison_ws(wsb))
+        if in_flight_of_b:
+            lib.hx_sim_in_flight_source(Y.data_ptr(), Y.numel())
         rc = lib.hx_fp8_gemm(X.data_ptr(), Y.data_ptr(), C.data_ptr(), m, n, k, lda, ldb_k, ldb_n, n, _p(sa), _p(sb), _DT[out_dtype],
                              _p(ws), wsb, None)
+        lib.hx_sim_in_flight_source(None, 0)
         simlib.check(rc, "hx_fp8_gemm")
         if ws_after is not None and ws is not None:
             ws_after.append(ws.clone())

@@ -284,3 +284,58 @@ def test_persistent_kernel_is_chosen_only_where_every_workgroup_gets_two_tiles()
         assert path(1024, 1024, 640) != 7     # K % 256 != 0
     with simlib.cus(8):
         assert lib.hx_fp8_gemm_path(1024, 1024, 512, 512, 1, 512, 1024, None, None, None) != 7  # off by default
+
+
+# ---- opt-in: decode batches of 33..128 rows with separate A / B rings (HX_FEATURE_FP8_GEMM_DECODE_RING) ---------------------
+def _decode_ring(m, n, k, variant, od=torch.bfloat16, **kw):
+    from helion_amd import _lib
+    a, y = _ops(m, n, k, 11 + m + n + k, False)
+    sa, sb = torch.tensor(1.25), torch.tensor(0.5)
+    simlib.configure(variant)
+    base = simops.fp8_gemm(a, y, sa, sb, od, want_path=5)
+    with simlib.features(_lib.HX_FEATURE_FP8_GEMM_DECODE_RING):
+        simlib.work()
+        out = simops.fp8_gemm(a, y, sa, sb, od, want_path=8, **kw)
+        w = simlib.work()
+    return out, base, orc.fp8_gemm(a, y, 1.25, 0.5, od), w
+
+
+@pytest.mark.parametrize("variant", ALL)
+@pytest.mark.parametrize("m", [64, 128])   # 64: B waves issue pairs of k-tiles into a ring of 8; 128: single k-tiles into a ring of 7
+def test_decode_ring_kernel_every_variant(variant, m):
+    out, base, ref, _ = _decode_ring(m, 256, 2560, variant)   # 20 k-tiles: every ring wraps at least twice
+    assert torch.equal(out.view(torch.int16), base.view(torch.int16))  # same MFMA order as the kernel it replaces
+    assert rel_err(out, ref) <= 1e-2
+
+
+@pytest.mark.parametrize("m,n,k,od", [
+    (33, 100, 128, torch.bfloat16),     # a single k-tile: the prologue re-fetches it into every stage
+    (40, 512, 1024, torch.bfloat16),    # few tiles, K >= 1024: split-K slabs + reduce
+    (100, 640, 512, torch.float16),     # ragged rows and a column pitch below 128
+    (64, 144, 256, torch.float32),      # two k-tiles, a last tile of 16 columns
+    (65, 112, 1280, torch.bfloat16),
+    (128, 1792, 1024, torch.bfloat16),
+    (96, 128, 8192, torch.bfloat16),    # 64 k-tiles in 8 splits
+])
+def test_decode_ring_kernel_shapes(m, n, k, od):
+    for variant in FAST:
+        out, base, ref, _ = _decode_ring(m, n, k, variant, od)
+        assert torch.equal(out.view(torch.uint8), base.view(torch.uint8)), variant
+        assert rel_err(out, ref) <= 1e-2, variant
+
+
+def test_decode_ring_kernel_keeps_twice_the_weight_bytes_in_flight():
+    """What the kernel is for: with 128 rows the single-ring kernel lets 2 - 3 weight stages (32 - 48 KB) per workgroup be in
+    flight, the two-ring one 5 - 6 (80 - 96 KB).  Counted by the model under lazy landing: bytes of B issued and not yet
+    covered by a wait of the issuing wave, at their peak and right after the waits."""
+    from helion_amd import _lib
+    a, y = _ops(128, 896, 2048, 3, False)
+    simlib.configure("lazy")
+    fig = {}
+    for mask, path in ((0, 5), (_lib.HX_FEATURE_FP8_GEMM_DECODE_RING, 8)):
+        with simlib.features(mask):
+            simlib.work()
+            simops.fp8_gemm(a, y, None, None, torch.bfloat16, want_path=path, ws_bytes=0, in_flight_of_b=True)  # (no workspace: no split-K)
+            fig[path] = simlib.work()
+    assert fig[5]["dma_in_flight_max"] <= 3 * 16384 + 4096 and fig[8]["dma_in_flight_max"] >= 6 * 16384
+    assert fig[8]["dma_in_flight_after_waits"] >= 2 * fig[5]["dma_in_flight_after_waits"]

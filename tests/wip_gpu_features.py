@@ -105,3 +105,31 @@ def test_persistent_256_tile_kernel(persistent, m, n, k, od):
     rows = torch.arange(0, m, 131)
     ref = orc.fp8_gemm(a[rows.to(DEV)].cpu(), bt.t().cpu(), 1.25, 0.5, od)
     assert rel_err(out[rows.to(DEV)].cpu(), ref) <= 1e-2
+
+
+@pytest.fixture
+def decode_ring():
+    old = hx.set_features(hx.HX_FEATURE_FP8_GEMM_DECODE_RING)
+    yield
+    hx.set_features(old)
+
+
+@pytest.mark.parametrize("m,n,k,od", [(33, 100, 128, torch.bfloat16), (64, 256, 2560, torch.bfloat16), (128, 256, 2560, torch.float16),
+                                      (100, 640, 512, torch.float32), (40, 512, 1024, torch.bfloat16), (96, 128, 8192, torch.bfloat16),
+                                      (64, 28672, 8192, torch.bfloat16), (128, 28672, 8192, torch.bfloat16)])
+def test_decode_ring_kernel(decode_ring, m, n, k, od):
+    """Bit-equal to the kernel it replaces (hx_fp8_gemm_tileN128: same MFMA order), and within tolerance of the oracle."""
+    g = torch.Generator().manual_seed(m + n + k)
+    a = (torch.randn(m, k, generator=g) * 0.5).to(E4)
+    bt = (torch.randn(n, k, generator=g) * 0.5).to(E4)
+    ad, btd = a.to(DEV), bt.to(DEV)
+    sa, sb = torch.tensor(1.25, device=DEV), torch.tensor(0.5, device=DEV)
+    assert _lib.load().hx_fp8_gemm_path(m, n, k, k, 1, k, n, ad.data_ptr(), btd.data_ptr(), ad.data_ptr()) == 8
+    print(f"decode ring case M={m} N={n} K={k} {od}", flush=True)
+    out = hx.fp8_gemm(ad, btd.t(), scale_a=sa, scale_b=sb, out_dtype=od)
+    hx.set_features(0)
+    base = hx.fp8_gemm(ad, btd.t(), scale_a=sa, scale_b=sb, out_dtype=od)
+    assert torch.equal(out.view(torch.uint8), base.view(torch.uint8))
+    cols = torch.arange(0, n, max(1, n // 512))
+    ref = orc.fp8_gemm(a, bt[cols].t(), 1.25, 0.5, od)
+    assert rel_err(out[:, cols.to(DEV)].cpu(), ref) <= 1e-2
