@@ -14,7 +14,8 @@
 #include "hx_common.h"
 
 #define RT_WAVES 16
-#define RT_MAX_E 512
+#define RT_MAX_E 512        // experts of the default instantiation (32 KB of per-wave counters)
+#define RT_MAX_E_WIDE 2048  // opt-in (HX_FEATURE_ROUTING_WIDE): 128 KB of per-wave counters, two experts per work-item in the scans
 #define RT_UNROLL 8
 
 // lanes of this wave that hold the same in-range expert id as the calling lane (0 for out-of-range lanes)
@@ -56,17 +57,19 @@ __device__ __forceinline__ void rt_for_rows(const IdT* __restrict__ ids, int beg
 // MODE 0: the whole job in one workgroup.  MODE 1 (count): workgroup b writes its per-expert row counts to
 // block_tab[b][E].  MODE 2 (scatter): block_tab[b][e] holds the first output slot of workgroup b's rows of expert e
 // (hx_moe_routing_scan turned the counts into slots) and the workgroup scatters its rows.
-template <typename IdT, int MODE>
+// ME: experts the LDS tables hold (RT_MAX_E or RT_MAX_E_WIDE); a work-item owns experts tid, tid + 1024, ... below ME.
+template <typename IdT, int MODE, int ME = RT_MAX_E>
 __global__ __launch_bounds__(64 * RT_WAVES) void hx_moe_routing_kernel(const IdT* __restrict__ ids, int T, int E, int nbits,
                                                                       int block_rows, int32_t* __restrict__ counts,
                                                                       int32_t* __restrict__ offsets, int32_t* __restrict__ idx,
                                                                       int32_t* __restrict__ max_count, int32_t* __restrict__ block_tab) {
-  __shared__ int hist[RT_WAVES][RT_MAX_E];  // count pass: rows per (wave, expert); afterwards: next output slot
-  __shared__ int scan[2][RT_MAX_E];
+  __shared__ int hist[RT_WAVES][ME];  // count pass: rows per (wave, expert); afterwards: next output slot
+  __shared__ int scan[2][ME];
   __shared__ int s_max;
+  constexpr int NT = 64 * RT_WAVES, EPT = (ME + NT - 1) / NT;  // experts per work-item
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const uint64_t lt_mask = ((uint64_t)1 << lane) - 1;
-  for (int i = tid; i < RT_WAVES * RT_MAX_E; i += 64 * RT_WAVES) (&hist[0][0])[i] = 0;
+  for (int i = tid; i < RT_WAVES * ME; i += 64 * RT_WAVES) (&hist[0][0])[i] = 0;
   if (tid == 0) s_max = 0;
   __syncthreads();
 
@@ -112,38 +115,57 @@ __global__ __launch_bounds__(64 * RT_WAVES) void hx_moe_routing_kernel(const IdT
   __syncthreads();
 
   // ---- per expert: prefix over the waves of this workgroup
-  int total = 0;
-  if (tid < E) {
-    for (int ww = 0; ww < RT_WAVES; ++ww) {
-      const int v = hist[ww][tid];
-      hist[ww][tid] = total;
-      total += v;
+  int total[EPT];
+#pragma unroll
+  for (int u = 0; u < EPT; ++u) {
+    const int e = tid + u * NT;
+    total[u] = 0;
+    if (e < E) {
+      for (int ww = 0; ww < RT_WAVES; ++ww) {
+        const int v = hist[ww][e];
+        hist[ww][e] = total[u];
+        total[u] += v;
+      }
     }
   }
   if (MODE == 1) {
-    if (tid < E) block_tab[(long long)blockIdx.x * E + tid] = total;
+#pragma unroll
+    for (int u = 0; u < EPT; ++u)
+      if (tid + u * NT < E) block_tab[(long long)blockIdx.x * E + tid + u * NT] = total[u];
     return;
   }
   int covered;
   if (MODE == 0) {
-    // exclusive prefix over experts (inclusive Hillis-Steele scan over RT_MAX_E slots, minus the own count)
-    if (tid < E) {
-      counts[tid] = total;
-      atomicMax(&s_max, total);
+    // exclusive prefix over experts (inclusive Hillis-Steele scan over ME slots, minus the own count)
+#pragma unroll
+    for (int u = 0; u < EPT; ++u) {
+      const int e = tid + u * NT;
+      if (e < E) {
+        counts[e] = total[u];
+        atomicMax(&s_max, total[u]);
+      }
+      if (e < ME) scan[0][e] = e < E ? total[u] : 0;
     }
-    if (tid < RT_MAX_E) scan[0][tid] = tid < E ? total : 0;
     __syncthreads();
     int src = 0;
-    for (int d = 1; d < RT_MAX_E; d <<= 1) {
-      if (tid < RT_MAX_E) scan[src ^ 1][tid] = scan[src][tid] + (tid >= d ? scan[src][tid - d] : 0);
+    for (int d = 1; d < ME; d <<= 1) {
+#pragma unroll
+      for (int u = 0; u < EPT; ++u) {
+        const int e = tid + u * NT;
+        if (e < ME) scan[src ^ 1][e] = scan[src][e] + (e >= d ? scan[src][e - d] : 0);
+      }
       src ^= 1;
       __syncthreads();
     }
     covered = E > 0 ? scan[src][E - 1] : 0;
-    if (tid < E) {
-      const int excl = scan[src][tid] - total;
-      offsets[tid] = excl;
-      for (int ww = 0; ww < RT_WAVES; ++ww) hist[ww][tid] += excl;
+#pragma unroll
+    for (int u = 0; u < EPT; ++u) {
+      const int e = tid + u * NT;
+      if (e < E) {
+        const int excl = scan[src][e] - total[u];
+        offsets[e] = excl;
+        for (int ww = 0; ww < RT_WAVES; ++ww) hist[ww][e] += excl;
+      }
     }
     if (tid == 0) {
       offsets[E] = covered;
@@ -151,9 +173,13 @@ __global__ __launch_bounds__(64 * RT_WAVES) void hx_moe_routing_kernel(const IdT
     }
   } else {
     covered = offsets[E];
-    if (tid < E) {
-      const int first = block_tab[(long long)blockIdx.x * E + tid];
-      for (int ww = 0; ww < RT_WAVES; ++ww) hist[ww][tid] += first;
+#pragma unroll
+    for (int u = 0; u < EPT; ++u) {
+      const int e = tid + u * NT;
+      if (e < E) {
+        const int first = block_tab[(long long)blockIdx.x * E + e];
+        for (int ww = 0; ww < RT_WAVES; ++ww) hist[ww][e] += first;
+      }
     }
   }
   __syncthreads();
@@ -171,35 +197,52 @@ __global__ __launch_bounds__(64 * RT_WAVES) void hx_moe_routing_kernel(const IdT
 }
 
 // block_tab[b][e] (counts) -> first output slot of workgroup b's rows of expert e; also counts, offsets, max_count.
-__global__ __launch_bounds__(RT_MAX_E) void hx_moe_routing_scan(int32_t* __restrict__ block_tab, int B, int E, int32_t* __restrict__ counts,
-                                                                int32_t* __restrict__ offsets, int32_t* __restrict__ max_count) {
-  __shared__ int scan[2][RT_MAX_E];
+// One workgroup of min(ME, 1024) work-items.
+template <int ME>
+__global__ __launch_bounds__(ME < 1024 ? ME : 1024) void hx_moe_routing_scan(int32_t* __restrict__ block_tab, int B, int E,
+                                                                             int32_t* __restrict__ counts, int32_t* __restrict__ offsets,
+                                                                             int32_t* __restrict__ max_count) {
+  __shared__ int scan[2][ME];
   __shared__ int s_max;
+  constexpr int NT = ME < 1024 ? ME : 1024, EPT = ME / NT;
   const int tid = threadIdx.x;
   if (tid == 0) s_max = 0;
   __syncthreads();
-  int total = 0;
-  if (tid < E) {
-    for (int b = 0; b < B; ++b) {
-      const int v = block_tab[(long long)b * E + tid];
-      block_tab[(long long)b * E + tid] = total;
-      total += v;
+  int total[EPT];
+#pragma unroll
+  for (int u = 0; u < EPT; ++u) {
+    const int e = tid + u * NT;
+    total[u] = 0;
+    if (e < E) {
+      for (int b = 0; b < B; ++b) {
+        const int v = block_tab[(long long)b * E + e];
+        block_tab[(long long)b * E + e] = total[u];
+        total[u] += v;
+      }
+      counts[e] = total[u];
+      atomicMax(&s_max, total[u]);
     }
-    counts[tid] = total;
-    atomicMax(&s_max, total);
+    scan[0][e] = e < E ? total[u] : 0;
   }
-  scan[0][tid] = tid < E ? total : 0;
   __syncthreads();
   int src = 0;
-  for (int d = 1; d < RT_MAX_E; d <<= 1) {
-    scan[src ^ 1][tid] = scan[src][tid] + (tid >= d ? scan[src][tid - d] : 0);
+  for (int d = 1; d < ME; d <<= 1) {
+#pragma unroll
+    for (int u = 0; u < EPT; ++u) {
+      const int e = tid + u * NT;
+      scan[src ^ 1][e] = scan[src][e] + (e >= d ? scan[src][e - d] : 0);
+    }
     src ^= 1;
     __syncthreads();
   }
-  if (tid < E) {
-    const int excl = scan[src][tid] - total;
-    offsets[tid] = excl;
-    for (int b = 0; b < B; ++b) block_tab[(long long)b * E + tid] += excl;
+#pragma unroll
+  for (int u = 0; u < EPT; ++u) {
+    const int e = tid + u * NT;
+    if (e < E) {
+      const int excl = scan[src][e] - total[u];
+      offsets[e] = excl;
+      for (int b = 0; b < B; ++b) block_tab[(long long)b * E + e] += excl;
+    }
   }
   if (tid == 0) {
     offsets[E] = E > 0 ? scan[src][E - 1] : 0;
@@ -218,30 +261,33 @@ static inline void rt_blocks(int64_t T, int64_t* block_rows, int64_t* blocks) {
   *blocks = (T + br - 1) / br;
 }
 
+// most experts a call may name: RT_MAX_E, or RT_MAX_E_WIDE with the opt-in instantiation
+static int64_t rt_max_e() { return hx_feature(HX_FEATURE_ROUTING_WIDE) ? RT_MAX_E_WIDE : RT_MAX_E; }
+
 extern "C" size_t hx_moe_routing_workspace_bytes(int64_t T, int64_t E) {
-  if (T <= RT_SINGLE_MAX_T || E <= 0 || E > RT_MAX_E) return 0;
+  if (T <= RT_SINGLE_MAX_T || E <= 0 || E > rt_max_e()) return 0;
   int64_t br, nb;
   rt_blocks(T, &br, &nb);
   return (size_t)nb * (size_t)E * 4;
 }
 
-template <typename IdT>
+template <typename IdT, int ME>
 static void rt_launch(const IdT* ids, int64_t T, int64_t E, int nbits, int32_t* counts, int32_t* offsets, int32_t* idx,
                       int32_t* max_count, void* ws, size_t ws_bytes, hipStream_t s) {
   const size_t need = hx_moe_routing_workspace_bytes(T, E);
   if (need == 0 || !ws || ws_bytes < need) {
     const int block_rows = (int)((((T + RT_WAVES - 1) / RT_WAVES + 63) & ~(int64_t)63) * RT_WAVES);
-    hx_launch((hx_moe_routing_kernel<IdT, 0>), dim3(1), dim3(64 * RT_WAVES), 0, s, ids, (int)T, (int)E, nbits,
+    hx_launch((hx_moe_routing_kernel<IdT, 0, ME>), dim3(1), dim3(64 * RT_WAVES), 0, s, ids, (int)T, (int)E, nbits,
                        block_rows > 0 ? block_rows : 64 * RT_WAVES, counts, offsets, idx, max_count, (int32_t*)nullptr);
     return;
   }
   int64_t br, nb;
   rt_blocks(T, &br, &nb);
   int32_t* tab = (int32_t*)ws;
-  hx_launch((hx_moe_routing_kernel<IdT, 1>), dim3((unsigned)nb), dim3(64 * RT_WAVES), 0, s, ids, (int)T, (int)E, nbits, (int)br,
+  hx_launch((hx_moe_routing_kernel<IdT, 1, ME>), dim3((unsigned)nb), dim3(64 * RT_WAVES), 0, s, ids, (int)T, (int)E, nbits, (int)br,
                      counts, offsets, idx, max_count, tab);
-  hx_launch(hx_moe_routing_scan, dim3(1), dim3(RT_MAX_E), 0, s, tab, (int)nb, (int)E, counts, offsets, max_count);
-  hx_launch((hx_moe_routing_kernel<IdT, 2>), dim3((unsigned)nb), dim3(64 * RT_WAVES), 0, s, ids, (int)T, (int)E, nbits, (int)br,
+  hx_launch(hx_moe_routing_scan<ME>, dim3(1), dim3(ME < 1024 ? ME : 1024), 0, s, tab, (int)nb, (int)E, counts, offsets, max_count);
+  hx_launch((hx_moe_routing_kernel<IdT, 2, ME>), dim3((unsigned)nb), dim3(64 * RT_WAVES), 0, s, ids, (int)T, (int)E, nbits, (int)br,
                      counts, offsets, idx, max_count, tab);
 }
 
@@ -251,8 +297,8 @@ extern "C" int hx_moe_routing(const void* expert_ids, int ids_are_int64, int64_t
     hx_set_error("hx_moe_routing: negative size");
     return HX_ERR_BAD_ARG;
   }
-  if (E > RT_MAX_E || T >= (1LL << 31) - 64 * RT_WAVES * RT_UNROLL) {
-    hx_set_error("hx_moe_routing: unsupported size T=%lld E=%lld (E <= %d)", (long long)T, (long long)E, RT_MAX_E);
+  if (E > rt_max_e() || T >= (1LL << 31) - 64 * RT_WAVES * RT_UNROLL) {
+    hx_set_error("hx_moe_routing: unsupported size T=%lld E=%lld (E <= %d)", (long long)T, (long long)E, (int)rt_max_e());
     return HX_ERR_UNSUPPORTED;
   }
   if (!offsets || !max_count || (E > 0 && !counts) || (T > 0 && (!expert_ids || !idx))) {
@@ -266,8 +312,11 @@ extern "C" int hx_moe_routing(const void* expert_ids, int ids_are_int64, int64_t
   int nbits = 0;
   while ((1LL << nbits) < E) ++nbits;
   hipStream_t s = (hipStream_t)stream;
-  if (ids_are_int64) rt_launch((const long long*)expert_ids, T, E, nbits, counts, offsets, idx, max_count, workspace, workspace_bytes, s);
-  else rt_launch((const int*)expert_ids, T, E, nbits, counts, offsets, idx, max_count, workspace, workspace_bytes, s);
+  if (E > RT_MAX_E) {
+    if (ids_are_int64) rt_launch<long long, RT_MAX_E_WIDE>((const long long*)expert_ids, T, E, nbits, counts, offsets, idx, max_count, workspace, workspace_bytes, s);
+    else rt_launch<int, RT_MAX_E_WIDE>((const int*)expert_ids, T, E, nbits, counts, offsets, idx, max_count, workspace, workspace_bytes, s);
+  } else if (ids_are_int64) rt_launch<long long, RT_MAX_E>((const long long*)expert_ids, T, E, nbits, counts, offsets, idx, max_count, workspace, workspace_bytes, s);
+  else rt_launch<int, RT_MAX_E>((const int*)expert_ids, T, E, nbits, counts, offsets, idx, max_count, workspace, workspace_bytes, s);
   hipError_t err = hx_launch_status();
   if (err != hipSuccess) {
     hx_set_error("hx_moe_routing: launch failed: %s", hipGetErrorString(err));

@@ -16,13 +16,19 @@ def moe_matmul_ogs(A: torch.Tensor, W: torch.Tensor, expert_token_counts: torch.
                              int(max_T_per_expert_tensor.numel()))
 
 
+def _routing_max_experts() -> int:
+    """Experts the routing kernel's LDS tables hold: 512, or 2048 with the opt-in instantiation switched on."""
+    from . import _lib
+    return 2048 if _lib.load().hx_get_features() & _lib.HX_FEATURE_ROUTING_WIDE else 512
+
+
 def moe_matmul_ogs_helion_kernel_args_gen(A: torch.Tensor, W: torch.Tensor, top1_expert_per_token: torch.Tensor):
     """examples/moe_matmul_ogs.py:84-121: stable sort of rows by expert, per-expert counts and offsets.
     On the GPU the three tables come from one routing kernel; the host synchronisation the reference has
     (``.item()`` for the size of the dummy tensor, :113) is kept because the signature needs that size."""
     E = W.size(0)
     device = A.device
-    if A.is_cuda and E <= 512 and top1_expert_per_token.dtype in (torch.int32, torch.int64):
+    if A.is_cuda and E <= _routing_max_experts() and top1_expert_per_token.dtype in (torch.int32, torch.int64):
         counts, offsets, idx, max_count = moe_routing_call(top1_expert_per_token, E)
         return (A, W, counts, offsets, idx, torch.empty(int(max_count.item()), device=device))
     sorted_to_orig_token_idx = torch.argsort(top1_expert_per_token, stable=True).to(torch.int32)

@@ -57,8 +57,10 @@ enum {
   HX_FEATURE_FP8_GEMM_PERSISTENT = 8, /* hx_fp8_gemm on the 256x256 tile kernel with at least two tiles per CU, K % 256 == 0
                                     and a 16-bit output: persistent workgroups whose epilogue runs inside the next tile's
                                     first k-tile (path 7) */
-  HX_FEATURE_FP8_GEMM_DECODE_RING = 16 /* hx_fp8_gemm with 33..128 rows and a column-major b: the weight-streaming kernel with
+  HX_FEATURE_FP8_GEMM_DECODE_RING = 16, /* hx_fp8_gemm with 33..128 rows and a column-major b: the weight-streaming kernel with
                                     separate LDS rings and wave streams for a and b (path 8 where path 5 ran before) */
+  HX_FEATURE_ROUTING_WIDE = 32  /* hx_moe_routing with 513..2048 experts (HX_ERR_UNSUPPORTED before): the same kernels with
+                                    LDS tables for 2048 experts */
 };
 unsigned hx_set_features(unsigned mask);
 unsigned hx_get_features(void);
@@ -178,7 +180,7 @@ int hx_moe_grouped_gemm_static(const void* A, const void* W, void* C, const int3
  *   offsets = [0, cumsum(counts)]; *max_count = max(counts)   (the reference's `.item()` value, left on the device).
  * expert_ids: [T] device array of int32 (ids_are_int64 == 0) or int64; counts [E], offsets [E+1], idx [T],
  * max_count [1] are int32 device arrays.  Ids outside [0, E) are skipped: their rows appear in no expert's list,
- * offsets[E] is then < T and idx[offsets[E]..T) is filled with -1.  Supported: E <= 512, T < 2^31 - 8192.
+ * offsets[E] is then < T and idx[offsets[E]..T) is filled with -1.  Supported: E <= 512 (E <= 2048 with HX_FEATURE_ROUTING_WIDE), T < 2^31 - 8192.
  * workspace: hx_moe_routing_workspace_bytes(T, E) bytes of device scratch (0 up to 32768 rows, where one workgroup
  * does the whole job in one launch); with less, larger inputs also run on that one workgroup, correct but slow. */
 int hx_moe_routing(const void* expert_ids, int ids_are_int64, int64_t T, int64_t E, int32_t* counts, int32_t* offsets,

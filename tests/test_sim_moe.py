@@ -108,6 +108,30 @@ def test_routing_tables(T, E, dtype):
         assert int(offsets[0]) == 0 and torch.equal(offsets[1:], torch.cumsum(rc, 0).int()) and int(mx) == int(rc.max())
 
 
+@pytest.mark.parametrize("T,E,dtype", [(3000, 513, torch.int64), (5000, 1100, torch.int32), (20000, 2048, torch.int64), (70000, 2048, torch.int32),
+                                       (40000, 1500, torch.int64), (100, 2000, torch.int32)])
+def test_routing_tables_for_513_to_2048_experts(T, E, dtype):
+    """Opt-in (HX_FEATURE_ROUTING_WIDE): the same kernels with LDS tables for 2048 experts, two experts per work-item in the
+    scans; one workgroup up to 32768 rows, count / scan / scatter launches above."""
+    from helion_amd import _lib
+    g = torch.Generator().manual_seed(T + E)
+    ids = torch.randint(0, E, (T,), generator=g).to(dtype)
+    ids[::7] = E - 1   # a crowded last expert, and most experts nearly empty at the small T
+    lib = simlib.load()
+    simlib.configure("lazy")
+    out = [torch.zeros(n, dtype=torch.int32) for n in (E, E + 1, max(T, 1), 1)]
+    assert lib.hx_moe_routing(ids.data_ptr(), int(dtype == torch.int64), T, E, *[t.data_ptr() for t in out], None, 0, None) != 0  # off by default
+    lib.hx_sim_reset()
+    with simlib.features(_lib.HX_FEATURE_ROUTING_WIDE):
+        for variant in ("lazy", "eager-interleaved"):
+            simlib.configure(variant)
+            counts, offsets, idx, mx = simops.moe_routing(ids, E)
+            rc = torch.bincount(ids.long(), minlength=E).int()
+            assert torch.equal(counts, rc) and torch.equal(idx, torch.argsort(ids.long(), stable=True).int())
+            assert int(offsets[0]) == 0 and torch.equal(offsets[1:], torch.cumsum(rc, 0).int()) and int(mx) == int(rc.max())
+        assert lib.hx_moe_routing(ids.data_ptr(), int(dtype == torch.int64), T, 2049, *[t.data_ptr() for t in out], None, 0, None) != 0
+
+
 def test_routing_skips_ids_out_of_range():
     ids = torch.tensor([3, -1, 0, 9, 3, 2, 100, 0], dtype=torch.int64)
     simlib.configure("lazy")

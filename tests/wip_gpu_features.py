@@ -133,3 +133,21 @@ def test_decode_ring_kernel(decode_ring, m, n, k, od):
     cols = torch.arange(0, n, max(1, n // 512))
     ref = orc.fp8_gemm(a, bt[cols].t(), 1.25, 0.5, od)
     assert rel_err(out[:, cols.to(DEV)].cpu(), ref) <= 1e-2
+
+
+@pytest.fixture
+def routing_wide():
+    old = hx.set_features(hx.HX_FEATURE_ROUTING_WIDE)
+    yield
+    hx.set_features(old)
+
+
+@pytest.mark.parametrize("T,E,dtype", [(3000, 513, torch.int64), (20000, 2048, torch.int64), (70000, 2048, torch.int32), (1 << 20, 1024, torch.int64)])
+def test_routing_tables_for_513_to_2048_experts(routing_wide, T, E, dtype):
+    g = torch.Generator().manual_seed(T + E)
+    ids = torch.randint(0, E, (T,), generator=g).to(dtype)
+    print(f"wide routing case T={T} E={E} {dtype}", flush=True)
+    counts, offsets, idx, mx = hx.moe_routing(ids.to(DEV), E)
+    rc = torch.bincount(ids.long(), minlength=E).int()
+    assert torch.equal(counts.cpu(), rc) and torch.equal(idx.cpu(), torch.argsort(ids.long(), stable=True).int())
+    assert torch.equal(offsets.cpu()[1:], torch.cumsum(rc, 0).int()) and int(mx) == int(rc.max())
