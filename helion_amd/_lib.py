@@ -14,6 +14,7 @@ HX_FEATURE_ATTENTION_D256 = 4
 HX_FEATURE_FP8_GEMM_PERSISTENT = 8
 HX_FEATURE_FP8_GEMM_DECODE_RING = 16
 HX_FEATURE_ROUTING_WIDE = 32
+HX_FEATURE_MOE_PERSISTENT = 64
 
 _LIB_PATH = pathlib.Path(__file__).resolve().parent / "libhx_kernels.so"
 _lib = None

@@ -18,6 +18,9 @@
 //   * waits: the stores of a hand-over are newer than the DMA instructions the next counted wait is for and older than
 //     the ones issued after them, so the two waits that follow a hand-over allow 32 instructions in flight instead of 16
 //     (16 DMA + 16 stores); all other waits are the plain kernel's.
+// Every MFMA is written as an instruction with its accumulator an explicit operand (hx_common.h: hx_mfma_..._acc /
+// _overwrite, hx_acc_read), so that all 256 accumulators keep their registers around the tile loop and nothing is spilled:
+// a reload from scratch memory would make the compiler wait for every DMA in flight.
 // Tiles are dealt to the workgroups so that the 32 workgroups of an XCD work on 32 consecutive tiles of that XCD's range
 // of the grouped raster at any time, as the plain kernel's launch order does.
 #pragma once
@@ -105,10 +108,11 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256p(const uint8_t* __res
   // waited for).
   auto ktile = [&](int stage, const uint8_t* pa, const uint8_t* pb, long kb, auto keep_c) {
     constexpr int KEEP = decltype(keep_c)::value;
+    HX_OPAQUE_S(stage);  // (every k-tile computes its fragment addresses from the stage it is given, at run time)
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
       const int bi = i >> 2, bj = i & 3;
-      acc[bj][bi] = hx_mfma_16x16x128_e4m3(fb[bj], fa[bi], acc[bj][bi]);
+      hx_mfma_16x16x128_e4m3_acc(acc[bj][bi], fb[bj], fa[bi]);
       if (i & 1) issue_one(pa, pb, kb, stage, i >> 1);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -117,7 +121,7 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256p(const uint8_t* __res
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
       const int bi = i >> 2, bj = 4 + (i & 3);
-      acc[bj][bi] = hx_mfma_16x16x128_e4m3(fb[bj], fa[bi], acc[bj][bi]);
+      hx_mfma_16x16x128_e4m3_acc(acc[bj][bi], fb[bj], fa[bi]);
       if ((i & 3) == 3) load_a(fa[bi], stage ^ 1, bi);
       if ((i & 7) == 1) load_b(fb[i >> 3], stage ^ 1, i >> 3);
       if (i >= 28) load_b(fb[4 + (i - 28)], stage ^ 1, 4 + (i - 28));
@@ -136,7 +140,7 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256p(const uint8_t* __res
       for (int bj = 0; bj < 8; ++bj) {
         ov4 o;
 #pragma unroll
-        for (int b = 0; b < 4; ++b) o[b] = (out_t)(acc[bj][2 * g32 + h][b] * alpha);
+        for (int b = 0; b < 4; ++b) o[b] = (out_t)(hx_acc_read(acc[bj][2 * g32 + h][b]) * alpha);
         const int row = h * 16 + r16;  // row of the group; columns 16 bj + 4 gq .. + 3 = bytes 32 bj + 8 gq .. + 7
         *(ov4*)(st + row * 256 + (((2 * bj + (gq >> 1)) ^ (row & 15)) * 16) + (gq & 1) * 8) = o;
         // one block at a time: with all 256 accumulators and 128 fragment registers live there is no room for the
@@ -176,7 +180,6 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256p(const uint8_t* __res
   // tile's accumulators, or, for the workgroup's first tile, of the zeros the accumulators start with, which go to the
   // tile's own (not yet written) part of C and are overwritten by its real values later - then k-tiles 1 .. nk-1.
   long mp = m0, np = n0;  // the tile whose accumulators the next hand-over stores
-  const v4f zero4 = {0.f, 0.f, 0.f, 0.f};
   for (int ti = 0; ti < nt; ++ti) {
     // where the DMA goes on once this tile's own k-tiles are all issued: the next tile, or (last tile) this tile's last
     // k-tile again, into a stage nobody reads any more - every k-tile issues its 16 DMA instructions, the waits stay constant
@@ -194,7 +197,7 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_tile256p(const uint8_t* __res
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int bi = 2 * g32 + (i & 1), bj = i >> 1;
-        acc[bj][bi] = hx_mfma_16x16x128_e4m3(fb[bj], fa[bi], zero4);
+        hx_mfma_16x16x128_e4m3_overwrite(acc[bj][bi], fb[bj], fa[bi]);
         if (decltype(with_dma)::value && (i & 1)) issue_one(pa, pb, 2L * T256_BK, 0, 8 * (g32 & 1) + (i >> 1));
         if (decltype(second_half)::value) {
           // fragments die in this order: the A blocks of the first half are dead already, this group's after their last

@@ -58,6 +58,14 @@ __device__ __forceinline__ uint32_t hx_lds_addr(const void* p) {
   return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t*)p;
 }
 
+// The value goes through an empty instruction the compiler cannot see through (in a vector / a scalar register): what is
+// computed from it afterwards cannot be folded to a constant or moved out of the enclosing loop.  The persistent tile
+// kernels use it to keep address arithmetic inside their tile loop: hoisted, the several hundred loop-invariant addresses
+// are kept in scratch memory, and a reload from scratch makes the compiler wait for every vector-memory operation in
+// flight, the hand-counted DMA included.
+#define HX_OPAQUE_V(x) asm volatile("" : "+v"(x))
+#define HX_OPAQUE_S(x) asm volatile("" : "+s"(x))
+
 // s_waitcnt encodings (gfx9): vmcnt [3:0]+[15:14], expcnt [6:4], lgkmcnt [11:8]
 #define HX_WAIT_VM0() __builtin_amdgcn_s_waitcnt(0x0F70)
 #define HX_WAIT_LGKM0() __builtin_amdgcn_s_waitcnt(0xC07F)
@@ -75,6 +83,31 @@ __device__ __forceinline__ v4f hx_mfma_16x16x128_e4m3(v8i a, v8i b, v4f c) {
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
 }
 
+// The matrix instructions of the persistent tile kernels, written as instructions rather than builtins so that the 256
+// accumulators of a wave have one register class and one home each.  Left to the compiler's own accumulator handling, a
+// kernel whose accumulators are carried around a tile loop, read out for conversion in one place and restarted from zero
+// in another, has its live ranges split between accumulator and ordinary registers, with hundreds of copies and spills
+// where the pieces meet - and a reload from scratch memory makes the compiler wait for every vector-memory operation in
+// flight, the hand-counted DMA included.
+//   *_acc:       D = A x B + D, the accumulator an in-and-out operand in an accumulator register;
+//   *_overwrite: D = A x B, the accumulator an output only (its old value is dead: it has just been read out);
+//   hx_acc_read: one element of an accumulator copied to an ordinary register at exactly this point.
+// The operands come from LDS reads, which the compiler's own waits cover for inline assembly too.  What it does not know
+// for inline assembly is the matrix pipe's result latency: the kernels never touch an accumulator within several MFMAs
+// of the instruction that wrote it (an accumulator is used once per 64 MFMAs, and read out only after a barrier).
+__device__ __forceinline__ void hx_mfma_16x16x128_e4m3_overwrite(v4f& acc, v8i a, v8i b) {
+  asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0" : "=a"(acc) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void hx_mfma_16x16x128_e4m3_acc(v4f& acc, v8i a, v8i b) {
+  asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+
+__device__ __forceinline__ float hx_acc_read(float e) {
+  float t;
+  asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t) : "a"(e));
+  return t;
+}
+
 // 16-bit MFMA (32x32x16, fp32 accumulate): lane l supplies 8 elements of row/col l%32, k = 8*(l/32) .. +7; the result
 // layout is that of the 32x32 fp8 MFMA above.  run16 is the 16x16x32 shape: lane l supplies row/col l%16, k = 8*(l/16)
 // .. +7, and receives D[4*(l/16) + r][l%16], r = 0..3.
@@ -86,6 +119,13 @@ struct Mfma16<true> {
   typedef v8bf V8;
   static __device__ __forceinline__ v16f run(v8bf a, v8bf b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
   static __device__ __forceinline__ v4f run16(v8bf a, v8bf b, v4f c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
+  // (see hx_mfma_16x16x128_e4m3_overwrite)
+  static __device__ __forceinline__ void overwrite16(v4f& acc, v8bf a, v8bf b) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=a"(acc) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void acc16(v4f& acc, v8bf a, v8bf b) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+  }
 };
 template <>
 struct Mfma16<false> {
@@ -93,6 +133,12 @@ struct Mfma16<false> {
   typedef v8h V8;
   static __device__ __forceinline__ v16f run(v8h a, v8h b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
   static __device__ __forceinline__ v4f run16(v8h a, v8h b, v4f c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ void overwrite16(v4f& acc, v8h a, v8h b) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(acc) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void acc16(v4f& acc, v8h a, v8h b) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+  }
 };
 
 template <int OUT>

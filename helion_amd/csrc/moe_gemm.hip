@@ -16,6 +16,7 @@
 
 #include "gemm16_tile128.h"
 #include "gemm16_rows32.h"
+#include "gemm16_tile256p.h"
 
 // workspace layout: [0] int num_tiles | [16 ..) MoeTile table[max_tiles] | flags[T] bytes
 static inline size_t moe_table_bytes(int64_t max_tiles) { return 16 + (size_t)max_tiles * sizeof(MoeTile); }
@@ -234,13 +235,15 @@ extern "C" size_t hx_moe_workspace_bytes(int64_t T, int64_t E) {
   // sized for the smallest row tile (32), which needs the longest table
   size_t b = moe_table_bytes(moe_max_tiles(T, E, 32));
   b = (b + 255) & ~(size_t)255;
-  return b + (size_t)T + 256;
+  // (with the persistent kernel switched on: room behind the flags for its store sink, 16-byte aligned)
+  return b + (size_t)T + 256 + (hx_feature(HX_FEATURE_MOE_PERSISTENT) ? G16P_SINK_BYTES + 16 : 0);
 }
 
 // Which kernel multiplies a grouped GEMM: 0 = hx_moe_general (fp32 FMAs; rows that are not 16-byte aligned, K % 8 != 0 or
 // N % 8 != 0), 1 = 32-row tiles, 2 = 128-row tiles, 3 = 256-row tiles, 4 = 128-row tiles with a partial last k-tile
 // (K % 64 != 0), 5 = the same with A fetched in 4-byte pieces (K even but not a multiple of 8: 4-byte aligned rows, e.g.
-// the K = 500 of the reference's own check); 1-5 are MFMA kernels.
+// the K = 500 of the reference's own check); 1-5 are MFMA kernels.  6 (opt-in, HX_FEATURE_MOE_PERSISTENT): the 256-row
+// tiles in persistent workgroups, where 3 would run and N % 256 == 0, K % 128 == 0, K >= 256.
 static int moe_path(const void* A, const void* W, const void* C, int64_t T, int64_t K, int64_t N, int64_t E, int64_t a_div) {
   const bool fast = (K % 2 == 0) && (N % 8 == 0) && K >= 2 && (((T + a_div - 1) / a_div) * K * 2 < (1LL << 32)) && (N * 4 < (1LL << 31)) &&
                     (((uintptr_t)A | (uintptr_t)W | (uintptr_t)C) & 15) == 0;
@@ -253,7 +256,9 @@ static int moe_path(const void* A, const void* W, const void* C, int64_t T, int6
   const bool small = E > 0 && (T / E < 512 || ((T + MOE_BM - 1) / MOE_BM + E / 2) * tn256 < 192);
   // a handful of rows in all: 32-row tiles (a quarter of the A bytes per stage, more weight bytes in flight per CU)
   if (T <= R32_BM) return 1;
-  return small ? 2 : 3;
+  if (small) return 2;
+  if (hx_feature(HX_FEATURE_MOE_PERSISTENT) && N % MOE_BN == 0 && K % (2 * MOE_BK) == 0 && K >= 4 * MOE_BK && hx_cu_count() >= 8) return 6;
+  return 3;
 }
 
 extern "C" int hx_moe_path(int64_t T, int64_t K, int64_t N, int64_t E, int64_t a_div, const void* A, const void* W, const void* C) {
@@ -267,7 +272,7 @@ static int launch_moe(const void* A, const void* W, void* C, const int32_t* coun
   typedef typename Mfma16<BF>::T T16;
   const int path = moe_path(A, W, C, T, K, N, E, a_div);
   const bool fast = path != 0;
-  const int bm = path == 1 ? R32_BM : path == 3 ? MOE_BM : path == 0 ? 64 : G128_BM;
+  const int bm = path == 1 ? R32_BM : (path == 3 || path == 6) ? MOE_BM : path == 0 ? 64 : G128_BM;
   const int max_tiles = (int)moe_max_tiles(T, E, bm);
   int* num_tiles = (int*)ws;
   MoeTile* table = (MoeTile*)((uint8_t*)ws + 16);
@@ -288,7 +293,12 @@ static int launch_moe(const void* A, const void* W, void* C, const int32_t* coun
   if (fast) {
     G16Dense d = {};
     d.lda = K; d.ldb = N; d.ldc = N;
-    if (bm == R32_BM) {
+    if (path == 6) {
+      const int tiles_n = (int)(N / MOE_BN), grid = (hx_cu_count() / 8) * 8;
+      uint8_t* sink = (uint8_t*)(((uintptr_t)flags + (size_t)T + 15) & ~(uintptr_t)15);  // behind the flags (hx_moe_workspace_bytes)
+      hx_launch((hx_gemm16_tile256p<BF>), dim3(grid), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W, (void*)C,
+                (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, tiles_n, (int)a_div, sink);
+    } else if (bm == R32_BM) {
       const int tiles_n = (int)((N + R32_BN - 1) / R32_BN);
       hx_launch((hx_gemm16_rows32<BF, 3>), dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W,
                          (void*)C, (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, max_tiles, tiles_n,

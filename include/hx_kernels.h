@@ -59,8 +59,11 @@ enum {
                                     first k-tile (path 7) */
   HX_FEATURE_FP8_GEMM_DECODE_RING = 16, /* hx_fp8_gemm with 33..128 rows and a column-major b: the weight-streaming kernel with
                                     separate LDS rings and wave streams for a and b (path 8 where path 5 ran before) */
-  HX_FEATURE_ROUTING_WIDE = 32  /* hx_moe_routing with 513..2048 experts (HX_ERR_UNSUPPORTED before): the same kernels with
+  HX_FEATURE_ROUTING_WIDE = 32, /* hx_moe_routing with 513..2048 experts (HX_ERR_UNSUPPORTED before): the same kernels with
                                     LDS tables for 2048 experts */
+  HX_FEATURE_MOE_PERSISTENT = 64 /* the grouped GEMM's 256-row tiles (hx_moe_path 3) with N % 256 == 0, K % 128 == 0, K >= 256
+                                    in persistent workgroups whose epilogue runs inside the next tile's first k-tile
+                                    (hx_moe_path 6); hx_moe_workspace_bytes grows by about 1 KB while it is on */
 };
 unsigned hx_set_features(unsigned mask);
 unsigned hx_get_features(void);

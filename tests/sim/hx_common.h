@@ -43,6 +43,9 @@ inline const uint8_t* hx_uniform_ptr(const uint8_t* p) {
 }
 inline uint32_t hx_lds_addr(const void* p) { return hxsim::lds_addr(p); }
 
+#define HX_OPAQUE_V(x) ((void)(x))
+#define HX_OPAQUE_S(x) ((void)(x))
+
 #define HX_WAIT_VM0() __builtin_amdgcn_s_waitcnt(0x0F70)
 #define HX_WAIT_LGKM0() __builtin_amdgcn_s_waitcnt(0xC07F)
 inline constexpr int hx_vmcnt_imm(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
@@ -54,6 +57,10 @@ inline v4f hx_mfma_16x16x128_e4m3(v8i a, v8i b, v4f c) {
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
 }
 
+inline float hx_acc_read(float e) { return e; }
+inline void hx_mfma_16x16x128_e4m3_overwrite(v4f& acc, v8i a, v8i b) { acc = hx_mfma_16x16x128_e4m3(a, b, (v4f){0.f, 0.f, 0.f, 0.f}); }
+inline void hx_mfma_16x16x128_e4m3_acc(v4f& acc, v8i a, v8i b) { acc = hx_mfma_16x16x128_e4m3(a, b, acc); }
+
 template <bool BF>
 struct Mfma16;
 template <>
@@ -62,6 +69,8 @@ struct Mfma16<true> {
   typedef v8bf V8;
   static inline v16f run(v8bf a, v8bf b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
   static inline v4f run16(v8bf a, v8bf b, v4f c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
+  static inline void overwrite16(v4f& acc, v8bf a, v8bf b) { acc = run16(a, b, (v4f){0.f, 0.f, 0.f, 0.f}); }
+  static inline void acc16(v4f& acc, v8bf a, v8bf b) { acc = run16(a, b, acc); }
 };
 template <>
 struct Mfma16<false> {
@@ -69,6 +78,8 @@ struct Mfma16<false> {
   typedef v8h V8;
   static inline v16f run(v8h a, v8h b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
   static inline v4f run16(v8h a, v8h b, v4f c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
+  static inline void overwrite16(v4f& acc, v8h a, v8h b) { acc = run16(a, b, (v4f){0.f, 0.f, 0.f, 0.f}); }
+  static inline void acc16(v4f& acc, v8h a, v8h b) { acc = run16(a, b, acc); }
 };
 
 template <int OUT>

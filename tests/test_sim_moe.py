@@ -146,3 +146,58 @@ def test_topk_entry_equals_the_replicated_rows_form(tokens, K, N, E, topk, dtype
     simlib.configure("lazy-reverse")
     out = simops.moe_topk(A[::topk].contiguous(), W, ex, topk)
     assert rel_err(out, orc.moe_matmul_ogs_reference(A, W, ex)) <= 1e-2
+
+
+# ---- opt-in: the 256-row tiles in persistent workgroups (HX_FEATURE_MOE_PERSISTENT, hx_moe_path 6) ---------------------------
+def _persistent(T, K, N, E, cus, variant, dtype=torch.bfloat16, drop_expert=None, with_base=True):
+    from helion_amd import _lib
+    A, W, ex = inputs.moe_inputs(T, K, N, E, 1, seed=T + K, dtype=dtype)
+    counts, offsets, idx = _tables(ex, E)
+    if drop_expert is not None:
+        counts[drop_expert] = 0   # its rows are covered by nobody: they must come out zero
+    simlib.configure(variant)
+    with simlib.cus(cus):
+        base = simops.moe_grouped_gemm(A, W, counts, offsets, idx, want_path=3, poison=7.0) if with_base else None
+        with simlib.features(_lib.HX_FEATURE_MOE_PERSISTENT):
+            simlib.work()
+            out = simops.moe_grouped_gemm(A, W, counts, offsets, idx, want_path=6, poison=5.0)
+            w = simlib.work()
+    w["row_tiles"] = int(((counts + 255) // 256).sum())
+    return out, base, orc.moe_matmul_ogs(A, W, counts, offsets, idx), w
+
+
+@pytest.mark.parametrize("T,K,N,E,cus,variant,dtype,with_base", [
+    (6144, 256, 2048, 2, 8, "lazy", torch.bfloat16, True),                # the shortest K the path takes: k-tiles 0, 1, nk-2, nk-1 only
+    (6144, 256, 2048, 3, 16, "lazy-reverse", torch.bfloat16, False),      # 200-odd tiles on 16 workgroups: a ragged last step
+    (6144, 384, 2048, 3, 8, "eager-interleaved", torch.float16, False),   # six k-tiles: a steady loop of two
+] + ([(6400, 512, 2048, 4, 24, "lazy-interleaved", torch.bfloat16, True)] if __import__("os").environ.get("HX_SIM_SWEEP") == "1" else []))
+def test_persistent_grouped_kernel(T, K, N, E, cus, variant, dtype, with_base):
+    """Every workgroup hands each tile's accumulators over inside the next tile's first k-tile and ends with a plain
+    epilogue; rows that are not stored go to the sink behind the row flags.  Bit-equal to the kernel it replaces."""
+    out, base, ref, w = _persistent(T, K, N, E, cus, variant, dtype, with_base=with_base)
+    if with_base:
+        assert torch.equal(out.view(torch.int16), base.view(torch.int16))
+    assert rel_err(out, ref) <= 1e-2
+    # 4 waves x 128 MFMAs per tile and k-tile: the hand-over adds none
+    assert w["mfma"] == w["row_tiles"] * (N // 256) * (K // 64) * 512
+
+
+def test_persistent_grouped_kernel_with_an_expert_switched_off():
+    out, _, ref, _ = _persistent(6144, 256, 2048, 3, 8, "lazy", drop_expert=1, with_base=False)
+    assert rel_err(out, ref) <= 1e-2 and bool((ref == 0).any())
+
+
+def test_persistent_grouped_kernel_is_chosen_only_for_whole_column_tiles_and_even_k_tiles():
+    from helion_amd import _lib
+    lib = simlib.load()
+    with simlib.cus(8):
+        def path(T, K, N, E):
+            return lib.hx_moe_path(T, K, N, E, 1, None, None, None)
+        assert path(6144, 256, 2048, 2) == 3                  # off by default
+        with simlib.features(_lib.HX_FEATURE_MOE_PERSISTENT):
+            assert path(6144, 256, 2048, 2) == 6
+            assert path(6144, 128, 2048, 2) == 3              # two k-tiles: nothing to overlap with
+            assert path(6144, 320, 2048, 2) != 6              # an odd number of k-tiles
+            assert path(6144, 256, 2176, 2) == 3              # a ragged last column tile
+            assert path(1024, 256, 2048, 8) == 2              # small experts keep the 128-row tiles
+            assert lib.hx_moe_workspace_bytes(6144, 2) >= 1024 + 6144

@@ -151,3 +151,29 @@ def test_routing_tables_for_513_to_2048_experts(routing_wide, T, E, dtype):
     rc = torch.bincount(ids.long(), minlength=E).int()
     assert torch.equal(counts.cpu(), rc) and torch.equal(idx.cpu(), torch.argsort(ids.long(), stable=True).int())
     assert torch.equal(offsets.cpu()[1:], torch.cumsum(rc, 0).int()) and int(mx) == int(rc.max())
+
+
+@pytest.fixture
+def moe_persistent():
+    old = hx.set_features(hx.HX_FEATURE_MOE_PERSISTENT)
+    yield
+    hx.set_features(old)
+
+
+@pytest.mark.parametrize("T,K,N,E,dtype", [(65536, 256, 2048, 4, torch.bfloat16), (65536, 384, 1024, 8, torch.float16),
+                                           (40000, 1024, 4096, 3, torch.bfloat16), (65536, 4096, 14336, 8, torch.bfloat16)])
+def test_persistent_grouped_gemm(moe_persistent, T, K, N, E, dtype):
+    """Bit-equal to the default 256-row-tile kernel (same MFMA order per accumulator); a sample of rows against the oracle."""
+    from helion_amd import inputs
+    A, W, ex = inputs.moe_inputs(T, K, N, E, 1, seed=T + K, dtype=dtype, device=DEV)
+    lib = _lib.load()
+    assert lib.hx_moe_path(T, K, N, E, 1, A.data_ptr(), W.data_ptr(), A.data_ptr()) == 6
+    print(f"persistent grouped case T={T} K={K} N={N} E={E} {dtype}", flush=True)
+    args = hx.moe_matmul_ogs_helion_kernel_args_gen(A, W, ex)
+    out = hx.moe_matmul_ogs(*args)
+    hx.set_features(0)
+    base = hx.moe_matmul_ogs(*args)
+    assert torch.equal(out.view(torch.int16), base.view(torch.int16))
+    rows = torch.arange(0, T, 997, device=DEV)
+    ref = orc.moe_matmul_ogs_reference(A[rows].cpu(), W.cpu(), ex[rows].cpu())
+    assert rel_err(out[rows].cpu(), ref) <= 1e-2
