@@ -103,3 +103,35 @@ def test_attention_check(batch, heads, seq, dim, dtype):
     out = simops.attention16(q, k, v)
     ref = orc.attention(q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0))[0]
     torch.testing.assert_close(out.float(), ref.float(), atol=1e-2, rtol=1e-2)
+
+
+def test_the_smoke_run_case_by_case():
+    """The cases of `__graft_entry__.smoke()` (same seeded inputs, same tolerances) in the host execution model, so that a
+    change that would break the smoke run on the GPU is seen on the CPU first."""
+    from helion_amd import inputs
+
+    def rel(a, b):
+        return float((a.float() - b.float()).abs().max() / b.float().abs().max())
+
+    simlib.configure("lazy")
+    a, b, sa, sb = inputs.gemm_scaled(256, 512, 384, 1)
+    assert rel(simops.fp8_gemm(a, b, sa, sb, torch.bfloat16), orc.fp8_gemm(a, b, sa, sb, torch.bfloat16)) <= 1e-2
+    a, b, sa, sb = inputs.gemm_scaled(16, 256, 1024, 2)
+    assert rel(simops.fp8_gemm(a, b, sa, sb, torch.bfloat16, want_path=2), orc.fp8_gemm(a, b, sa, sb, torch.bfloat16)) <= 1e-2
+    for s, seed in ((256, 3), (208, 4)):   # 208: a partial last key tile
+        q, k, v = inputs.attention_inputs(1, 2, s, 128, seed)
+        out = simops.fp8_attention(q, k, v, 1, 2, torch.float32, True, "DS", want_path=1)
+        assert rel(out, orc.fp8_attention(q, k, v, 1, 2, torch.float32)) <= 2e-2
+    for (T, K, N, E, seed), path in (((300, 120, 256, 5, 6), 4), ((512, 256, 512, 4, 4), 2)):   # K = 120: a partial last k-tile
+        A, W, ex = inputs.moe_inputs(T, K, N, E, 1, seed)
+        counts, offsets, idx, _ = simops.moe_routing(ex, E)
+        out = simops.moe_grouped_gemm(A, W, counts, offsets, idx, want_path=path, poison=2.0)
+        assert rel(out, orc.moe_matmul_ogs_reference(A, W, ex)) <= 1e-2
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(300, 256, generator=g).bfloat16()
+    y = torch.randn(256, 264, generator=g).bfloat16()
+    bias = torch.randn(264, generator=g).bfloat16()
+    assert rel(simops.matmul(x, y, bias=bias, relu=True), orc.matmul(x, y, bias, relu=True)) <= 1e-2
+    q, k, v = (torch.randn(2, 2, 192, 128, generator=g).half() for _ in range(3))
+    out = simops.attention16(q.reshape(4, 192, 128), k.reshape(4, 192, 128), v.reshape(4, 192, 128))
+    assert rel(out, orc.attention(q, k, v).reshape(4, 192, 128)) <= 2e-2
