@@ -15,6 +15,7 @@ HX_FEATURE_FP8_GEMM_PERSISTENT = 8
 HX_FEATURE_FP8_GEMM_DECODE_RING = 16
 HX_FEATURE_ROUTING_WIDE = 32
 HX_FEATURE_MOE_PERSISTENT = 64
+HX_FEATURE_MATMUL_PERSISTENT = 128
 
 _LIB_PATH = pathlib.Path(__file__).resolve().parent / "libhx_kernels.so"
 _lib = None

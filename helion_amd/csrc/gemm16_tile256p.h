@@ -1,5 +1,5 @@
-// hx_gemm16_tile256p: the grouped (MoE) 256x256x64 16-bit tile kernel as a persistent workgroup (opt-in,
-// HX_FEATURE_MOE_PERSISTENT; not yet run on the hardware).  Same tile, LDS layout, fragment scheme, k-tile schedule and
+// hx_gemm16_tile256p: the 256x256x64 16-bit tile kernel - grouped (MoE) or dense - as a persistent workgroup (opt-in,
+// HX_FEATURE_MOE_PERSISTENT / HX_FEATURE_MATMUL_PERSISTENT; not yet run on the hardware).  Same tile, LDS layout, fragment scheme, k-tile schedule and
 // MFMA order per accumulator as hx_gemm16_tile256<BF, 0> (results bit-equal); what changes is what happens between two
 // tiles of one workgroup, as in hx_fp8_gemm_tile256p:
 //
@@ -30,11 +30,15 @@
 
 // K % 128 == 0 and K >= 256 (an even number of k-tiles, at least four), N % 256 == 0 (the host checks).
 // sink: G16P_SINK_BYTES of device memory, 16-byte aligned, written and never read.
-template <bool BF>
+// DENSE: C = A @ W without the tile table and the row list: row tile t covers rows 256 t .. of A and C, T % 256 == 0 (no row
+// is ever left out, so the sink is not used), tiles_m row tiles; the row tables are filled by the waves themselves.
+// lda, ldb, ldc: row strides of A, W and C in elements (grouped: K, N, N).
+template <bool BF, bool DENSE>
 __global__ __launch_bounds__(256) void hx_gemm16_tile256p(const uint8_t* __restrict__ A, const uint8_t* __restrict__ W,
                                                          void* __restrict__ Cv, const int* __restrict__ num_tiles,
                                                          const MoeTile* __restrict__ table, const int32_t* __restrict__ idx, int T,
-                                                         int K, int N, int tiles_n, int a_div, uint8_t* __restrict__ sink) {
+                                                         int K, int N, int tiles_n, int a_div, uint8_t* __restrict__ sink, long lda,
+                                                         long ldb, long ldc, int tiles_m) {
   typedef typename Mfma16<BF>::T out_t;
   typedef typename Mfma16<BF>::V8 V8;
   __shared__ __attribute__((aligned(1024))) uint8_t smem[2][2][MOE_TILE_BYTES];  // [stage][A|W][32 KB]
@@ -45,10 +49,10 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256p(const uint8_t* __restr
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = w >> 1, wn = w & 1;
   const int nk = K / MOE_BK;
-  const long ldb2 = (long)N * 2, lda2 = (long)K * 2;  // row strides in bytes
+  const long ldb2 = ldb * 2, lda2 = lda * 2, ldc2 = ldc * 2;  // row strides in bytes
 
   // ---- this workgroup's tiles
-  const int total = *num_tiles * tiles_n, nrt = *num_tiles;
+  const int nrt = DENSE ? tiles_m : *num_tiles, total = nrt * tiles_n;
   const int G = (int)gridDim.x, b = (int)blockIdx.x, cpx = G >> 3;
   auto tile_of = [&](int s) {  // tile of step s, or -1
     const int base = s * G, R = total - base;
@@ -64,7 +68,9 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256p(const uint8_t* __restr
   auto tile_info = [&](int tile, MoeTile& mt, int& tn) {
     const int GM = 4, group_size = GM * tiles_n, first_m = (tile / group_size) * GM;
     const int gm = min(nrt - first_m, GM);
-    mt = table[first_m + (tile % group_size) % gm];
+    const int tm = first_m + (tile % group_size) % gm;
+    if (DENSE) mt.expert = 0, mt.row_start = tm * MOE_BM, mt.rows = min(MOE_BM, T - tm * MOE_BM), mt.pad = 0;
+    else mt = table[tm];
     tn = (tile % group_size) / gm;
   };
 
@@ -86,7 +92,8 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256p(const uint8_t* __restr
   // the rows of a tile -> row table `slot`, this wave's 64 of them by one 4-byte DMA instruction (entries past the end of
   // idx re-read its last one; they belong to rows past the tile's count, which are masked wherever the table is read)
   auto fetch_rows = [&](int row_start, int slot) {
-    hx_g2l4_s(idx, (uint32_t)min(row_start + w * 64 + lane, T - 1) * 4u, hx_lds_addr(&rowtab[slot][w * 64]));
+    if (DENSE) rowtab[slot][w * 64 + lane] = row_start + w * 64 + lane;
+    else hx_g2l4_s(idx, (uint32_t)min(row_start + w * 64 + lane, T - 1) * 4u, hx_lds_addr(&rowtab[slot][w * 64]));
   };
   // ---- W DMA: wave w owns k rows [16w, 16w+16), 8 instructions of 2 rows x 512 B (N % 256 == 0: no ragged column tile)
   const int wk_l = lane >> 5, wpos = lane & 31;
@@ -208,7 +215,7 @@ __global__ __launch_bounds__(256) void hx_gemm16_tile256p(const uint8_t* __restr
       const int r = tab[grp * 16 + p * 4];
       const v4i v = *(const v4i*)(&stg[0][0] + L.st_r + p * 1024 + ((L.y0 ^ (4 * p)) * 16));
       const bool ok = (int)L.rb_row < rows - (wm * 128 + grp * 16 + p * 4) && r >= 0 && r < T;
-      const uint8_t* dst = cbase + (long)r * ldb2 + L.rb16;
+      const uint8_t* dst = cbase + (long)r * ldc2 + L.rb16;
       // (non-temporal, as in the plain kernel; rows that are not stored go to the sink so that the instruction is issued anyway)
       __builtin_nontemporal_store(v, (v4i*)(ok ? dst : (const uint8_t*)sink + (L.rb_row * 16 + (L.rb16 >> 4)) * 16));
       if (p & 1) __builtin_amdgcn_sched_barrier(0);

@@ -8,6 +8,7 @@
 // mode computes — is the formula above, and that is what every split count gives here.
 // Anything the tile kernel does not cover (fp32 operands, odd sizes, strided B) runs a plain fp32-FMA kernel.
 #include "gemm16_tile128.h"
+#include "gemm16_tile256p.h"
 
 template <typename T>
 __device__ __forceinline__ float mm_ld(const T* p) { return (float)*p; }
@@ -163,6 +164,14 @@ static void mm_launch_general(const void* a, const void* b, void* c, int64_t M, 
                      (long)lda, (long)ldb_k, (long)ldb_n, (long)ldc, bias, bias_f32, relu);
 }
 
+// The dense 256x256 kernel in persistent workgroups (opt-in, HX_FEATURE_MATMUL_PERSISTENT): a row-major B, no epilogue, a
+// 16-bit output, whole tiles, an even number (at least four) of k-tiles, and at least two tiles for every workgroup.
+static bool mm_persistent_ok(int64_t M, int64_t N, int64_t K, int64_t ldb_n, const void* bias, int relu, int out_dtype, int tile, int splits) {
+  const int64_t grid = (hx_cu_count() / 8) * 8;
+  return hx_feature(HX_FEATURE_MATMUL_PERSISTENT) && tile == 256 && splits == 1 && ldb_n == 1 && !bias && !relu && out_dtype != HX_F32 &&
+         M % MOE_BM == 0 && N % MOE_BN == 0 && K % (2 * MOE_BK) == 0 && K >= 4 * MOE_BK && grid >= 8 && (M / MOE_BM) * (N / MOE_BN) >= 2 * grid;
+}
+
 template <bool BF, bool BCOL>
 static void mm_launch_fast(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k,
                            int64_t ldc, const void* bias, int bias_f32, int relu, int out_dtype, int tile, int splits, void* ws,
@@ -176,7 +185,11 @@ static void mm_launch_fast(const void* a, const void* b, void* c, int64_t M, int
   const bool partial = splits > 1 || (out_dtype == HX_F32 && (bias || relu));
   if (!partial && out_dtype != HX_F32) {
     d.ldc = ldc;
-    if (tile == 256)
+    if (!BCOL && mm_persistent_ok(M, N, K, 1, bias, relu, out_dtype, tile, splits))
+      hx_launch((hx_gemm16_tile256p<BF, true>), dim3((hx_cu_count() / 8) * 8), dim3(256), 0, s, (const uint8_t*)a, (const uint8_t*)b, c,
+                (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M, (int)K, (int)N, tiles_n, 1, (uint8_t*)c, (long)lda,
+                (long)ldb_k, (long)ldc, tiles_m);
+    else if (tile == 256)
       hx_launch((hx_gemm16_tile256<BF, 1, BCOL>), dim3(tiles_m * tiles_n), dim3(256), 0, s, (const uint8_t*)a, (const uint8_t*)b, c,
                          (const int*)nullptr, (const MoeTile*)nullptr, (const int32_t*)nullptr, (int)M, (int)K, (int)N, tiles_m, tiles_n, 1, d);
     else if (tiles_m * tiles_n <= 256)
@@ -218,7 +231,10 @@ static void mm_launch_fast(const void* a, const void* b, void* c, int64_t M, int
 extern "C" int hx_matmul_path(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc, int in_dtype,
                               const void* a, const void* b, const void* c, const void* bias) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
-  return mm_fast_ok(a, b, c, M, N, K, lda, ldb_k, ldb_n, ldc, bias, in_dtype) ? 1 : 0;
+  if (!mm_fast_ok(a, b, c, M, N, K, lda, ldb_k, ldb_n, ldc, bias, in_dtype)) return 0;
+  // 2: the persistent form of the 256x256 kernel (for a call without epilogue, a 16-bit output and the library's own split)
+  const MmPlan plan = mm_plan(M, N, K, 0);
+  return mm_persistent_ok(M, N, K, ldb_n, bias, 0, in_dtype, plan.tile, plan.splits) ? 2 : 1;
 }
 
 extern "C" int hx_matmul(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k,

@@ -296,8 +296,9 @@ static int launch_moe(const void* A, const void* W, void* C, const int32_t* coun
     if (path == 6) {
       const int tiles_n = (int)(N / MOE_BN), grid = (hx_cu_count() / 8) * 8;
       uint8_t* sink = (uint8_t*)(((uintptr_t)flags + (size_t)T + 15) & ~(uintptr_t)15);  // behind the flags (hx_moe_workspace_bytes)
-      hx_launch((hx_gemm16_tile256p<BF>), dim3(grid), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W, (void*)C,
-                (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, tiles_n, (int)a_div, sink);
+      hx_launch((hx_gemm16_tile256p<BF, false>), dim3(grid), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W, (void*)C,
+                (const int*)num_tiles, (const MoeTile*)table, idx, (int)T, (int)K, (int)N, tiles_n, (int)a_div, sink, (long)K, (long)N,
+                (long)N, 0);
     } else if (bm == R32_BM) {
       const int tiles_n = (int)((N + R32_BN - 1) / R32_BN);
       hx_launch((hx_gemm16_rows32<BF, 3>), dim3(max_tiles * tiles_n), dim3(256), 0, s, (const uint8_t*)A, (const uint8_t*)W,

@@ -61,6 +61,9 @@ enum {
                                     separate LDS rings and wave streams for a and b (path 8 where path 5 ran before) */
   HX_FEATURE_ROUTING_WIDE = 32, /* hx_moe_routing with 513..2048 experts (HX_ERR_UNSUPPORTED before): the same kernels with
                                     LDS tables for 2048 experts */
+  HX_FEATURE_MATMUL_PERSISTENT = 128, /* hx_matmul on the 256x256 tile kernel with a row-major b, no epilogue, a 16-bit output,
+                                    M % 256 == 0, N % 256 == 0, K % 128 == 0, K >= 256 and at least two tiles per CU: persistent
+                                    workgroups, as HX_FEATURE_MOE_PERSISTENT (hx_matmul_path 2) */
   HX_FEATURE_MOE_PERSISTENT = 64 /* the grouped GEMM's 256-row tiles (hx_moe_path 3) with N % 256 == 0, K % 128 == 0, K >= 256
                                     in persistent workgroups whose epilogue runs inside the next tile's first k-tile
                                     (hx_moe_path 6); hx_moe_workspace_bytes grows by about 1 KB while it is on */
@@ -238,7 +241,8 @@ size_t hx_fp8_quantize_workspace_bytes(int64_t n);
  * (splits only while the output tiles alone do not fill the chip).  Splits go through fp32 partial sums in the
  * workspace (hx_matmul_workspace_bytes(...) bytes, 16-byte aligned; 0 for one split) and are summed in a fixed order,
  * with the epilogue applied to the whole sum: every split count gives the reference's one-split (eager) result up to
- * fp32 summation order.  hx_matmul_splits tells the split count used; hx_matmul_path 1 = tile kernel, 0 = plain. */
+ * fp32 summation order.  hx_matmul_splits tells the split count used; hx_matmul_path 1 = tile kernel, 0 = plain, 2 = the 256x256
+ * tile kernel in persistent workgroups (opt-in; the answer for a call without epilogue and with the library's own split). */
 int hx_matmul(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k,
               int64_t ldb_n, int64_t ldc, const void* bias, int bias_dtype, int relu, int in_dtype, int out_dtype,
               int split_k, void* workspace, size_t workspace_bytes, void* stream);

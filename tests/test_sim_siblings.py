@@ -112,3 +112,26 @@ def test_quantize_per_tensor(n, dtype):
     rq, rs = orc.fp8_quantize_per_tensor(x)
     assert float(scale) == float(rs)
     assert torch.equal(q.view(torch.uint8), rq.view(torch.uint8))
+
+
+# ---- opt-in: the dense 256x256 kernel in persistent workgroups (HX_FEATURE_MATMUL_PERSISTENT, hx_matmul_path 2) -------------
+@pytest.mark.parametrize("m,n,k,cus,variant,dtype", [(3072, 3072, 256, 8, "lazy", torch.bfloat16),
+                                                     (2304, 4096, 384, 16, "eager-interleaved", torch.float16)])
+def test_persistent_dense_matmul(m, n, k, cus, variant, dtype):
+    """144 tiles on 8 / 16 persistent workgroups: every tile's epilogue runs inside the next tile's first k-tile.  Bit-equal
+    to the kernel it replaces (same MFMA order per accumulator)."""
+    from helion_amd import _lib
+    g = torch.Generator().manual_seed(m + k)
+    x = (torch.randn(m, k, generator=g) * 0.5).to(dtype)
+    y = (torch.randn(k, n, generator=g) * 0.5).to(dtype)
+    simlib.configure(variant)
+    with simlib.cus(cus):
+        base = simops.matmul(x, y, want_path=1)
+        with simlib.features(_lib.HX_FEATURE_MATMUL_PERSISTENT):
+            simlib.work()
+            out = simops.matmul(x, y, want_path=2)
+            w = simlib.work()
+            assert simlib.load().hx_matmul_path(m, n + 8, k, k, n + 8, 1, n + 8, _lib.HX_BF16, None, None, None, None) == 1  # ragged column tile
+    assert torch.equal(out.view(torch.int16), base.view(torch.int16))
+    assert rel_err(out, orc.matmul(x, y)) <= 1e-2
+    assert w["workgroups"] == cus and w["mfma"] == (m // 256) * (n // 256) * (k // 64) * 512

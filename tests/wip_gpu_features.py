@@ -177,3 +177,26 @@ def test_persistent_grouped_gemm(moe_persistent, T, K, N, E, dtype):
     rows = torch.arange(0, T, 997, device=DEV)
     ref = orc.moe_matmul_ogs_reference(A[rows].cpu(), W.cpu(), ex[rows].cpu())
     assert rel_err(out[rows].cpu(), ref) <= 1e-2
+
+
+@pytest.fixture
+def matmul_persistent():
+    old = hx.set_features(hx.HX_FEATURE_MATMUL_PERSISTENT)
+    yield
+    hx.set_features(old)
+
+
+@pytest.mark.parametrize("m,n,k,dtype", [(8192, 8192, 256, torch.bfloat16), (8192, 16384, 384, torch.float16), (8192, 8192, 8192, torch.bfloat16)])
+def test_persistent_dense_matmul(matmul_persistent, m, n, k, dtype):
+    """Bit-equal to the default 256x256 kernel; a sample of rows against the oracle."""
+    g = torch.Generator().manual_seed(m + k)
+    x = (torch.randn(m, k, generator=g) * 0.5).to(dtype).to(DEV)
+    y = (torch.randn(k, n, generator=g) * 0.5).to(dtype).to(DEV)
+    assert _lib.load().hx_matmul_path(m, n, k, k, n, 1, n, _lib.HX_BF16, x.data_ptr(), y.data_ptr(), x.data_ptr(), None) == 2
+    print(f"persistent dense case M={m} N={n} K={k} {dtype}", flush=True)
+    out = hx.matmul(x, y)
+    hx.set_features(0)
+    base = hx.matmul(x, y)
+    assert torch.equal(out.view(torch.int16), base.view(torch.int16))
+    rows = torch.arange(0, m, 509, device=DEV)
+    assert rel_err(out[rows].cpu(), orc.matmul(x[rows].cpu(), y.cpu())) <= 1e-2
