@@ -215,6 +215,14 @@ def _traffic(name):
     return None, None
 
 
+def _features():
+    try:
+        from helion_amd import _lib
+        return int(_lib.load().hx_get_features())
+    except Exception:  # noqa: BLE001
+        return None
+
+
 def _counters(name):
     """Engine clock and matrix-pipe occupancy of a kernel from hardware counters: a recorded profile value like _traffic's,
     read from the line `kernel_counters <name> <clock_mhz> <mfma_busy> <digest> <source files...>` of the counter summary
@@ -745,7 +753,10 @@ def main():
                                "fp32 accumulate, bf16 out",
                    "device": _DEV.get("market_name") or f"{props.gcnArchName.split(':')[0]} ({props.name})",
                    "device_arch": props.gcnArchName, "compute_units": _DEV.get("compute_units"),
-                   "max_engine_clock_mhz": _DEV.get("max_engine_clock_mhz")},
+                   "max_engine_clock_mhz": _DEV.get("max_engine_clock_mhz"),
+                   # opt-in kernel paths switched on for this run (HX_FEATURES / helion_amd.set_features; 0 = the default
+                   # kernels, which is what every "kernel" label in this line names)
+                   "opt_in_features": _features()},
         "roofline": roof,
         "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(),
         "parity_and_oracle_times": None if args.no_cpu_baseline else cpu_checks(),
