@@ -201,3 +201,14 @@ def test_persistent_grouped_kernel_is_chosen_only_for_whole_column_tiles_and_eve
             assert path(6144, 256, 2176, 2) == 3              # a ragged last column tile
             assert path(1024, 256, 2048, 8) == 2              # small experts keep the 128-row tiles
             assert lib.hx_moe_workspace_bytes(6144, 2) >= 1024 + 6144
+
+
+def test_persistent_grouped_kernel_through_the_top_k_entry():
+    """a_div = 2: C row r is the product of A row r / 2; routing on the device, the sink inside the top-k workspace."""
+    from helion_amd import _lib
+    A, W, ex = inputs.moe_inputs(3072, 256, 2048, 2, 2, seed=9, dtype=torch.bfloat16)
+    simlib.configure("lazy-reverse")
+    with simlib.cus(8), simlib.features(_lib.HX_FEATURE_MOE_PERSISTENT):
+        assert simlib.load().hx_moe_path(6144, 256, 2048, 2, 2, None, None, None) == 6
+        out = simops.moe_topk(A[::2].contiguous(), W, ex, 2)
+    assert rel_err(out, orc.moe_matmul_ogs_reference(A, W, ex)) <= 1e-2
