@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only c2,lib,c3,c4,c5,next,sib[,lib16]] [--no-cpu-baseline] [--clock-probe]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only c2,lib,c3,c4,c5,next,sib[,lib16][,optin]] [--no-cpu-baseline] [--clock-probe]
 
 A "step" is one launch of the FP8 GEMM at the headline configuration (M=N=K=8192, e4m3 operands, B column-major,
 per-tensor fp32 scales, bf16 output) with inputs resident in HBM.
@@ -593,6 +593,83 @@ def bench_siblings(steps, warmup):
     return out
 
 
+def bench_opt_in(steps, warmup):
+    """`--only optin` (not part of the default run): each opt-in kernel path against the default kernel on the same
+    operands, in one process.  A path is timed only after its output has been compared with the default kernel's - bit for
+    bit where the two run the same MFMA order, within the parity tolerance otherwise; a mismatch is reported instead of a
+    time.  Every row restores the feature mask it found."""
+    import torch
+    import helion_amd as hx
+    from helion_amd import inputs
+
+    out = {}
+
+    def compare(key, mask, fn, exact, what, timed=None):
+        """fn: the call whose outputs are compared; timed: the call that is timed (fn itself if None)."""
+        old = hx.set_features(0)
+        try:
+            ref = fn()
+            hx.set_features(mask)
+            got = fn()
+            torch.cuda.synchronize()
+            if exact:
+                same = bool(torch.equal(got.view(torch.uint8), ref.view(torch.uint8)))
+            else:
+                same = float((got.float() - ref.float()).abs().max() / ref.float().abs().max()) <= 1e-2
+            row = {"workload": what, "feature_mask": mask, "check": "bit-equal to the default kernel" if exact else "max|err| <= 1e-2 max|ref| of the default kernel",
+                   "check_passed": same}
+            del ref, got
+            if same:
+                hx.set_features(0)
+                t0 = _time_launches(timed or fn, steps, warmup)
+                hx.set_features(mask)
+                t1 = _time_launches(timed or fn, steps, warmup)
+                row.update({"default_ms": t0["median_ms"], "opt_in_ms": t1["median_ms"], "speedup": t0["median_ms"] / t1["median_ms"]})
+            out[key] = row
+        except Exception as e:  # noqa: BLE001
+            out[key + "_error"] = f"{type(e).__name__}: {e}"[:400]
+        finally:
+            hx.set_features(old)
+            torch.cuda.empty_cache()
+
+    a, b, sa, sb = inputs.gemm_c2("cuda")
+    compare("c2_persistent", hx.HX_FEATURE_FP8_GEMM_PERSISTENT, lambda: hx.fp8_gemm(a, b, scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16), True,
+            "C2 fp8_gemm 8192^3: hx_fp8_gemm_tile256p against hx_fp8_gemm_tile256")
+    del a, b
+    # decode rows: weight matrices rotated so that every launch streams from HBM
+    bufs = [(torch.randn(28672, 8192, device="cuda") * 0.5).to(torch.float8_e4m3fn).t() for _ in range(4)]
+    turn = [0]
+    for rows in (64, 128):
+        xr = (torch.randn(rows, 8192, device="cuda") * 0.5).to(torch.float8_e4m3fn)
+
+        def decode(xr=xr):
+            turn[0] = (turn[0] + 1) % len(bufs)
+            return hx.fp8_gemm(xr, bufs[turn[0]], out_dtype=torch.bfloat16)
+
+        def decode_fixed(xr=xr):  # (one buffer for the comparison)
+            return hx.fp8_gemm(xr, bufs[0], out_dtype=torch.bfloat16)
+
+        compare(f"decode_m{rows}", hx.HX_FEATURE_FP8_GEMM_DECODE_RING, decode_fixed, True,
+                f"fp8_gemm M{rows} N28672 K8192 bf16 out: hx_fp8_gemm_decode_ring against hx_fp8_gemm_tileN128 (compared on one weight "
+                "buffer, timed over 4 rotating ones: HBM-cold)", timed=decode)
+    x16 = (torch.randn(16, 8192, device="cuda") * 0.5).to(torch.float8_e4m3fn)
+    yrm = bufs[0].contiguous()  # [K, N] row-major: the layout the reference's own check feeds
+    compare("c3_rowmajor_y", hx.HX_FEATURE_SKINNY_ROWMAJOR, lambda: hx.fp8_gemm(x16, yrm, out_dtype=torch.bfloat16), False,
+            "C3 with a row-major y: hx_fp8_gemm_skinny_rm in place against transpose-through-the-workspace + hx_fp8_gemm_skinny_direct")
+    del bufs, x16, yrm
+    A, W, ex = inputs.moe_c5("cuda")
+    args = hx.moe_matmul_ogs_helion_kernel_args_gen(A, W, ex)
+    compare("c5_persistent", hx.HX_FEATURE_MOE_PERSISTENT, lambda: hx.moe_matmul_ogs(*args), True,
+            "C5 moe_matmul_ogs: hx_gemm16_tile256p<grouped> against hx_gemm16_tile256<grouped>")
+    del A, W, ex, args
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn(8192, 8192, device="cuda", generator=g).to(torch.bfloat16)
+    y = torch.randn(8192, 8192, device="cuda", generator=g).to(torch.bfloat16)
+    compare("matmul_bf16_persistent", hx.HX_FEATURE_MATMUL_PERSISTENT, lambda: hx.matmul(x, y), True,
+            "matmul 8192^3 bf16 without epilogue: hx_gemm16_tile256p<dense> against hx_gemm16_tile256<dense>")
+    return out
+
+
 # ----------------------------------------------------------------------------------------------------------------
 # the CPU leg: the ref-eager baseline, the oracle's wall times, and the kernels' measured error against the oracle
 # ----------------------------------------------------------------------------------------------------------------
@@ -742,6 +819,8 @@ def main():
         section("next_rows", bench_next_rows, merge=True)
     if "sib" in only:
         section("siblings", bench_siblings, merge=True)
+    if "optin" in only:  # opt-in: the opt-in kernel paths against the default kernels (not in the default run)
+        section("opt_in_paths", bench_opt_in, merge=True)
     if "lib16" in only:  # opt-in: vendor-library rows for the 16-bit GEMMs
         section("library_baselines_16bit", bench_16bit_library_baselines)
     line = {
