@@ -639,7 +639,7 @@ def bench_opt_in(steps, warmup):
     # decode rows: weight matrices rotated so that every launch streams from HBM
     bufs = [(torch.randn(28672, 8192, device="cuda") * 0.5).to(torch.float8_e4m3fn).t() for _ in range(4)]
     turn = [0]
-    for rows in (64, 128):
+    for rows in (64, 128, 160, 256):
         xr = (torch.randn(rows, 8192, device="cuda") * 0.5).to(torch.float8_e4m3fn)
 
         def decode(xr=xr):

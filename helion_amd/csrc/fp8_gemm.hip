@@ -1060,11 +1060,13 @@ static bool tile256p_ok(int64_t M, int64_t N, int64_t K) {
   return hx_feature(HX_FEATURE_FP8_GEMM_PERSISTENT) && K % 256 == 0 && K >= 512 && grid >= 8 && tiles >= 2 * grid;
 }
 
-// decode batches of 33..128 rows on the kernel with separate A / B rings (opt-in: HX_FEATURE_FP8_GEMM_DECODE_RING), where
+// decode batches of 33..256 rows on the kernel with separate A / B rings (opt-in: HX_FEATURE_FP8_GEMM_DECODE_RING), where
 // hx_fp8_gemm_tileN128 runs otherwise (path 5 becomes 8)
 static bool decode_ring_ok(int64_t M, int64_t N, int64_t K) {
-  return hx_feature(HX_FEATURE_FP8_GEMM_DECODE_RING) && M > 32 && M <= 128 && tileN128_rows(M, N, K) <= 128;
+  return hx_feature(HX_FEATURE_FP8_GEMM_DECODE_RING) && M > 32 && M <= 256 && tileN128_rows(M, N, K) != 0;
 }
+// its row tile: 64, 128, 192 or 256 rows
+static int decode_ring_rows(int64_t M) { return M <= 64 ? 64 : M <= 128 ? 128 : M <= 192 ? 192 : 256; }
 
 extern "C" int hx_fp8_gemm_path(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
                                 const void* a, const void* b, const void* c) {
@@ -1108,9 +1110,15 @@ static void launch_decode_ring(int bm, bool b_read_once, dim3 grid, hipStream_t 
   if (bm == 64) {
     if (b_read_once) hx_launch((hx_fp8_gemm_decode_ring<OUT, 64, true, true>), grid, dim3(256), 0, stream, args...);
     else hx_launch((hx_fp8_gemm_decode_ring<OUT, 64, true, false>), grid, dim3(256), 0, stream, args...);
-  } else {
+  } else if (bm == 128) {
     if (b_read_once) hx_launch((hx_fp8_gemm_decode_ring<OUT, 128, false, true>), grid, dim3(256), 0, stream, args...);
     else hx_launch((hx_fp8_gemm_decode_ring<OUT, 128, false, false>), grid, dim3(256), 0, stream, args...);
+  } else if (bm == 192) {
+    if (b_read_once) hx_launch((hx_fp8_gemm_decode_ring<OUT, 192, false, true>), grid, dim3(256), 0, stream, args...);
+    else hx_launch((hx_fp8_gemm_decode_ring<OUT, 192, false, false>), grid, dim3(256), 0, stream, args...);
+  } else {
+    if (b_read_once) hx_launch((hx_fp8_gemm_decode_ring<OUT, 256, false, true>), grid, dim3(256), 0, stream, args...);
+    else hx_launch((hx_fp8_gemm_decode_ring<OUT, 256, false, false>), grid, dim3(256), 0, stream, args...);
   }
 }
 
@@ -1173,7 +1181,7 @@ static void launch_kmajor(int path, const void* a, const void* bt, void* c, int6
     if (split) {
       float* part = (float*)ws;
       if (decode_ring_ok(M, N, K))
-        launch_decode_ring<HX_F32>(bm, b_once, grid, stream, (const uint8_t*)a, (const uint8_t*)bt, part, (int)M, (int)N, (int)K, (long)lda,
+        launch_decode_ring<HX_F32>(decode_ring_rows(M), b_once, grid, stream, (const uint8_t*)a, (const uint8_t*)bt, part, (int)M, (int)N, (int)K, (long)lda,
                                    (long)ldb, (long)N, (const float*)nullptr, (const float*)nullptr, bn, ktps);
       else if (bm == 64)
         launch_tileN128<HX_F32, 64, true>(b_once, grid, stream, (const uint8_t*)a, (const uint8_t*)bt,
@@ -1188,7 +1196,7 @@ static void launch_kmajor(int path, const void* a, const void* bt, void* c, int6
       hx_launch((hx_fp8_gemm_split_reduce<OUT>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream,
                          (const float*)part, (out_t*)c, (int)M, (int)N, (long)ldc, splits, sa, sb);
     } else if (decode_ring_ok(M, N, K)) {
-      launch_decode_ring<OUT>(bm, b_once, grid, stream, (const uint8_t*)a, (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda,
+      launch_decode_ring<OUT>(decode_ring_rows(M), b_once, grid, stream, (const uint8_t*)a, (const uint8_t*)bt, (out_t*)c, (int)M, (int)N, (int)K, (long)lda,
                               (long)ldb, (long)ldc, sa, sb, bn, 0);
     } else if (bm == 64) {
       launch_tileN128<OUT, 64, true>(b_once, grid, stream, (const uint8_t*)a, (const uint8_t*)bt,

@@ -1,4 +1,4 @@
-// hx_fp8_gemm_decode_ring: the FP8 GEMM for a decode batch of 33..128 rows against a wide column-major weight matrix
+// hx_fp8_gemm_decode_ring: the FP8 GEMM for a decode batch of 33..256 rows against a wide column-major weight matrix
 // (B^T rows of K): one row tile, so the kernel is a weight-streaming loop bound by HBM, and what decides its speed is how
 // many weight bytes every CU keeps in flight.
 //
@@ -6,11 +6,13 @@
 // results are the same bit for bit), but A and B have rings of their own in the LDS and wave streams of their own:
 //   * waves 0 and 1 issue all DMA of A (BM x 128 bytes per k-tile; the same few rows for every workgroup, so L2 hits with
 //     a short latency): a ring of 3 stages is enough;
-//   * waves 2 and 3 issue all DMA of B (128 columns x 128 bytes per k-tile, from HBM): a ring of 7 (BM = 128) or 8 (BM = 64)
-//     stages of 16 KB, so five to seven stages - 80 to 112 KB per CU - are in flight while one is consumed.
+//   * waves 2 and 3 issue all DMA of B (128 columns x 128 bytes per k-tile, from HBM): a ring of 8 / 7 / 5 / 4 stages of
+//     16 KB for BM = 64 / 128 / 192 / 256 (whatever the A ring leaves of the 160 KB), so that six / five / three / two of
+//     them are in flight while one is consumed and one is being refilled.
 // A wave's vmcnt counts only its own instructions and they complete in order, so a single stream carrying both operands
 // would tie B's depth to A's: waiting for a recently issued A tile would also wait for every B tile issued before it.
-// With one stage ring for both (tileN128) the 128-row tile has two to three B stages in flight (32 - 48 KB per CU).
+// With one stage ring for both (tileN128) the 128-row tile has two to three B stages in flight (32 - 48 KB per CU) and the
+// 256-row tile one to two.  BM = 192 exists only here: 129..192 rows do three quarters of the 256-row tile's MFMAs.
 // PAIR (BM = 64): the B waves issue two consecutive k-tiles together at every other step, row piece by row piece, so
 // that memory sees 256 contiguous bytes of a weight row back to back.
 // All four waves multiply; the barrier at the top of a step makes both streams' landed tiles visible to everybody.
@@ -28,13 +30,13 @@ __global__ __launch_bounds__(256) void hx_fp8_gemm_decode_ring(const uint8_t* __
                                                               long ldb, long ldc, const float* __restrict__ scale_a,
                                                               const float* __restrict__ scale_b, int bn, int kt_per_split) {
   typedef typename OutT<OUT>::T out_t;
-  static_assert(BM == 64 || BM == 128, "one row tile of 64 or 128 rows");
+  static_assert(BM == 64 || BM == 128 || BM == 192 || BM == 256, "one row tile of 64, 128, 192 or 256 rows");
   constexpr int BK = 128;
-  constexpr int NA = 3, NB = BM == 64 ? 8 : 7;
+  constexpr int NA = 3, NB = BM == 64 ? 8 : BM == 128 ? 7 : BM == 192 ? 5 : 4;
   static_assert(!PAIR || NB % 2 == 0, "pairs of k-tiles need an even ring");
   constexpr int ASTAGE = BM * 128, BSTAGE = 128 * 128;
   constexpr int WMB = BM / 32;  // 16-row blocks per wave
-  __shared__ __attribute__((aligned(1024))) uint8_t smem[NA * ASTAGE + NB * BSTAGE];  // BM 64: 152 KB, BM 128: 160 KB
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[NA * ASTAGE + NB * BSTAGE];  // 152 / 160 / 152 / 160 KB
   const int kt0 = kt_per_split * (int)blockIdx.y;
   const int nk = kt_per_split ? min(kt_per_split, K / BK - kt0) : K / BK;
   const uint8_t* A = A_ + (long)kt0 * BK;

@@ -57,7 +57,7 @@ enum {
   HX_FEATURE_FP8_GEMM_PERSISTENT = 8, /* hx_fp8_gemm on the 256x256 tile kernel with at least two tiles per CU, K % 256 == 0
                                     and a 16-bit output: persistent workgroups whose epilogue runs inside the next tile's
                                     first k-tile (path 7) */
-  HX_FEATURE_FP8_GEMM_DECODE_RING = 16, /* hx_fp8_gemm with 33..128 rows and a column-major b: the weight-streaming kernel with
+  HX_FEATURE_FP8_GEMM_DECODE_RING = 16, /* hx_fp8_gemm with 33..256 rows and a column-major b: the weight-streaming kernel with
                                     separate LDS rings and wave streams for a and b (path 8 where path 5 ran before) */
   HX_FEATURE_ROUTING_WIDE = 32, /* hx_moe_routing with 513..2048 experts (HX_ERR_UNSUPPORTED before): the same kernels with
                                     LDS tables for 2048 experts */
@@ -83,7 +83,7 @@ unsigned hx_get_features(void);
  *    1.0, helion/language/matmul_ops.py:232-233).
  * hx_fp8_gemm_path: 0 plain kernel (or a row-major b transposed through the workspace), 1 256x256 tiles, 2 decode kernel,
  * 3 256x256 tiles with guarded edges / K tail, 4 256x256 tiles on a row-major b, 5 128-column tiles, 6 decode kernel on a
- * row-major b (opt-in), 7 256x256 tiles in persistent workgroups (opt-in), 8 decode batch of 33..128 rows with separate
+ * row-major b (opt-in), 7 256x256 tiles in persistent workgroups (opt-in), 8 decode batch of 33..256 rows with separate
  * a / b rings (opt-in).
  * Chooses between the 256x256 MFMA tile kernel (with guarded edge tiles when M or N is ragged or K is not a multiple
  * of 128 — K % 16 == 0 suffices, the last k-tile is zero-padded in LDS; it reads a column-major B directly and a

@@ -286,7 +286,7 @@ def test_persistent_kernel_is_chosen_only_where_every_workgroup_gets_two_tiles()
         assert lib.hx_fp8_gemm_path(1024, 1024, 512, 512, 1, 512, 1024, None, None, None) != 7  # off by default
 
 
-# ---- opt-in: decode batches of 33..128 rows with separate A / B rings (HX_FEATURE_FP8_GEMM_DECODE_RING) ---------------------
+# ---- opt-in: decode batches of 33..256 rows with separate A / B rings (HX_FEATURE_FP8_GEMM_DECODE_RING) ---------------------
 def _decode_ring(m, n, k, variant, od=torch.bfloat16, **kw):
     from helion_amd import _lib
     a, y = _ops(m, n, k, 11 + m + n + k, False)
@@ -301,7 +301,8 @@ def _decode_ring(m, n, k, variant, od=torch.bfloat16, **kw):
 
 
 @pytest.mark.parametrize("variant", ALL)
-@pytest.mark.parametrize("m", [64, 128])   # 64: B waves issue pairs of k-tiles into a ring of 8; 128: single k-tiles into a ring of 7
+# 64: B waves issue pairs of k-tiles into a ring of 8; 128 / 192 / 256: single k-tiles into a ring of 7 / 5 / 4 (192: a tile only this kernel has)
+@pytest.mark.parametrize("m", [64, 128, 192, 256])
 def test_decode_ring_kernel_every_variant(variant, m):
     out, base, ref, _ = _decode_ring(m, 256, 2560, variant)   # 20 k-tiles: every ring wraps at least twice
     assert torch.equal(out.view(torch.int16), base.view(torch.int16))  # same MFMA order as the kernel it replaces
@@ -316,6 +317,10 @@ def test_decode_ring_kernel_every_variant(variant, m):
     (65, 112, 1280, torch.bfloat16),
     (128, 1792, 1024, torch.bfloat16),
     (96, 128, 8192, torch.bfloat16),    # 64 k-tiles in 8 splits
+    (130, 256, 1024, torch.bfloat16),   # 192-row tile, 62 rows of padding
+    (160, 144, 128, torch.float16),     # 192-row tile, a single k-tile
+    (200, 640, 512, torch.bfloat16),    # 256-row tile
+    (256, 384, 2048, torch.float32),
 ])
 def test_decode_ring_kernel_shapes(m, n, k, od):
     for variant in FAST:

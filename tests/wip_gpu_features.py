@@ -116,7 +116,8 @@ def decode_ring():
 
 @pytest.mark.parametrize("m,n,k,od", [(33, 100, 128, torch.bfloat16), (64, 256, 2560, torch.bfloat16), (128, 256, 2560, torch.float16),
                                       (100, 640, 512, torch.float32), (40, 512, 1024, torch.bfloat16), (96, 128, 8192, torch.bfloat16),
-                                      (64, 28672, 8192, torch.bfloat16), (128, 28672, 8192, torch.bfloat16)])
+                                      (64, 28672, 8192, torch.bfloat16), (128, 28672, 8192, torch.bfloat16), (130, 256, 1024, torch.bfloat16),
+                                      (200, 640, 512, torch.float16), (160, 28672, 8192, torch.bfloat16), (256, 28672, 8192, torch.bfloat16)])
 def test_decode_ring_kernel(decode_ring, m, n, k, od):
     """Bit-equal to the kernel it replaces (hx_fp8_gemm_tileN128: same MFMA order), and within tolerance of the oracle."""
     g = torch.Generator().manual_seed(m + n + k)
