@@ -16,6 +16,7 @@ HX_FEATURE_FP8_GEMM_DECODE_RING = 16
 HX_FEATURE_ROUTING_WIDE = 32
 HX_FEATURE_MOE_PERSISTENT = 64
 HX_FEATURE_MATMUL_PERSISTENT = 128
+HX_FEATURE_MOE_ANY_SHAPE = 256
 
 _LIB_PATH = pathlib.Path(__file__).resolve().parent / "libhx_kernels.so"
 _lib = None
@@ -50,6 +51,7 @@ _SIGNATURES = {
          _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int, _c.c_void_p, _c.c_size_t, _c.c_void_p],
     ),
     "hx_moe_workspace_bytes": (_c.c_size_t, [_c.c_int64, _c.c_int64]),
+    "hx_moe_workspace_bytes_shape": (_c.c_size_t, [_c.c_int64] * 4),
     "hx_moe_grouped_gemm_static": (
         _c.c_int,
         [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int64,

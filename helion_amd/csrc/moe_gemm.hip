@@ -340,6 +340,57 @@ static int launch_moe(const void* A, const void* W, void* C, const int32_t* coun
   return 0;
 }
 
+// ------------------------------------------------------------------------------------------
+// Any K, any N through the MFMA kernels (opt-in, HX_FEATURE_MOE_ANY_SHAPE): an odd K leaves the rows of A only 2-byte
+// aligned and N % 8 != 0 those of W and C, which no DMA instruction can fetch - such calls ran the fp32-FMA kernel.  With
+// room in the workspace the operands are copied once into 16-byte-friendly form, zero-padded (zeros add nothing to a dot
+// product): A as [rows][K8], W as [E][K8][N8] with K8 / N8 the next multiples of 8, and, when N itself is padded, C as
+// [T][N8] with a crop back afterwards.  Cost: one read and write of A and W (and C) against 2 T K N flops.
+// ------------------------------------------------------------------------------------------
+// dst[b][r][c] = src[b][r][c] inside rows x cols, 0 in the padding; 16-bit elements; one work-item per 8 elements of dst
+__global__ __launch_bounds__(256) void hx_pad2d_u16(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst, int rows, int cols,
+                                                   int drows, int dcols, long n_chunks) {
+  const long id = (long)blockIdx.x * 256 + threadIdx.x;
+  if (id >= n_chunks) return;
+  const int cpr = dcols / 8;
+  const long br = id / cpr;  // batch * drows + row
+  const int c0 = (int)(id % cpr) * 8, r = (int)(br % drows);
+  const long b = br / drows;
+  uint16_t v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = (r < rows && c0 + i < cols) ? src[(b * rows + r) * (long)cols + c0 + i] : (uint16_t)0;
+  *(v4i*)(dst + (br * dcols + c0)) = *(const v4i*)v;
+}
+// dst[r][c] = src[r][c] for c < cols; src rows are scols apart
+__global__ __launch_bounds__(256) void hx_crop2d_u16(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst, long rows, int cols, int scols) {
+  const long id = (long)blockIdx.x * 256 + threadIdx.x;
+  if (id >= rows * cols) return;
+  dst[id] = src[(id / cols) * scols + id % cols];
+}
+
+static bool moe_repack_wanted(int64_t K, int64_t N) { return hx_feature(HX_FEATURE_MOE_ANY_SHAPE) && K >= 1 && N >= 1 && (K % 2 != 0 || N % 8 != 0); }
+static inline size_t up256(size_t b) { return (b + 255) & ~(size_t)255; }
+struct MoeRepack {
+  int64_t K8, N8, rows_a;
+  size_t a_off, w_off, c_off, total;  // byte offsets in the workspace behind the plain layout; c_off == 0: C is written in place
+};
+static MoeRepack moe_repack_plan(int64_t T, int64_t K, int64_t N, int64_t E, int64_t a_div) {
+  MoeRepack r;
+  r.K8 = (K + 7) & ~(int64_t)7, r.N8 = (N + 7) & ~(int64_t)7, r.rows_a = (T + a_div - 1) / a_div;
+  r.a_off = up256(hx_moe_workspace_bytes(T, E));
+  r.w_off = r.a_off + up256((size_t)r.rows_a * r.K8 * 2);
+  const size_t end_w = r.w_off + up256((size_t)E * r.K8 * r.N8 * 2);
+  r.c_off = N % 8 != 0 ? end_w : 0;
+  r.total = N % 8 != 0 ? end_w + up256((size_t)T * r.N8 * 2) : end_w;
+  return r;
+}
+
+extern "C" size_t hx_moe_workspace_bytes_shape(int64_t T, int64_t K, int64_t N, int64_t E) {
+  if (T < 0 || K < 0 || N < 0 || E < 0) return 0;
+  if (!moe_repack_wanted(K, N) || T == 0) return hx_moe_workspace_bytes(T, E);
+  return moe_repack_plan(T, K, N, E, 1).total;
+}
+
 extern "C" int hx_moe_grouped_gemm(const void* A, const void* W, void* C, const int32_t* counts, const int32_t* offsets,
                                    const int32_t* idx, int64_t T, int64_t K, int64_t N, int64_t E, int64_t max_T, int dtype,
                                    void* workspace, size_t workspace_bytes, void* stream) {
@@ -366,6 +417,30 @@ extern "C" int hx_moe_grouped_gemm(const void* A, const void* W, void* C, const 
     return HX_ERR_WORKSPACE;
   }
   hipStream_t s = (hipStream_t)stream;
+  if (moe_repack_wanted(K, N) && E > 0) {
+    const MoeRepack rp = moe_repack_plan(T, K, N, E, 1);
+    if (workspace_bytes >= rp.total && (size_t)rp.rows_a * rp.K8 * 2 < (1ULL << 32)) {
+      uint8_t* base = (uint8_t*)workspace;
+      uint16_t* a2 = (uint16_t*)(base + rp.a_off);
+      uint16_t* w2 = (uint16_t*)(base + rp.w_off);
+      uint16_t* c2 = rp.c_off ? (uint16_t*)(base + rp.c_off) : (uint16_t*)C;
+      const long ca = (long)rp.rows_a * (rp.K8 / 8), cw = (long)E * rp.K8 * (rp.N8 / 8);
+      hx_launch(hx_pad2d_u16, dim3((unsigned)((ca + 255) / 256)), dim3(256), 0, s, (const uint16_t*)A, a2, (int)rp.rows_a, (int)K, (int)rp.rows_a,
+                (int)rp.K8, ca);
+      hx_launch(hx_pad2d_u16, dim3((unsigned)((cw + 255) / 256)), dim3(256), 0, s, (const uint16_t*)W, w2, (int)K, (int)N, (int)rp.K8, (int)rp.N8, cw);
+      const int rc = dtype == HX_BF16 ? launch_moe<true>(a2, w2, c2, counts, offsets, idx, T, rp.K8, rp.N8, E, 1, workspace, s)
+                                      : launch_moe<false>(a2, w2, c2, counts, offsets, idx, T, rp.K8, rp.N8, E, 1, workspace, s);
+      if (rc != 0 || !rp.c_off) return rc;
+      const long n = (long)T * N;
+      hx_launch(hx_crop2d_u16, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (const uint16_t*)c2, (uint16_t*)C, (long)T, (int)N, (int)rp.N8);
+      const hipError_t e = hx_launch_status();
+      if (e != hipSuccess) {
+        hx_set_error("hx_moe_grouped_gemm: launch failed: %s", hipGetErrorString(e));
+        return (int)e;
+      }
+      return 0;
+    }
+  }
   if (dtype == HX_BF16) return launch_moe<true>(A, W, C, counts, offsets, idx, T, K, N, E, 1, workspace, s);
   return launch_moe<false>(A, W, C, counts, offsets, idx, T, K, N, E, 1, workspace, s);
 }

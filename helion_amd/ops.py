@@ -161,7 +161,7 @@ def _moe_matmul_ogs_impl(A: torch.Tensor, W: torch.Tensor, expert_token_counts: 
     if T == 0 or N == 0:
         return C
     lib = _lib.load()
-    ws_bytes = lib.hx_moe_workspace_bytes(T, E)
+    ws_bytes = lib.hx_moe_workspace_bytes_shape(T, K, N, E)  # (= hx_moe_workspace_bytes(T, E) unless an opt-in path wants more)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=A.device)
     rc = lib.hx_moe_grouped_gemm(A.data_ptr(), W.data_ptr(), C.data_ptr(), counts.data_ptr(), offsets.data_ptr(),
                                  idx.data_ptr(), T, K, N, E, max_T_per_expert, _DT[dtype], ws.data_ptr(), ws_bytes,

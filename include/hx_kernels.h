@@ -64,9 +64,13 @@ enum {
   HX_FEATURE_MATMUL_PERSISTENT = 128, /* hx_matmul on the 256x256 tile kernel with a row-major b, no epilogue, a 16-bit output,
                                     M % 256 == 0, N % 256 == 0, K % 128 == 0, K >= 256 and at least two tiles per CU: persistent
                                     workgroups, as HX_FEATURE_MOE_PERSISTENT (hx_matmul_path 2) */
-  HX_FEATURE_MOE_PERSISTENT = 64 /* the grouped GEMM's 256-row tiles (hx_moe_path 3) with N % 256 == 0, K % 128 == 0, K >= 256
+  HX_FEATURE_MOE_PERSISTENT = 64, /* the grouped GEMM's 256-row tiles (hx_moe_path 3) with N % 256 == 0, K % 128 == 0, K >= 256
                                     in persistent workgroups whose epilogue runs inside the next tile's first k-tile
                                     (hx_moe_path 6); hx_moe_workspace_bytes grows by about 1 KB while it is on */
+  HX_FEATURE_MOE_ANY_SHAPE = 256 /* hx_moe_grouped_gemm with an odd K or N % 8 != 0 and a workspace of
+                                    hx_moe_workspace_bytes_shape(T, K, N, E) bytes: the operands are copied once into it,
+                                    zero-padded to multiples of 8, and the MFMA kernels run on the copies where the fp32
+                                    kernel ran before (hx_moe_path still answers 0 for such a call) */
 };
 unsigned hx_set_features(unsigned mask);
 unsigned hx_get_features(void);
@@ -164,6 +168,9 @@ int hx_moe_grouped_gemm(const void* A, const void* W, void* C, const int32_t* co
                         int64_t E, int64_t max_T, int dtype, void* workspace, size_t workspace_bytes,
                         void* stream);
 size_t hx_moe_workspace_bytes(int64_t T, int64_t E);
+/* The same, plus room for the padded copies of HX_FEATURE_MOE_ANY_SHAPE when that feature is on and the shape needs them
+ * (otherwise equal to hx_moe_workspace_bytes(T, E)).  No counterpart in the reference. */
+size_t hx_moe_workspace_bytes_shape(int64_t T, int64_t K, int64_t N, int64_t E);
 int hx_moe_path(int64_t T, int64_t K, int64_t N, int64_t E, int64_t a_div, const void* A, const void* W, const void* C);
 
 /* hx_moe_grouped_gemm for callers that cannot allocate device memory (code under HIP graph capture, tight serving

@@ -98,7 +98,7 @@ def moe_grouped_gemm(A, W, counts, offsets, idx, static=False, end_flush=True, w
                                                 T, K, N, E, mt, _DT[dt], None)
             simlib.check(rc, "hx_moe_grouped_gemm_static")
         else:
-            wsb = lib.hx_moe_workspace_bytes(T, E)
+            wsb = lib.hx_moe_workspace_bytes_shape(T, K, N, E)
             ws = ar.empty(wsb)
             ws.fill_(0xA5)
             rc = lib.hx_moe_grouped_gemm(a.data_ptr(), w.data_ptr(), c.data_ptr(), cn.data_ptr(), of.data_ptr(), ix.data_ptr(),

@@ -212,3 +212,33 @@ def test_persistent_grouped_kernel_through_the_top_k_entry():
         assert simlib.load().hx_moe_path(6144, 256, 2048, 2, 2, None, None, None) == 6
         out = simops.moe_topk(A[::2].contiguous(), W, ex, 2)
     assert rel_err(out, orc.moe_matmul_ogs_reference(A, W, ex)) <= 1e-2
+
+
+# ---- opt-in: odd K / N % 8 != 0 through the MFMA kernels (HX_FEATURE_MOE_ANY_SHAPE) -----------------------------------------
+@pytest.mark.parametrize("T,K,N,E,dtype", [
+    (37, 101, 24, 3, torch.bfloat16),      # odd K: A and W repacked, C written in place
+    (37, 100, 19, 3, torch.bfloat16),      # N % 8 != 0: W and C padded, C cropped back
+    (300, 251, 203, 5, torch.float16),     # both
+    (600, 65, 260, 4, torch.bfloat16),     # K8 = 72: a partial last k-tile after padding
+    (20, 1, 9, 2, torch.bfloat16),         # a single k, a single padded chunk of columns
+])
+def test_any_shape_through_the_mfma_kernels(T, K, N, E, dtype):
+    import ctypes
+    from helion_amd import _lib
+    A, W, ex = inputs.moe_inputs(T, K, N, E, 1, seed=T + K + N, dtype=dtype)
+    counts, offsets, idx = _tables(ex, E)
+    counts[E - 1] = 0   # an expert switched off: its rows must come out zero after the crop as well
+    ref = orc.moe_matmul_ogs(A, W, counts, offsets, idx)
+    lib, c = simlib.load(), (ctypes.c_uint64 * 4)()
+    assert lib.hx_moe_workspace_bytes_shape(T, K, N, E) == lib.hx_moe_workspace_bytes(T, E)   # off by default
+    for variant in ("lazy-reverse", "eager-interleaved"):
+        simlib.configure(variant)
+        with simlib.features(_lib.HX_FEATURE_MOE_ANY_SHAPE):
+            assert lib.hx_moe_workspace_bytes_shape(T, K, N, E) > lib.hx_moe_workspace_bytes(T, E)
+            lib.hx_sim_counters(c)
+            before = c[0]
+            out = simops.moe_grouped_gemm(A, W, counts, offsets, idx, want_path=0, poison=4.0)
+            lib.hx_sim_counters(c)
+        assert c[0] > before, "no cross-lane instruction ran: the fp32 kernel took the call, not the repacked route"
+        assert rel_err(out, ref) <= 1e-2, variant
+        assert bool((out[ex == E - 1] == 0).all())

@@ -201,3 +201,20 @@ def test_persistent_dense_matmul(matmul_persistent, m, n, k, dtype):
     assert torch.equal(out.view(torch.int16), base.view(torch.int16))
     rows = torch.arange(0, m, 509, device=DEV)
     assert rel_err(out[rows].cpu(), orc.matmul(x[rows].cpu(), y.cpu())) <= 1e-2
+
+
+@pytest.fixture
+def moe_any_shape():
+    old = hx.set_features(hx.HX_FEATURE_MOE_ANY_SHAPE)
+    yield
+    hx.set_features(old)
+
+
+@pytest.mark.parametrize("T,K,N,E,dtype", [(37, 101, 24, 3, torch.bfloat16), (37, 100, 19, 3, torch.bfloat16), (300, 251, 203, 5, torch.float16),
+                                           (600, 65, 260, 4, torch.bfloat16), (20, 1, 9, 2, torch.bfloat16), (5000, 1001, 1003, 8, torch.bfloat16)])
+def test_moe_any_shape_through_the_mfma_kernels(moe_any_shape, T, K, N, E, dtype):
+    from helion_amd import inputs
+    A, W, ex = inputs.moe_inputs(T, K, N, E, 1, seed=T + K + N, dtype=dtype)
+    print(f"moe any-shape case T={T} K={K} N={N} E={E} {dtype}", flush=True)
+    out = hx.moe_matmul_ogs(*hx.moe_matmul_ogs_helion_kernel_args_gen(A.to(DEV), W.to(DEV), ex.to(DEV)))
+    assert rel_err(out.cpu(), orc.moe_matmul_ogs_reference(A, W, ex)) <= 1e-2
