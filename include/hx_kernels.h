@@ -162,7 +162,7 @@ int hx_fp8_attention_path(int64_t BH, int64_t S, int64_t D, int64_t v_stride_d, 
  * reference's own check, examples/moe_matmul_ogs.py:186) has A fetched in 4-byte pieces.  Anything else (odd K,
  * N % 8 != 0) runs an fp32-FMA kernel.  hx_moe_path (a_div = 1 for this entry point): 0 = the FMA kernel, 1 / 2 / 3 =
  * MFMA kernel with 32- / 128- / 256-row tiles, 4 = 128-row tiles with a partial last k-tile, 5 = the same with A in
- * 4-byte pieces. */
+ * 4-byte pieces, 6 = the 256-row tiles in persistent workgroups (opt-in, HX_FEATURE_MOE_PERSISTENT). */
 int hx_moe_grouped_gemm(const void* A, const void* W, void* C, const int32_t* counts,
                         const int32_t* offsets, const int32_t* idx, int64_t T, int64_t K, int64_t N,
                         int64_t E, int64_t max_T, int dtype, void* workspace, size_t workspace_bytes,
