@@ -126,3 +126,30 @@ def test_product_package_never_touches_the_host_execution_model():
             assert "hx_sim" not in text and "hxsim" not in text and "tests.sim" not in text and "tests/sim" not in text, f
     from helion_amd import _lib
     assert _lib.lib_path().name == "libhx_kernels.so" and _lib.lib_path().parent.name == "helion_amd"
+
+
+def test_the_inline_mfma_distance_scanner_sees_both_kinds_of_pair():
+    """helion_amd/csrc/scan_mfma_hazards.py on a hand-made listing: an accumulator read 2 instructions after the MFMA that
+    wrote it, and an MFMA 1 instruction after a vector-ALU write to one of its sources."""
+    import importlib.util
+    import pathlib
+    path = pathlib.Path(__file__).resolve().parent.parent / "helion_amd" / "csrc" / "scan_mfma_hazards.py"
+    spec = importlib.util.spec_from_file_location("scan_mfma_hazards", path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    asm = """
+_Z6kernelv:
+	v_mfma_f32_16x16x32_bf16 a[4:7], v[10:13], v[20:23], a[4:7]
+	s_nop 1
+	v_accvgpr_read_b32 v1, a5
+	ds_read_b128 v[30:33], v2
+	v_mov_b32_e32 v31, v9
+	v_mfma_f32_16x16x32_bf16 a[8:11], v[30:33], v[20:23], 0
+	v_accvgpr_read_b32 v3, a100
+.Lfunc_end0:
+"""
+    (name, n, d_read, d_src), = mod.scan(asm, "kernel", 16)
+    assert (n, d_read, d_src) == (7, 2, 1)
+    clean = asm.replace("a5", "a200").replace("v_mov_b32_e32 v31, v9", "s_nop 0")
+    (_, _, d_read, d_src), = mod.scan(clean, "kernel", 16)
+    assert d_read == 17 and d_src == 17   # nothing within the window
