@@ -66,7 +66,18 @@ def is_current() -> bool:
     return LIB.exists() and s.exists() and s.read_text() == _stamp()
 
 
-def build(verbose: bool = False) -> pathlib.Path:
+def build(verbose: bool = False, only_if_stale: bool = False) -> pathlib.Path:
+    """Builds tests/sim/libhx_sim.so.  One build at a time: processes that find the library stale together (parallel test
+    workers, two scripts started side by side) queue up on a lock file, and with only_if_stale the later ones find the work done."""
+    import fcntl
+    with open(SIM / ".build.lock", "w") as lock:
+        fcntl.flock(lock, fcntl.LOCK_EX)
+        if only_if_stale and is_current():
+            return LIB
+        return _build_locked(verbose)
+
+
+def _build_locked(verbose: bool) -> pathlib.Path:
     if BUILD.exists():
         shutil.rmtree(BUILD)
     BUILD.mkdir(parents=True)

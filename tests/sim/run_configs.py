@@ -1,7 +1,7 @@
 """The BASELINE configurations executed in the host execution model (tests/sim) against the oracle, at their real sizes
 where the model finishes in minutes: a parity record that needs no GPU.
 
-    python tests/sim/run_configs.py [--only c1,c2,c3,c4,c5] [--c4-heads 2] [--c5-columns 512]
+    python tests/sim/run_configs.py [--only c1,c2,c3,c4,c5,d64,d128,d256] [--c4-heads 2] [--c5-columns 512] [--features MASK]
 
   C1  fp8_gemm 1024^3 (the reference's own CPU case)                         whole output, bit for bit
   C2  fp8_gemm 8192^3, per-tensor scales, bf16 out (the headline kernel)     whole output (about ten minutes)
@@ -13,6 +13,11 @@ where the model finishes in minutes: a parity record that needs no GPU.
                                                                              tables, the first `--c5-columns` of the 14336
                                                                              output columns (the kernel treats column tiles
                                                                              independently)
+
+  D64 / D128 / D256  decode fp8_gemm M64 / M128 / M256 N28672 K8192           whole output
+
+--features MASK switches opt-in kernel paths on (helion_amd.HX_FEATURE_*): C2 then runs on the persistent 256x256 kernel
+(mask 8), C5 on the persistent grouped kernel (64), the decode rows on the kernel with separate A / B rings (16).
 
 Every operand sits in a guarded buffer and the LDS access check is on, as in the tests.  Prints one line per
 configuration; exit status 1 if any is out of tolerance.  Not part of the default test run (tests/test_sim_configs.py
@@ -52,8 +57,16 @@ def _gemm(a, b, sa, sb, path):
     return e <= 1e-2, f"max|err|/max|ref| {e:.2e} (tolerance 2e-2); {diff} of {out.numel()} bf16 results differ by a rounding step"
 
 
+FEATURES = 0
+
+
 def c2():
-    return _gemm(*inputs.gemm_c2(), path=1)
+    return _gemm(*inputs.gemm_c2(), path=7 if FEATURES & 8 else 1)
+
+
+def decode(rows):
+    a, b, sa, sb = inputs.gemm_scaled(rows, 28672, 8192, rows)
+    return _gemm(a, b, sa, sb, path=8 if FEATURES & 16 else 5)
 
 
 def c3():
@@ -82,7 +95,7 @@ def c5(columns):
     counts = torch.bincount(ex, minlength=E).to(torch.int32)
     offsets = torch.zeros(E + 1, dtype=torch.int32)
     offsets[1:] = torch.cumsum(counts, 0)
-    out = simops.moe_grouped_gemm(A, W, counts, offsets, idx, want_path=3, poison=9.0)
+    out = simops.moe_grouped_gemm(A, W, counts, offsets, idx, want_path=6 if FEATURES & 64 else 3, poison=9.0)
     ref = orc.moe_matmul_ogs_reference(A, W, ex)
     e = rel_err(out, ref)
     return e <= 1e-2, f"rows per expert {counts.tolist()}, columns 0..{columns - 1}: max|err|/max|ref| {e:.2e} (tolerance 2e-2)"
@@ -94,9 +107,14 @@ def main():
     ap.add_argument("--c4-heads", type=int, default=2)
     ap.add_argument("--c5-columns", type=int, default=512)
     ap.add_argument("--variant", default="lazy", choices=list(simlib.VARIANTS))
+    ap.add_argument("--features", type=int, default=0)
     args = ap.parse_args()
     simlib.configure(args.variant)
-    runs = {"c1": c1, "c2": c2, "c3": c3, "c4": lambda: c4(args.c4_heads), "c5": lambda: c5(args.c5_columns)}
+    global FEATURES
+    FEATURES = args.features
+    simlib.load().hx_set_features(FEATURES)
+    runs = {"c1": c1, "c2": c2, "c3": c3, "c4": lambda: c4(args.c4_heads), "c5": lambda: c5(args.c5_columns),
+            "d64": lambda: decode(64), "d128": lambda: decode(128), "d256": lambda: decode(256)}
     bad = 0
     for name in args.only.split(","):
         t0 = time.time()
@@ -104,7 +122,7 @@ def main():
         ok, note = runs[name]()
         w = simlib.work()
         print(f"{name.upper()} {'ok ' if ok else 'BAD'} {note}  [{w['workgroups']} workgroups, {w['mfma']} wave-level MFMAs, "
-              f"{w['dma_bytes'] / 2**20:.0f} MiB by DMA, {time.time() - t0:.0f} s, variant {args.variant}]", flush=True)
+              f"{w['dma_bytes'] / 2**20:.0f} MiB by DMA, {time.time() - t0:.0f} s, variant {args.variant}, features {FEATURES}]", flush=True)
         bad += not ok
     sys.exit(1 if bad else 0)
 

@@ -23,7 +23,7 @@ def load():
     global _lib
     if _lib is None:
         if not _build.is_current():
-            _build.build()
+            _build.build(only_if_stale=True)
         lib = ctypes.CDLL(str(_build.LIB))
         for name, (res, args) in _real._SIGNATURES.items():
             fn = getattr(lib, name)
