@@ -3,6 +3,10 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--only c2,lib,c3,c4,c5,next,sib[,lib16][,optin]] [--no-cpu-baseline] [--clock-probe]
 
+`--only ...,optin` adds, per opt-in kernel path (helion_amd.set_features), a row that first compares the path's output with
+the default kernel's on the same operands and then times both; `HX_FEATURES=<mask> python bench.py` runs the whole
+benchmark with paths switched on and says so in `config.opt_in_features` (the "kernel" labels name the default kernels).
+
 A "step" is one launch of the FP8 GEMM at the headline configuration (M=N=K=8192, e4m3 operands, B column-major,
 per-tensor fp32 scales, bf16 output) with inputs resident in HBM.
 
